@@ -1,0 +1,142 @@
+/*
+ * C ABI of the MI355X (gfx950) TTT-MLP forward / remat-backward kernels.
+ *
+ * This is the drop-in boundary below the Python operator module
+ * `test_time_training`: plain pointers and sizes, no torch types.  Every
+ * pointer is a DEVICE pointer to a contiguous row-major tensor owned by the
+ * caller; the library allocates nothing, keeps no state between calls and
+ * never synchronises the stream (the launch is asynchronous on `stream`).
+ *
+ * Fixed sizes of the shipped kernels: mini-batch CS = 64 tokens, head dim
+ * F = 64, hidden dim H = 256.  B = batch, NH = heads, NC = mini-batches,
+ * K = ceil(NC / checkpoint_group_size) checkpoints.
+ *
+ * Reference interfaces replaced (upstream repository paths):
+ *   ttt_mlp_fwd_launch  <- host launcher `ttt_forward`   kernels/ttt/ttt.cu:594-721
+ *                          + kernel fwd_ttt_mlp_ker<64>   kernels/ttt/ttt.cu:85-586
+ *   ttt_mlp_bwd_launch  <- host launcher `ttt_backward`  kernels/ttt_backward/ttt.cu:1451-1917
+ *                          + kernel bwd_ttt_mlp_ker<64>   kernels/ttt_backward/ttt.cu:179-1443
+ * The argument structs list the tensors in the exact order of the operator's
+ * positional arguments (test_time_training.cpp:25-42 and :47-91).
+ */
+#ifndef TTT_MLP_H_
+#define TTT_MLP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TTT_MLP_ABI_VERSION 1
+
+#define TTT_MLP_CS 64   /* tokens per mini-batch        */
+#define TTT_MLP_F 64    /* head dimension               */
+#define TTT_MLP_HID 256 /* inner MLP hidden dimension   */
+
+/* Return codes (0 = success; positive values below 1000 are hipError_t codes). */
+#define TTT_MLP_OK 0
+#define TTT_MLP_ERR_BAD_ARG 1001   /* null pointer or non-positive size           */
+#define TTT_MLP_ERR_BAD_CKPT 1002  /* K != ceil(NC / checkpoint_group_size)       */
+#define TTT_MLP_ERR_ALIGN 1003     /* a pointer is not 16-byte aligned            */
+#define TTT_MLP_ERR_TOO_LARGE 1004 /* B*NH exceeds the grid limit                 */
+
+/* Forward scan.  Replaces the 16 positional arguments of `ttt_forward`
+ * (test_time_training.cpp:25-42).  bf16 tensors are passed as uint16_t bit patterns. */
+typedef struct ttt_mlp_fwd_args {
+  const uint16_t* XQ;              /* [B,NH,NC,CS,F]  bf16 in  */
+  const uint16_t* XK;              /* [B,NH,NC,CS,F]  bf16 in  */
+  const uint16_t* XV;              /* [B,NH,NC,CS,F]  bf16 in  */
+  const uint16_t* last_eta;        /* [B,NH,NC,CS,1]  bf16 in  */
+  const float* ttt_norm_weight;    /* [1,NH,1,F]      fp32 in  */
+  const float* ttt_norm_bias;      /* [1,NH,1,F]      fp32 in  */
+  const float* W1;                 /* [B,NH,F,HID]    fp32 in (initial state, not modified) */
+  const float* b1;                 /* [B,NH,1,HID]    fp32 in  */
+  const float* W2;                 /* [B,NH,HID,F]    fp32 in  */
+  const float* b2;                 /* [B,NH,1,F]      fp32 in  */
+  float* W1_checkpoints;           /* [B,NH,K,F,HID]  fp32 out */
+  float* b1_checkpoints;           /* [B,NH,K,1,HID]  fp32 out */
+  float* W2_checkpoints;           /* [B,NH,K,HID,F]  fp32 out */
+  float* b2_checkpoints;           /* [B,NH,K,1,F]    fp32 out */
+  uint16_t* Out;                   /* [B,NH,NC,CS,F]  bf16 out */
+  int32_t checkpoint_group_size;
+  int32_t B, NH, NC, K;
+} ttt_mlp_fwd_args;
+
+/* Remat backward.  Replaces the 43 positional arguments of `ttt_backward`
+ * (test_time_training.cpp:47-91).  The sixteen *_group tensors are caller-owned
+ * scratch of checkpoint_group_size mini-batches; the library uses them as
+ * workspace and leaves their contents unspecified.  grad_L_last_eta / grad_L_XQ /
+ * grad_L_XK / grad_L_XV are accumulated into (the caller zero-fills them), all
+ * other outputs are overwritten.  `Out` is not touched. */
+typedef struct ttt_mlp_bwd_args {
+  const uint16_t* XQ;
+  const uint16_t* XK;
+  const uint16_t* XV;
+  const uint16_t* last_eta;
+  const float* ttt_norm_weight;
+  const float* ttt_norm_bias;
+  const float* W1_checkpoints;     /* [B,NH,K,F,HID]  fp32 in */
+  const float* b1_checkpoints;
+  const float* W2_checkpoints;
+  const float* b2_checkpoints;
+  uint16_t* Out;                   /* unused */
+  float* W1_init_group;            /* [B,NH,cgs,F,HID]  fp32 scratch */
+  float* b1_init_group;            /* [B,NH,cgs,1,HID]  fp32 scratch */
+  float* W2_init_group;            /* [B,NH,cgs,HID,F]  fp32 scratch */
+  float* b2_init_group;            /* [B,NH,cgs,1,F]    fp32 scratch */
+  uint16_t* x_hat_ln_group;        /* [B,NH,cgs,CS,F]   bf16 scratch */
+  float* std_ln_group;             /* [B,NH,cgs,CS,1]   fp32 scratch */
+  uint16_t* X2_group;              /* [B,NH,cgs,CS,HID] bf16 scratch */
+  uint16_t* Z1_group;
+  uint16_t* Z1_bar_group;
+  uint16_t* X2_bar_group;
+  uint16_t* grad_l_wrt_Z2_group;   /* [B,NH,cgs,CS,F]   bf16 scratch */
+  uint16_t* grad_l_wrt_Z1_group;   /* [B,NH,cgs,CS,HID] bf16 scratch */
+  uint16_t* x_hat_fused_group;     /* [B,NH,cgs,CS,F]   bf16 scratch */
+  uint16_t* grad_x_hat_fused_group;
+  uint16_t* grad_output_fused_group;
+  float* std_fused_group;          /* [B,NH,cgs,CS,1]   fp32 scratch */
+  const float* grad_L_W1_last;     /* [B,NH,F,HID] fp32 in: grads wrt the state after the last mini-batch */
+  const float* grad_L_b1_last;
+  const float* grad_L_W2_last;
+  const float* grad_L_b2_last;
+  const uint16_t* grad_L_XQW_mini_batch; /* [B,NH,NC,CS,F] bf16 in */
+  float* grad_L_ttt_norm_weight;   /* [B,NH,1,F] fp32 out (per batch element) */
+  float* grad_L_ttt_norm_bias;
+  float* grad_L_W1_init;           /* as W1 ... fp32 out */
+  float* grad_L_b1_init;
+  float* grad_L_W2_init;
+  float* grad_L_b2_init;
+  uint16_t* grad_L_last_eta;       /* [B,NH,NC,CS,1] bf16, accumulated into */
+  uint16_t* grad_L_XQ;             /* [B,NH,NC,CS,F] bf16, accumulated into */
+  uint16_t* grad_L_XK;
+  uint16_t* grad_L_XV;
+  int32_t checkpoint_group_size;
+  int32_t B, NH, NC, K;
+} ttt_mlp_bwd_args;
+
+/* Version of this header the library was built against. */
+int ttt_mlp_abi_version(void);
+
+/* Validates sizes / alignment and enqueues the forward kernel on `stream`
+ * (a hipStream_t, NULL = the default stream).  Returns TTT_MLP_OK, one of the
+ * TTT_MLP_ERR_* codes, or the hipError_t of a failed launch. */
+int ttt_mlp_fwd_launch(const ttt_mlp_fwd_args* args, void* stream);
+
+/* Same for the remat backward. */
+int ttt_mlp_bwd_launch(const ttt_mlp_bwd_args* args, void* stream);
+
+/* Human-readable text for a return code of the two launchers. */
+const char* ttt_mlp_error_string(int code);
+
+/* Static facts about the compiled kernels, for harnesses: LDS bytes per
+ * workgroup and threads per workgroup of the forward (which = 0) or backward
+ * (which = 1) kernel.  Returns 0 on success. */
+int ttt_mlp_kernel_info(int which, int* lds_bytes, int* threads_per_workgroup);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TTT_MLP_H_ */

@@ -1,0 +1,200 @@
+// Python operator module `test_time_training` for ROCm: the same two functions, positional
+// argument lists, tensor layouts and return value as the upstream binding
+// (test_time_training.cpp:25-42, :47-91, :95-105), implemented on top of the C ABI in
+// include/ttt_mlp.h.  Shape / dtype / device / contiguity problems raise (TORCH_CHECK ->
+// RuntimeError) like upstream (kernels/ttt/ttt.cu:621-630, kernels/ttt_backward/ttt.cu:1507-1760);
+// unlike upstream, launch and execution errors raise as well instead of being printed.
+#include <torch/extension.h>
+#include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
+
+#include "../../include/ttt_mlp.h"
+
+namespace {
+
+constexpr int64_t F = TTT_MLP_F, CS = TTT_MLP_CS, HID = TTT_MLP_HID;
+bool g_synchronize = true;  // upstream blocks the host until the kernel has finished
+
+void check_tensor(const torch::Tensor& t, const char* name, c10::ScalarType dtype, std::initializer_list<int64_t> shape) {
+  TORCH_CHECK(t.device().is_cuda(), "Invalid dims for ", name, ": not a GPU tensor");
+  TORCH_CHECK(t.is_contiguous(), "Invalid dims for ", name, ": not contiguous");
+  TORCH_CHECK(t.scalar_type() == dtype, "Invalid dtype for ", name, ": expected ", c10::toString(dtype), ", got ",
+              c10::toString(t.scalar_type()));
+  TORCH_CHECK(t.dim() == (int64_t)shape.size(), "Invalid dims for ", name, ": expected ", shape.size(), " dims, got ", t.dim());
+  int64_t d = 0;
+  for (int64_t s : shape) {
+    TORCH_CHECK(s < 0 || t.size(d) == s, "Invalid dims for ", name, ": size(", d, ") is ", t.size(d), ", expected ", s);
+    ++d;
+  }
+}
+
+// last_eta is [B,NH,NC,CS,1]; the upstream forward also accepts [B,NH,NC,CS] (same bytes).
+void check_eta(const torch::Tensor& t, const char* name, int64_t B, int64_t NH, int64_t NC, bool allow_4d) {
+  if (allow_4d && t.dim() == 4) check_tensor(t, name, torch::kBFloat16, {B, NH, NC, CS});
+  else check_tensor(t, name, torch::kBFloat16, {B, NH, NC, CS, 1});
+}
+
+const uint16_t* bfp(const torch::Tensor& t) { return reinterpret_cast<const uint16_t*>(t.data_ptr<at::BFloat16>()); }
+uint16_t* bfp_mut(const torch::Tensor& t) { return reinterpret_cast<uint16_t*>(t.data_ptr<at::BFloat16>()); }
+
+void finish(int rc, hipStream_t stream, const char* what) {
+  TORCH_CHECK(rc == TTT_MLP_OK, what, " launch failed: ", ttt_mlp_error_string(rc));
+  if (g_synchronize) {
+    hipError_t e = hipStreamSynchronize(stream);
+    TORCH_CHECK(e == hipSuccess, what, " execution failed: ", hipGetErrorString(e));
+  }
+}
+
+}  // namespace
+
+torch::Tensor ttt_forward(const torch::Tensor XQ, const torch::Tensor XK, const torch::Tensor XV,
+                          const torch::Tensor last_eta, const torch::Tensor ttt_norm_weight,
+                          const torch::Tensor ttt_norm_bias, const torch::Tensor W1, const torch::Tensor b1,
+                          const torch::Tensor W2, const torch::Tensor b2, const torch::Tensor W1_checkpoints,
+                          const torch::Tensor b1_checkpoints, const torch::Tensor W2_checkpoints,
+                          const torch::Tensor b2_checkpoints, const torch::Tensor Out, const int checkpoint_group_size) {
+  TORCH_CHECK(XQ.dim() == 5, "Invalid dims for XQ");
+  const int64_t B = XQ.size(0), NH = XQ.size(1), NC = XQ.size(2);
+  TORCH_CHECK(W1_checkpoints.dim() == 5, "Invalid dims for W1_checkpoints");
+  const int64_t K = W1_checkpoints.size(2);
+  TORCH_CHECK(checkpoint_group_size > 0, "checkpoint_group_size must be positive");
+  TORCH_CHECK(K == (NC + checkpoint_group_size - 1) / checkpoint_group_size,
+              "Invalid dims for W1_checkpoints: ", K, " checkpoints for ", NC, " mini-batches in groups of ", checkpoint_group_size);
+  check_tensor(XQ, "XQ", torch::kBFloat16, {B, NH, NC, CS, F});
+  check_tensor(XK, "XK", torch::kBFloat16, {B, NH, NC, CS, F});
+  check_tensor(XV, "XV", torch::kBFloat16, {B, NH, NC, CS, F});
+  check_eta(last_eta, "last_eta", B, NH, NC, true);
+  check_tensor(ttt_norm_weight, "ttt_norm_weight", torch::kFloat32, {1, NH, 1, F});
+  check_tensor(ttt_norm_bias, "ttt_norm_bias", torch::kFloat32, {1, NH, 1, F});
+  check_tensor(W1, "W1", torch::kFloat32, {B, NH, F, HID});
+  check_tensor(b1, "b1", torch::kFloat32, {B, NH, 1, HID});
+  check_tensor(W2, "W2", torch::kFloat32, {B, NH, HID, F});
+  check_tensor(b2, "b2", torch::kFloat32, {B, NH, 1, F});
+  check_tensor(W1_checkpoints, "W1_checkpoints", torch::kFloat32, {B, NH, K, F, HID});
+  check_tensor(b1_checkpoints, "b1_checkpoints", torch::kFloat32, {B, NH, K, 1, HID});
+  check_tensor(W2_checkpoints, "W2_checkpoints", torch::kFloat32, {B, NH, K, HID, F});
+  check_tensor(b2_checkpoints, "b2_checkpoints", torch::kFloat32, {B, NH, K, 1, F});
+  check_tensor(Out, "Out", torch::kBFloat16, {B, NH, NC, CS, F});
+
+  ttt_mlp_fwd_args a;
+  a.XQ = bfp(XQ); a.XK = bfp(XK); a.XV = bfp(XV); a.last_eta = bfp(last_eta);
+  a.ttt_norm_weight = ttt_norm_weight.data_ptr<float>(); a.ttt_norm_bias = ttt_norm_bias.data_ptr<float>();
+  a.W1 = W1.data_ptr<float>(); a.b1 = b1.data_ptr<float>(); a.W2 = W2.data_ptr<float>(); a.b2 = b2.data_ptr<float>();
+  a.W1_checkpoints = W1_checkpoints.data_ptr<float>(); a.b1_checkpoints = b1_checkpoints.data_ptr<float>();
+  a.W2_checkpoints = W2_checkpoints.data_ptr<float>(); a.b2_checkpoints = b2_checkpoints.data_ptr<float>();
+  a.Out = bfp_mut(Out);
+  a.checkpoint_group_size = checkpoint_group_size;
+  a.B = (int32_t)B; a.NH = (int32_t)NH; a.NC = (int32_t)NC; a.K = (int32_t)K;
+  hipStream_t stream = c10::hip::getCurrentHIPStream(XQ.device().index()).stream();
+  finish(ttt_mlp_fwd_launch(&a, stream), stream, "ttt_forward");
+  return Out;
+}
+
+torch::Tensor ttt_backward(
+    const torch::Tensor XQ, const torch::Tensor XK, const torch::Tensor XV, const torch::Tensor last_eta,
+    const torch::Tensor ttt_norm_weight, const torch::Tensor ttt_norm_bias, const torch::Tensor W1_checkpoints,
+    const torch::Tensor b1_checkpoints, const torch::Tensor W2_checkpoints, const torch::Tensor b2_checkpoints,
+    const torch::Tensor Out, const torch::Tensor W1_init_group, const torch::Tensor b1_init_group,
+    const torch::Tensor W2_init_group, const torch::Tensor b2_init_group, const torch::Tensor x_hat_ln_group,
+    const torch::Tensor std_ln_group, const torch::Tensor X2_group, const torch::Tensor Z1_group,
+    const torch::Tensor Z1_bar_group, const torch::Tensor X2_bar_group, const torch::Tensor grad_l_wrt_Z2_group,
+    const torch::Tensor grad_l_wrt_Z1_group, const torch::Tensor x_hat_fused_group,
+    const torch::Tensor grad_x_hat_fused_group, const torch::Tensor grad_output_fused_group,
+    const torch::Tensor std_fused_group, const torch::Tensor grad_L_W1_last, const torch::Tensor grad_L_b1_last,
+    const torch::Tensor grad_L_W2_last, const torch::Tensor grad_L_b2_last, const torch::Tensor grad_L_XQW_mini_batch,
+    const torch::Tensor grad_L_ttt_norm_weight, const torch::Tensor grad_L_ttt_norm_bias,
+    const torch::Tensor grad_L_W1_init, const torch::Tensor grad_L_b1_init, const torch::Tensor grad_L_W2_init,
+    const torch::Tensor grad_L_b2_init, const torch::Tensor grad_L_last_eta, const torch::Tensor grad_L_XQ,
+    const torch::Tensor grad_L_XK, const torch::Tensor grad_L_XV, const int checkpoint_group_size) {
+  TORCH_CHECK(XQ.dim() == 5, "Invalid dims for XQ");
+  const int64_t B = XQ.size(0), NH = XQ.size(1), NC = XQ.size(2);
+  TORCH_CHECK(W1_checkpoints.dim() == 5, "Invalid dims for W1_checkpoints");
+  const int64_t K = W1_checkpoints.size(2);
+  const int64_t G = checkpoint_group_size;
+  TORCH_CHECK(G > 0, "checkpoint_group_size must be positive");
+  TORCH_CHECK(K == (NC + G - 1) / G, "Invalid dims for W1_checkpoints: ", K, " checkpoints for ", NC,
+              " mini-batches in groups of ", G);
+  const auto bf = torch::kBFloat16;
+  const auto f32 = torch::kFloat32;
+  check_tensor(XQ, "XQ", bf, {B, NH, NC, CS, F});
+  check_tensor(XK, "XK", bf, {B, NH, NC, CS, F});
+  check_tensor(XV, "XV", bf, {B, NH, NC, CS, F});
+  check_eta(last_eta, "last_eta", B, NH, NC, false);
+  check_tensor(ttt_norm_weight, "ttt_norm_weight", f32, {1, NH, 1, F});
+  check_tensor(ttt_norm_bias, "ttt_norm_bias", f32, {1, NH, 1, F});
+  check_tensor(W1_checkpoints, "W1_checkpoints", f32, {B, NH, K, F, HID});
+  check_tensor(b1_checkpoints, "b1_checkpoints", f32, {B, NH, K, 1, HID});
+  check_tensor(W2_checkpoints, "W2_checkpoints", f32, {B, NH, K, HID, F});
+  check_tensor(b2_checkpoints, "b2_checkpoints", f32, {B, NH, K, 1, F});
+  check_tensor(Out, "Out", bf, {B, NH, NC, CS, F});
+  check_tensor(W1_init_group, "W1_init_group", f32, {B, NH, G, F, HID});
+  check_tensor(b1_init_group, "b1_init_group", f32, {B, NH, G, 1, HID});
+  check_tensor(W2_init_group, "W2_init_group", f32, {B, NH, G, HID, F});
+  check_tensor(b2_init_group, "b2_init_group", f32, {B, NH, G, 1, F});
+  check_tensor(x_hat_ln_group, "x_hat_ln_group", bf, {B, NH, G, CS, F});
+  check_tensor(std_ln_group, "std_ln_group", f32, {B, NH, G, CS, 1});
+  check_tensor(X2_group, "X2_group", bf, {B, NH, G, CS, HID});
+  check_tensor(Z1_group, "Z1_group", bf, {B, NH, G, CS, HID});
+  check_tensor(Z1_bar_group, "Z1_bar_group", bf, {B, NH, G, CS, HID});
+  check_tensor(X2_bar_group, "X2_bar_group", bf, {B, NH, G, CS, HID});
+  check_tensor(grad_l_wrt_Z2_group, "grad_l_wrt_Z2_group", bf, {B, NH, G, CS, F});
+  check_tensor(grad_l_wrt_Z1_group, "grad_l_wrt_Z1_group", bf, {B, NH, G, CS, HID});
+  check_tensor(x_hat_fused_group, "x_hat_fused_group", bf, {B, NH, G, CS, F});
+  check_tensor(grad_x_hat_fused_group, "grad_x_hat_fused_group", bf, {B, NH, G, CS, F});
+  check_tensor(grad_output_fused_group, "grad_output_fused_group", bf, {B, NH, G, CS, F});
+  check_tensor(std_fused_group, "std_fused_group", f32, {B, NH, G, CS, 1});
+  check_tensor(grad_L_W1_last, "grad_L_W1_last", f32, {B, NH, F, HID});
+  check_tensor(grad_L_b1_last, "grad_L_b1_last", f32, {B, NH, 1, HID});
+  check_tensor(grad_L_W2_last, "grad_L_W2_last", f32, {B, NH, HID, F});
+  check_tensor(grad_L_b2_last, "grad_L_b2_last", f32, {B, NH, 1, F});
+  check_tensor(grad_L_XQW_mini_batch, "grad_L_XQW_mini_batch", bf, {B, NH, NC, CS, F});
+  check_tensor(grad_L_ttt_norm_weight, "grad_L_ttt_norm_weight", f32, {B, NH, 1, F});
+  check_tensor(grad_L_ttt_norm_bias, "grad_L_ttt_norm_bias", f32, {B, NH, 1, F});
+  check_tensor(grad_L_W1_init, "grad_L_W1_init", f32, {B, NH, F, HID});
+  check_tensor(grad_L_b1_init, "grad_L_b1_init", f32, {B, NH, 1, HID});
+  check_tensor(grad_L_W2_init, "grad_L_W2_init", f32, {B, NH, HID, F});
+  check_tensor(grad_L_b2_init, "grad_L_b2_init", f32, {B, NH, 1, F});
+  check_tensor(grad_L_last_eta, "grad_L_last_eta", bf, {B, NH, NC, CS, 1});
+  check_tensor(grad_L_XQ, "grad_L_XQ", bf, {B, NH, NC, CS, F});
+  check_tensor(grad_L_XK, "grad_L_XK", bf, {B, NH, NC, CS, F});
+  check_tensor(grad_L_XV, "grad_L_XV", bf, {B, NH, NC, CS, F});
+
+  ttt_mlp_bwd_args a;
+  a.XQ = bfp(XQ); a.XK = bfp(XK); a.XV = bfp(XV); a.last_eta = bfp(last_eta);
+  a.ttt_norm_weight = ttt_norm_weight.data_ptr<float>(); a.ttt_norm_bias = ttt_norm_bias.data_ptr<float>();
+  a.W1_checkpoints = W1_checkpoints.data_ptr<float>(); a.b1_checkpoints = b1_checkpoints.data_ptr<float>();
+  a.W2_checkpoints = W2_checkpoints.data_ptr<float>(); a.b2_checkpoints = b2_checkpoints.data_ptr<float>();
+  a.Out = bfp_mut(Out);
+  a.W1_init_group = W1_init_group.data_ptr<float>(); a.b1_init_group = b1_init_group.data_ptr<float>();
+  a.W2_init_group = W2_init_group.data_ptr<float>(); a.b2_init_group = b2_init_group.data_ptr<float>();
+  a.x_hat_ln_group = bfp_mut(x_hat_ln_group); a.std_ln_group = std_ln_group.data_ptr<float>();
+  a.X2_group = bfp_mut(X2_group); a.Z1_group = bfp_mut(Z1_group);
+  a.Z1_bar_group = bfp_mut(Z1_bar_group); a.X2_bar_group = bfp_mut(X2_bar_group);
+  a.grad_l_wrt_Z2_group = bfp_mut(grad_l_wrt_Z2_group); a.grad_l_wrt_Z1_group = bfp_mut(grad_l_wrt_Z1_group);
+  a.x_hat_fused_group = bfp_mut(x_hat_fused_group); a.grad_x_hat_fused_group = bfp_mut(grad_x_hat_fused_group);
+  a.grad_output_fused_group = bfp_mut(grad_output_fused_group); a.std_fused_group = std_fused_group.data_ptr<float>();
+  a.grad_L_W1_last = grad_L_W1_last.data_ptr<float>(); a.grad_L_b1_last = grad_L_b1_last.data_ptr<float>();
+  a.grad_L_W2_last = grad_L_W2_last.data_ptr<float>(); a.grad_L_b2_last = grad_L_b2_last.data_ptr<float>();
+  a.grad_L_XQW_mini_batch = bfp(grad_L_XQW_mini_batch);
+  a.grad_L_ttt_norm_weight = grad_L_ttt_norm_weight.data_ptr<float>();
+  a.grad_L_ttt_norm_bias = grad_L_ttt_norm_bias.data_ptr<float>();
+  a.grad_L_W1_init = grad_L_W1_init.data_ptr<float>(); a.grad_L_b1_init = grad_L_b1_init.data_ptr<float>();
+  a.grad_L_W2_init = grad_L_W2_init.data_ptr<float>(); a.grad_L_b2_init = grad_L_b2_init.data_ptr<float>();
+  a.grad_L_last_eta = bfp_mut(grad_L_last_eta);
+  a.grad_L_XQ = bfp_mut(grad_L_XQ); a.grad_L_XK = bfp_mut(grad_L_XK); a.grad_L_XV = bfp_mut(grad_L_XV);
+  a.checkpoint_group_size = checkpoint_group_size;
+  a.B = (int32_t)B; a.NH = (int32_t)NH; a.NC = (int32_t)NC; a.K = (int32_t)K;
+  hipStream_t stream = c10::hip::getCurrentHIPStream(XQ.device().index()).stream();
+  finish(ttt_mlp_bwd_launch(&a, stream), stream, "ttt_backward");
+  return Out;
+}
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.doc() = "Test Time Training Kernels";
+  m.def("ttt_forward", &ttt_forward, "TTT Forward.");
+  m.def("ttt_backward", &ttt_backward, "TTT Backward.");
+  // Not part of the upstream module: lets a harness time launches with events instead of paying
+  // the host synchronisation the upstream operator performs on every call.
+  m.def("set_synchronize", [](bool on) { g_synchronize = on; }, "Block the host after each launch (default true).");
+  m.def("abi_version", []() { return ttt_mlp_abi_version(); });
+}

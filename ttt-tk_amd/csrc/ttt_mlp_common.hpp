@@ -1,0 +1,202 @@
+// Shared device-side building blocks of the gfx950 TTT-MLP kernels.
+//
+// One workgroup of 4 wavefronts (256 threads) owns one (batch, head) recurrence.  Wave w owns
+// hidden columns [64w, 64w+64) of the inner MLP, so every per-wave contraction is a
+// 64x64x64 bf16 MFMA product with fp32 accumulate, built from 32x32x16 tiles.
+//
+// Register tile conventions (lane = 32*h + c, h in {0,1}, c in 0..31), verified on hardware:
+//   accumulator block (32x32 fp32, 16 regs): reg i holds row 8*(i/4) + 4*h + (i%4), column c
+//   operand block     (32x16 bf16,  8 slots): lane holds free index c, contraction index 8*h + slot
+// A 64x64 accumulator tile whose ROWS are the contraction index of the next product can be fed
+// to that product straight from registers ("chained"): packing regs 8t..8t+7 of a block gives the
+// operand of k-step (2*rowblock + t) with the contraction index permuted to
+//   kappa(s, h, slot) = 16*s + 8*(slot/4) + 4*h + (slot%4).
+// Every operand that meets a chained operand is therefore loaded in the same kappa order.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ttt {
+
+typedef __bf16 bf16;
+typedef bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int CS = 64;         // tokens per mini-batch
+constexpr int FD = 64;         // head dimension
+constexpr int HID = 256;       // hidden dimension of the inner MLP
+constexpr int NWAVE = 4;       // wavefronts per workgroup = hidden shards
+constexpr int NTHREADS = 256;
+constexpr int LDB = 72;        // row stride (elements) of a 64x64 bf16 tile in LDS: 144 B
+constexpr int LDP = 68;        // row stride (floats) of a 64x64 fp32 partial tile in LDS: 272 B
+constexpr float LN_EPS = 1e-8f;
+
+#define TTT_DEV __device__ __forceinline__
+
+struct Acc { f32x16 b[2][2]; };   // 64x64 fp32 tile: b[row block][column block]
+struct Opd { bf16x8 v[2][4]; };   // 64x64 bf16 operand: v[free-index block][k step]
+
+TTT_DEV void acc_zero(Acc& a) {
+#pragma unroll
+  for (int r = 0; r < 2; r++)
+#pragma unroll
+    for (int c = 0; c < 2; c++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) a.b[r][c][i] = 0.f;
+}
+
+// d[row block of a][column block of b] += a * b over the 64-long contraction.
+TTT_DEV void mma(Acc& d, const Opd& a, const Opd& b) {
+#pragma unroll
+  for (int s = 0; s < 4; s++)
+#pragma unroll
+    for (int r = 0; r < 2; r++)
+#pragma unroll
+      for (int c = 0; c < 2; c++)
+        d.b[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v[r][s], b.v[c][s], d.b[r][c], 0, 0, 0);
+}
+
+TTT_DEV bf16x8 pack8(const f32x16& x, int t) {
+  bf16x8 o;
+#pragma unroll
+  for (int j = 0; j < 8; j++) o[j] = (bf16)x[8 * t + j];
+  return o;
+}
+
+// Accumulator tile (rows = contraction index, columns = free index) -> chained operand.
+TTT_DEV Opd cvt_chain(const Acc& x) {
+  Opd o;
+#pragma unroll
+  for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+      for (int t = 0; t < 2; t++) o.v[cb][2 * rb + t] = pack8(x.b[rb][cb], t);
+  return o;
+}
+
+TTT_DEV bf16x8 cat(bf16x4 lo, bf16x4 hi) { return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7); }
+
+// Operand from an LDS tile stored [free index][contraction index] (contraction contiguous),
+// row stride LDB, in kappa order: two 8-byte reads per k-step.
+TTT_DEV Opd lds_rows_kappa(const bf16* base, int c, int h) {
+  Opd o;
+#pragma unroll
+  for (int fb = 0; fb < 2; fb++)
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      const bf16* p = base + (32 * fb + c) * LDB + 16 * s + 4 * h;
+      o.v[fb][s] = cat(*reinterpret_cast<const bf16x4*>(p), *reinterpret_cast<const bf16x4*>(p + 8));
+    }
+  return o;
+}
+
+TTT_DEV bf16x4 lds_tr4(const bf16* p) {
+  typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
+  s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
+  return __builtin_bit_cast(bf16x4, t);
+}
+
+// Operand from an LDS tile stored [contraction index][free index] (free index contiguous), row
+// stride LDB, in kappa order, using the transposing LDS read: within each group of 16 lanes, lane
+// i points at row k0 + i/4, columns m0 + 4*(i%4) .. +3, and receives rows k0..k0+3 of column m0 + i.
+TTT_DEV Opd lds_tr_kappa(const bf16* base, int lane) {
+  Opd o;
+  const int h = lane >> 5, c = lane & 31, i = lane & 15;
+#pragma unroll
+  for (int fb = 0; fb < 2; fb++)
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      const bf16* p = base + (16 * s + 4 * h + (i >> 2)) * LDB + 32 * fb + 16 * (c >> 4) + 4 * (i & 3);
+      o.v[fb][s] = cat(lds_tr4(p), lds_tr4(p + 8 * LDB));
+    }
+  return o;
+}
+
+// Writes a chained operand (lane = free index, slots = contraction index in kappa order) as an LDS
+// tile stored [free index][contraction index]; the inverse of lds_rows_kappa.
+TTT_DEV void lds_store_rows_kappa(bf16* base, const Opd& o, int c, int h) {
+#pragma unroll
+  for (int fb = 0; fb < 2; fb++)
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      bf16* p = base + (32 * fb + c) * LDB + 16 * s + 4 * h;
+      *reinterpret_cast<bf16x4*>(p) = __builtin_shufflevector(o.v[fb][s], o.v[fb][s], 0, 1, 2, 3);
+      *reinterpret_cast<bf16x4*>(p + 8) = __builtin_shufflevector(o.v[fb][s], o.v[fb][s], 4, 5, 6, 7);
+    }
+}
+
+// Writes an accumulator tile (lane = column, regs = rows) to an fp32 LDS tile stored
+// [column][row] with row stride LDP: 16-byte writes of 4 consecutive rows.
+TTT_DEV void lds_store_partial(float* base, const Acc& a, int c, int h) {
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+    for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        f32x4 v = {a.b[rb][cb][4 * g], a.b[rb][cb][4 * g + 1], a.b[rb][cb][4 * g + 2], a.b[rb][cb][4 * g + 3]};
+        *reinterpret_cast<f32x4*>(base + (32 * cb + c) * LDP + 32 * rb + 8 * g + 4 * h) = v;
+      }
+}
+
+// ---------------------------------------------------------------------------- cross-lane
+TTT_DEV float dpp_quad_xor1(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, false));
+}
+TTT_DEV float dpp_quad_xor2(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, false));
+}
+// Sum over the 4 lanes of a quad, result in all 4.
+TTT_DEV float quad_sum(float x) {
+  x += dpp_quad_xor1(x);
+  x += dpp_quad_xor2(x);
+  return x;
+}
+// Sum of lane l and lane l^32, result in both.
+TTT_DEV float half_sum(float x) { return x + __shfl_xor(x, 32, 64); }
+
+// ---------------------------------------------------------------------------- bf16 helpers
+TTT_DEV float bf_lo(uint32_t u) { return __builtin_bit_cast(float, u << 16); }
+TTT_DEV float bf_hi(uint32_t u) { return __builtin_bit_cast(float, u & 0xffff0000u); }
+TTT_DEV float bf2f(bf16 x) { return (float)x; }
+
+// ---------------------------------------------------------------------------- tanh-GELU family
+// gelu(x) = x * r with r = sigmoid(2c), c = K0 * x * (1 + K1 x^2); 1 - tanh(c)^2 = 4 r (1 - r).
+constexpr float GK0 = 0.79788456f;
+constexpr float GK1 = 0.044715f;
+constexpr float GK2 = 0.1070322243f;
+constexpr float LOG2E = 1.4426950408889634f;
+
+TTT_DEV float gelu_sigmoid(float x, float u) {
+  const float a = x * __builtin_fmaf(u, -2.f * GK0 * GK1 * LOG2E, -2.f * GK0 * LOG2E);  // -2c*log2(e)
+  const float e = __builtin_amdgcn_exp2f(a);
+  return __builtin_amdgcn_rcpf(1.f + e);
+}
+TTT_DEV float gelu_f(float x) { return x * gelu_sigmoid(x, x * x); }
+// value and first derivative
+TTT_DEV void gelu_fd(float x, float& g, float& d1) {
+  const float u = x * x;
+  const float r = gelu_sigmoid(x, u);
+  g = x * r;
+  d1 = __builtin_fmaf(g * (1.f - r), __builtin_fmaf(u, 2.f * GK2, 2.f * GK0), r);
+}
+// value, first and second derivative
+TTT_DEV void gelu_fdd(float x, float& g, float& d1, float& d2) {
+  const float u = x * x;
+  const float r = gelu_sigmoid(x, u);
+  const float t = __builtin_fmaf(2.f, r, -1.f);
+  const float s = 4.f * r * (1.f - r);  // 1 - t^2
+  g = x * r;
+  const float q = __builtin_fmaf(u, GK2, GK0);  // K0 + 3 K0 K1 x^2
+  d1 = __builtin_fmaf(0.5f * x * s, q, r);
+  d2 = s * (__builtin_fmaf(u, 2.f * GK2, GK0) - x * t * q * q);
+}
+
+}  // namespace ttt
