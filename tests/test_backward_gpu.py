@@ -1,0 +1,84 @@
+"""GPU parity of forward + remat backward against the CPU oracle (same seeded inputs).
+
+Bar: per tensor max|hw - ref| / max|ref| <= 2e-2 and cosine >= 0.9999 on Out and all ten gradients,
+reference = fp32 oracle on the bf16-rounded inputs."""
+import pytest
+import torch
+
+from oracle import ttt_mlp_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+MAX_REL, MIN_COS = 2e-2, 0.9999
+FWD_KEYS = ("XQ", "XK", "XV", "last_eta", "ttt_norm_weight", "ttt_norm_bias", "W1", "b1", "W2", "b2")
+UP_KEYS = ("grad_L_W1_last", "grad_L_b1_last", "grad_L_W2_last", "grad_L_b2_last", "grad_L_XQW_mini_batch")
+
+
+def run_fwd_bwd(d, cgs, hw_forward=True):
+    """Forward on the GPU (or oracle checkpoints when hw_forward is False), then backward on the GPU."""
+    import ttt_mlp_host as host
+    dev = torch.device("cuda:0")
+    B, NH, NC = d["XQ"].shape[:3]
+    t = {k: d[k].to(dev).contiguous() for k in FWD_KEYS + UP_KEYS}
+    t.update(host.alloc_forward_buffers(B, NH, NC, cgs, dev))
+    if hw_forward:
+        host.forward(t, cgs)
+    else:
+        _, ck, _ = orc.ttt_forward(*[d[k] for k in FWD_KEYS], cgs)
+        for name, v in zip(("W1_checkpoints", "b1_checkpoints", "W2_checkpoints", "b2_checkpoints"), ck):
+            t[name].copy_(v)
+        t["Out"].zero_()
+    out_before = t["Out"].clone()
+    t.update(host.alloc_backward_buffers(B, NH, NC, cgs, dev))
+    ret = host.backward(t, cgs)
+    assert ret.data_ptr() == t["Out"].data_ptr()
+    assert torch.equal(t["Out"], out_before), "backward must leave Out untouched"
+    return {k: v.float().cpu() for k, v in t.items()}
+
+
+def oracle_fwd_bwd(d, cgs):
+    out, ck, _ = orc.ttt_forward(*[d[k] for k in FWD_KEYS], cgs)
+    g = orc.ttt_backward(d["XQ"], d["XK"], d["XV"], d["last_eta"], d["ttt_norm_weight"], d["ttt_norm_bias"], ck,
+                         orc.State(d["grad_L_W1_last"], d["grad_L_b1_last"], d["grad_L_W2_last"], d["grad_L_b2_last"]),
+                         d["grad_L_XQW_mini_batch"], cgs)
+    return out, g
+
+
+def check(name, hw, ref, failures):
+    st = orc.parity_stats(hw, ref)
+    ok = bool(torch.isfinite(hw).all()) and st["max_rel"] <= MAX_REL and st["cosine"] >= MIN_COS
+    print(f"{name:24s} max_rel={st['max_rel']:.3e} cos={st['cosine']:.6f} max_abs={st['max_abs']:.3e}"
+          f"{'' if ok else '   <-- FAIL'}", flush=True)
+    if not ok:
+        failures.append((name, st["max_rel"], st["cosine"]))
+
+
+def randomize_affine(d, seed):
+    B, NH = d["XQ"].shape[:2]
+    g = torch.Generator().manual_seed(100 + seed)
+    d["b1"] = 0.02 * torch.randn(B, NH, 1, 256, generator=g)
+    d["b2"] = 0.02 * torch.randn(B, NH, 1, 64, generator=g)
+    d["ttt_norm_weight"] = 1 + 0.1 * torch.randn(1, NH, 1, 64, generator=g)
+    d["ttt_norm_bias"] = 0.1 * torch.randn(1, NH, 1, 64, generator=g)
+
+
+@pytest.mark.parametrize("B,NH,NC,cgs,seed,rand_affine", [
+    (1, 1, 1, 1, 0, False),
+    (1, 2, 4, 1, 0, False),      # the CPU-runnable reference configuration, with a backward
+    (1, 2, 4, 4, 1, True),
+    (2, 3, 9, 4, 2, True),       # ragged last checkpoint group
+    (1, 2, 6, 8, 3, True),       # group larger than the sequence
+    (1, 4, 32, 8, 4, False),
+])
+def test_backward_matches_oracle(B, NH, NC, cgs, seed, rand_affine):
+    print(f"case B={B} NH={NH} NC={NC} cgs={cgs} seed={seed}", flush=True)
+    d = orc.make_inputs(B, NH, NC, seed=seed)
+    if rand_affine:
+        randomize_affine(d, seed)
+    hw = run_fwd_bwd(d, cgs)
+    out, ref = oracle_fwd_bwd(d, cgs)
+    failures = []
+    check("Out", hw["Out"], out, failures)
+    for name, r in ref.items():
+        check(name, hw[name], r, failures)
+    assert not failures, failures

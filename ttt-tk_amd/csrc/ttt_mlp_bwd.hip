@@ -1,5 +1,858 @@
-// placeholder during bring-up
-#include "../../include/ttt_mlp.h"
+// Remat backward of the non-causal TTT-MLP layer for gfx950 (MI355X).
+//
+// Behaviour follows the upstream operator `ttt_backward` (kernel kernels/ttt_backward/ttt.cu:179-1443,
+// mathematics kernels/ttt_backward/matching.py:57-342, group walk :539-663): for every checkpoint
+// group, last to first, the forward is replayed from the checkpoint while the per-mini-batch
+// activations are saved, then the group is walked backwards producing the ten output gradients.
+//
+// Mapping: one workgroup of 4 wavefronts per (batch, head); wave w owns hidden columns [64w, 64w+64).
+// All [tokens x hidden] activations live in registers in the "Q" orientation (accumulator rows =
+// hidden, lane = token), so per-token scalars (eta, dEta partial sums) are per-lane values and sums
+// over the hidden dimension are in-register sums.  An activation that is also needed with tokens as
+// the contraction index is bounced once through a wave-private LDS tile (row store + transposing read).
+//
+// State in registers:
+//   replay : W1s [F x hid], W2s [hid x F], W2t [F x hid], b1 (accumulator-row form), b2
+//   reverse: gW1s [F x hid], gW2s [hid x F] (running gradients), W1t [hid x F], W2t [F x hid]
+//            (the weights themselves, stepped back one mini-batch at a time by undoing the update,
+//            so no per-mini-batch weight snapshot is ever written), gb1, gb2.
+// While a group is replayed the running gradients are parked in the caller's W*_init_group scratch.
+// Saved per mini-batch (caller's *_group scratch): Z1 and Z1_bar as bf16 register images
+// (Z1_group, Z1_bar_group); the two bf16 operands of the weight step, X2 (X2_group) and
+// G1 = -eta*dl/dZ1 (grad_l_wrt_Z1_group), as register images and G2 = -eta*dl/dZ2
+// (grad_x_hat_fused_group) as a tile, so that undoing the step reproduces the update bit for bit;
+// x_hat / grad_output of the fused LayerNorm loss, dl/dZ2 and the output LayerNorm's x_hat as bf16
+// [tok][F] tiles; the two std vectors in fp32.
+#include "ttt_mlp_common.hpp"
 #include "ttt_mlp_kernels.hpp"
-extern "C" int ttt_mlp_bwd_lds_bytes() { return 0; }
-extern "C" int ttt_mlp_bwd_launch(const ttt_mlp_bwd_args*, void*) { return (int)hipErrorNotSupported; }
+
+namespace ttt {
+
+constexpr int SB_TILE = 64 * LDB * 2;
+constexpr int SB_XQ = 0;
+constexpr int SB_XK = SB_XQ + SB_TILE;
+constexpr int SB_GZ2 = SB_XK + SB_TILE;   // replay: G2 = -eta*dl/dZ2 ; reverse: raw dl/dZ2
+constexpr int SB_E2 = SB_GZ2 + SB_TILE;   // reverse: G2 ; replay: XV
+constexpr int SB_A = SB_E2 + SB_TILE;     // reverse: gZ2_bar, later dZ2
+constexpr int SB_P = SB_A + SB_TILE;      // 4 fp32 partial tiles
+constexpr int SB_PTILE = 64 * LDP * 4;
+constexpr int SB_BNC = SB_P + 4 * SB_PTILE;   // 4 wave-private bounce tiles
+constexpr int SB_B2 = SB_BNC + 4 * SB_TILE;   // b2 (replay) / gb2 (reverse), 64 floats
+constexpr int SB_ETA = SB_B2 + FD * 4;
+constexpr int SB_DETA = SB_ETA + CS * 4;      // [2][4 waves][64 tokens] partial dEta sums
+constexpr int SB_RED = SB_DETA + 2 * 4 * CS * 4;  // [4 waves][2][64] final norm-grad reduction
+constexpr int SM_BWD_BYTES = SB_RED + 4 * 2 * FD * 4;
+static_assert(SM_BWD_BYTES <= 160 * 1024, "LDS budget of one gfx950 CU exceeded");
+
+// All waves run the same straight-line code, so a workgroup barrier is a valid (if heavier than
+// needed) way to order a wave-private LDS store against the transposing read that follows it.
+#define WAVE_SYNC() __syncthreads()
+
+// ------------------------------------------------------------------ register images in HBM
+// A 64x64 tile as 8 chunks of 8 bf16 per lane; chunk n of thread tid sits at (n*256 + tid)*16 bytes,
+// so every store/load instruction of a wave moves 1 KiB contiguous.
+TTT_DEV void opd_store(bf16* base, const Opd& o, int tid) {
+#pragma unroll
+  for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+    for (int s = 0; s < 4; s++) reinterpret_cast<bf16x8*>(base)[(cb * 4 + s) * NTHREADS + tid] = o.v[cb][s];
+}
+TTT_DEV Opd opd_load(const bf16* base, int tid) {
+  Opd o;
+#pragma unroll
+  for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+    for (int s = 0; s < 4; s++) o.v[cb][s] = reinterpret_cast<const bf16x8*>(base)[(cb * 4 + s) * NTHREADS + tid];
+  return o;
+}
+TTT_DEV void img_store(bf16* base, const Acc& x, int tid) { opd_store(base, cvt_chain(x), tid); }
+// Sign flip of every element (exact).
+TTT_DEV Opd opd_neg(const Opd& o) {
+  Opd r;
+#pragma unroll
+  for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      u32x4 u = __builtin_bit_cast(u32x4, o.v[cb][s]);
+      u ^= 0x80008000u;
+      r.v[cb][s] = __builtin_bit_cast(bf16x8, u);
+    }
+  return r;
+}
+TTT_DEV void img_load(const bf16* base, Acc& x, int tid) {
+#pragma unroll
+  for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      const bf16x8 v = reinterpret_cast<const bf16x8*>(base)[(cb * 4 + s) * NTHREADS + tid];
+#pragma unroll
+      for (int j = 0; j < 8; j++) x.b[s >> 1][cb][8 * (s & 1) + j] = (float)v[j];
+    }
+}
+
+// fp32 accumulator tile <-> HBM in the caller's row-major layout.  `ld` = row length, (r0, c0) =
+// origin of this wave's 64x64 block; accumulator rows are tensor rows.
+TTT_DEV void acc_load_rows(Acc& a, const float* g, int ld, int r0, int c0, int c, int h) {
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+    for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+      for (int i = 0; i < 16; i++)
+        a.b[rb][cb][i] = g[(size_t)(r0 + 32 * rb + 8 * (i >> 2) + 4 * h + (i & 3)) * ld + c0 + 32 * cb + c];
+}
+TTT_DEV void acc_store_rows(const Acc& a, float* g, int ld, int r0, int c0, int c, int h) {
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+    for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+      for (int i = 0; i < 16; i++)
+        g[(size_t)(r0 + 32 * rb + 8 * (i >> 2) + 4 * h + (i & 3)) * ld + c0 + 32 * cb + c] = a.b[rb][cb][i];
+}
+// Same, but accumulator rows are tensor COLUMNS (the tile holds the transpose of the block).
+TTT_DEV void acc_load_cols(Acc& a, const float* g, int ld, int r0, int c0, int c, int h) {
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+    for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+      for (int i = 0; i < 16; i++)
+        a.b[rb][cb][i] = g[(size_t)(r0 + 32 * cb + c) * ld + c0 + 32 * rb + 8 * (i >> 2) + 4 * h + (i & 3)];
+}
+// Bias vector in accumulator-row form: element of row r, identical in every lane column.
+TTT_DEV void rowvec_load(f32x16 (&v)[2], const float* g, int h) {
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) v[rb][i] = g[32 * rb + 8 * (i >> 2) + 4 * h + (i & 3)];
+}
+TTT_DEV void rowvec_store(const f32x16 (&v)[2], float* g, int h) {  // call from lanes with c == 0
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) g[32 * rb + 8 * (i >> 2) + 4 * h + (i & 3)] = v[rb][i];
+}
+TTT_DEV void rowvec_store_lds(const f32x16 (&v)[2], float* s, int h) {  // call from lanes with c == 0
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      f32x4 x = {v[rb][4 * g], v[rb][4 * g + 1], v[rb][4 * g + 2], v[rb][4 * g + 3]};
+      *reinterpret_cast<f32x4*>(s + 32 * rb + 8 * g + 4 * h) = x;
+    }
+}
+// v[row block] += sum over the 64-long contraction of operand `a` (lane = row index).
+TTT_DEV void rowsum_mma(f32x16 (&v)[2], const Opd& a, bf16x8 ones) {
+#pragma unroll
+  for (int s = 0; s < 4; s++)
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++) v[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v[rb][s], ones, v[rb], 0, 0, 0);
+}
+TTT_DEV void acc_init_rowvec(Acc& a, const f32x16 (&v)[2]) {
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+    for (int cb = 0; cb < 2; cb++) a.b[rb][cb] = v[rb];
+}
+// Swap the roles of lane index and contraction index of an operand through a wave-private tile.
+TTT_DEV Opd bounce(bf16* tile, const Opd& o, int lane) {
+  WAVE_SYNC();  // earlier readers of the tile are done
+  lds_store_rows_kappa(tile, o, lane & 31, lane >> 5);
+  WAVE_SYNC();
+  return lds_tr_kappa(tile, lane);
+}
+TTT_DEV void acc_scale(Acc& a, float s) {
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+    for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) a.b[rb][cb][i] *= s;
+}
+
+// ------------------------------------------------------------------ LayerNorm-lane helpers
+// A lane of the LayerNorm stage owns token `tok` and features 16r + 4fq + e (r, e in 0..3).
+TTT_DEV void ln_load(float (&x)[4][4], const bf16* row, int fq) {
+#pragma unroll
+  for (int r = 0; r < 4; r++) {
+    const bf16x4 v = *reinterpret_cast<const bf16x4*>(row + 16 * r + 4 * fq);
+#pragma unroll
+    for (int e = 0; e < 4; e++) x[r][e] = (float)v[e];
+  }
+}
+TTT_DEV void ln_store(bf16* row, const float (&x)[4][4], int fq) {
+#pragma unroll
+  for (int r = 0; r < 4; r++) {
+    bf16x4 v;
+#pragma unroll
+    for (int e = 0; e < 4; e++) v[e] = (bf16)x[r][e];
+    *reinterpret_cast<bf16x4*>(row + 16 * r + 4 * fq) = v;
+  }
+}
+// dst = bf16(float(dst) + x): the operator accumulates into these outputs.
+TTT_DEV void ln_accumulate(bf16* row, const float (&x)[4][4], int fq) {
+#pragma unroll
+  for (int r = 0; r < 4; r++) {
+    bf16x4 v = *reinterpret_cast<const bf16x4*>(row + 16 * r + 4 * fq);
+#pragma unroll
+    for (int e = 0; e < 4; e++) v[e] = (bf16)((float)v[e] + x[r][e]);
+    *reinterpret_cast<bf16x4*>(row + 16 * r + 4 * fq) = v;
+  }
+}
+// Sum of the 4 shard partial tiles (plus a bias vector) for this lane's 16 features.
+TTT_DEV void ln_gather(float (&z)[4][4], const float* s_P, const float* s_bias, int tok, int fq) {
+#pragma unroll
+  for (int r = 0; r < 4; r++) {
+    f32x4 a = *reinterpret_cast<const f32x4*>(s_bias + 16 * r + 4 * fq);
+#pragma unroll
+    for (int v = 0; v < 4; v++) a += *reinterpret_cast<const f32x4*>(s_P + v * 64 * LDP + tok * LDP + 16 * r + 4 * fq);
+#pragma unroll
+    for (int e = 0; e < 4; e++) z[r][e] = a[e];
+  }
+}
+TTT_DEV float sum16(const float (&x)[4][4]) {
+  float s = 0.f;
+#pragma unroll
+  for (int r = 0; r < 4; r++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) s += x[r][e];
+  return s;
+}
+TTT_DEV float dot16(const float (&x)[4][4], const float (&y)[4][4]) {
+  float s = 0.f;
+#pragma unroll
+  for (int r = 0; r < 4; r++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) s = __builtin_fmaf(x[r][e], y[r][e], s);
+  return s;
+}
+// z -> x_hat in place, returns 1/std; *std_out = std.
+TTT_DEV float ln_normalize(float (&z)[4][4], float* std_out) {
+  const float mu = quad_sum(sum16(z)) * (1.f / FD);
+  float var = 0.f;
+#pragma unroll
+  for (int r = 0; r < 4; r++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) { z[r][e] -= mu; var = __builtin_fmaf(z[r][e], z[r][e], var); }
+  const float v = quad_sum(var) * (1.f / FD) + LN_EPS;
+  const float rstd = __builtin_amdgcn_rsqf(v);
+#pragma unroll
+  for (int r = 0; r < 4; r++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) z[r][e] *= rstd;
+  *std_out = v * rstd;  // sqrt(v)
+  return rstd;
+}
+
+// 16-byte chunk staging of one [64][64] bf16 tile from HBM into an LDS tile with row stride LDB.
+TTT_DEV void stage_tile(bf16* s_tile, const bf16* g_tile, int tid) {
+#pragma unroll
+  for (int r = 0; r < 2; r++) {
+    const int id = tid + 256 * r;
+    *reinterpret_cast<u32x4*>(s_tile + (id >> 3) * LDB + (id & 7) * 8) = reinterpret_cast<const u32x4*>(g_tile)[id];
+  }
+}
+
+__global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  bf16* s_xq = reinterpret_cast<bf16*>(smem + SB_XQ);
+  bf16* s_xk = reinterpret_cast<bf16*>(smem + SB_XK);
+  bf16* s_gz2 = reinterpret_cast<bf16*>(smem + SB_GZ2);
+  bf16* s_e2 = reinterpret_cast<bf16*>(smem + SB_E2);
+  bf16* s_a = reinterpret_cast<bf16*>(smem + SB_A);
+  float* s_P = reinterpret_cast<float*>(smem + SB_P);
+  float* s_b2 = reinterpret_cast<float*>(smem + SB_B2);
+  float* s_eta = reinterpret_cast<float*>(smem + SB_ETA);
+  float* s_deta = reinterpret_cast<float*>(smem + SB_DETA);
+  float* s_red = reinterpret_cast<float*>(smem + SB_RED);
+
+  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, h = lane >> 5, c = lane & 31;
+  const int q = lane >> 2, fq = lane & 3, tok = 16 * w + q;
+  const int bh = blockIdx.x, head = bh % p.NH;
+  float* s_Pw = s_P + w * 64 * LDP;
+  bf16* s_bnc = reinterpret_cast<bf16*>(smem + SB_BNC) + w * 64 * LDB;
+  const int cgs = p.cgs;
+
+  float gam[4][4], bet[4][4];
+#pragma unroll
+  for (int r = 0; r < 4; r++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      gam[r][e] = p.ttt_norm_weight[head * FD + 16 * r + 4 * fq + e];
+      bet[r][e] = p.ttt_norm_bias[head * FD + 16 * r + 4 * fq + e];
+    }
+  float dgam[4][4], dbet[4][4];
+#pragma unroll
+  for (int r = 0; r < 4; r++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) dgam[r][e] = dbet[r][e] = 0.f;
+  bf16x8 ones;
+#pragma unroll
+  for (int j = 0; j < 8; j++) ones[j] = (bf16)1.0f;
+
+  const size_t x_base = (size_t)bh * p.NC * (CS * FD);
+  const size_t eta_base = (size_t)bh * p.NC * CS;
+  // per-(b,h) scratch bases
+  const size_t g_TF = (size_t)bh * cgs * (CS * FD);     // [cgs][64][64] tiles
+  const size_t g_TH = (size_t)bh * cgs * (CS * HID);    // [cgs][64][256] tiles (register images)
+  const size_t g_T = (size_t)bh * cgs * CS;             // [cgs][64] vectors
+  float* park_W1 = p.W1_init_group + (size_t)bh * cgs * FD * HID;
+  float* park_W2 = p.W2_init_group + (size_t)bh * cgs * HID * FD;
+  float* park_b1 = p.b1_init_group + (size_t)bh * cgs * HID;
+  float* park_b2 = p.b2_init_group + (size_t)bh * cgs * FD;
+
+  // running gradients wrt the state after the last mini-batch
+  Acc gW1s, gW2s;
+  f32x16 gb1[2], gb2[2];
+  acc_load_rows(gW1s, p.grad_L_W1_last + (size_t)bh * FD * HID, HID, 0, 64 * w, c, h);
+  acc_load_rows(gW2s, p.grad_L_W2_last + (size_t)bh * HID * FD, FD, 64 * w, 0, c, h);
+  rowvec_load(gb1, p.grad_L_b1_last + (size_t)bh * HID + 64 * w, h);
+  rowvec_load(gb2, p.grad_L_b2_last + (size_t)bh * FD, h);
+
+  for (int k = p.K - 1; k >= 0; k--) {
+    const int n_mb = min(cgs, p.NC - k * cgs);
+    Acc W2t;  // survives from the replay into the reverse walk
+    Acc W1t;
+    // ================================================================= replay
+    {
+      // park the running gradients
+      acc_store_rows(gW1s, park_W1, HID, 0, 64 * w, c, h);
+      acc_store_rows(gW2s, park_W2, FD, 64 * w, 0, c, h);
+      if (c == 0) {
+        rowvec_store(gb1, park_b1 + 64 * w, h);
+        if (w == 0) rowvec_store(gb2, park_b2, h);
+      }
+      Acc W1s, W2s;
+      f32x16 b1[2], b2[2];
+      const size_t slot = (size_t)bh * p.K + k;
+      acc_load_rows(W1s, p.W1_ck + slot * FD * HID, HID, 0, 64 * w, c, h);
+      acc_load_rows(W2s, p.W2_ck + slot * HID * FD, FD, 64 * w, 0, c, h);
+      acc_load_cols(W2t, p.W2_ck + slot * HID * FD, FD, 64 * w, 0, c, h);
+      rowvec_load(b1, p.b1_ck + slot * HID + 64 * w, h);
+      rowvec_load(b2, p.b2_ck + slot * FD, h);
+      __syncthreads();  // previous group's readers of s_b2 are done
+      if (tid < FD) s_b2[tid] = p.b2_ck[slot * FD + tid];
+
+      for (int j = 0; j < n_mb; j++) {
+        const int mb = k * cgs + j;
+        const size_t xo = x_base + (size_t)mb * (CS * FD);
+        __syncthreads();
+        stage_tile(s_xq, p.XQ + xo, tid);
+        stage_tile(s_xk, p.XK + xo, tid);
+        stage_tile(s_e2, p.XV + xo, tid);
+        if (tid < CS) s_eta[tid] = bf2f(p.last_eta[eta_base + (size_t)mb * CS + tid]);
+        __syncthreads();
+
+        // Z1^T = W1s^T XK^T + b1  (rows hid, lane = tok)
+        Acc x2, d1;
+        {
+          const Opd w1A = cvt_chain(W1s);
+          const Opd xkB = lds_rows_kappa(s_xk, c, h);
+          acc_init_rowvec(x2, b1);
+          mma(x2, w1A, xkB);
+          img_store(p.Z1_group + g_TH + (size_t)j * (CS * HID), x2, tid);
+#pragma unroll
+          for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+            for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+              for (int i = 0; i < 16; i++) {
+                float g, d;
+                gelu_fd(x2.b[rb][cb][i], g, d);
+                x2.b[rb][cb][i] = g;
+                d1.b[rb][cb][i] = d;
+              }
+        }
+        const Opd x2Q = cvt_chain(x2);  // lane = tok, contraction = hid
+        opd_store(p.X2_group + g_TH + (size_t)j * (CS * HID), x2Q, tid);
+        {
+          const Opd w2A = cvt_chain(W2s);
+          Acc z2;
+          acc_zero(z2);
+          mma(z2, w2A, x2Q);
+          lds_store_partial(s_Pw, z2, c, h);
+        }
+        __syncthreads();
+        // fused LayerNorm + reconstruction-loss gradient; saves for the reverse walk
+        {
+          float z[4][4], kv[4][4], vv[4][4];
+          ln_gather(z, s_P, s_b2, tok, fq);
+          float sd;
+          const float rstd = ln_normalize(z, &sd);
+          ln_load(kv, s_xk + tok * LDB, fq);
+          ln_load(vv, s_e2 + tok * LDB, fq);
+          float go[4][4], gx[4][4];
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              go[r][e] = __builtin_fmaf(gam[r][e], z[r][e], bet[r][e]) - (vv[r][e] - kv[r][e]);
+              gx[r][e] = go[r][e] * gam[r][e];
+            }
+          const float s1 = quad_sum(sum16(gx)), s2 = quad_sum(dot16(gx, z));
+          const float sc = rstd * (1.f / FD), neg_eta = -s_eta[tok];
+          float gz[4][4], g2[4][4];
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              gz[r][e] = (FD * gx[r][e] - s1 - z[r][e] * s2) * sc;
+              g2[r][e] = neg_eta * gz[r][e];
+            }
+          ln_store(s_gz2 + tok * LDB, g2, fq);
+          const size_t so = g_TF + (size_t)j * (CS * FD) + tok * FD;
+          ln_store(p.x_hat_fused_group + so, z, fq);
+          ln_store(p.grad_output_fused_group + so, go, fq);
+          ln_store(p.grad_l_wrt_Z2_group + so, gz, fq);
+          ln_store(p.grad_x_hat_fused_group + so, g2, fq);   // the exact bf16 operand of the weight step
+          if (fq == 0) p.std_fused_group[g_T + (size_t)j * CS + tok] = sd;
+        }
+        __syncthreads();
+        // G1^T = (W2t^T... rows hid, lane = tok) * gelu'(Z1); weight step
+        {
+          const Opd g2B = lds_rows_kappa(s_gz2, c, h);   // lane = tok, contraction = F
+          const Opd w2tA = cvt_chain(W2t);               // lane = hid, contraction = F
+          Acc g1;
+          acc_zero(g1);
+          mma(g1, w2tA, g2B);
+#pragma unroll
+          for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+            for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+              for (int i = 0; i < 16; i++) g1.b[rb][cb][i] *= d1.b[rb][cb][i];
+          const Opd g1Q = cvt_chain(g1);
+          opd_store(p.grad_l_wrt_Z1_group + g_TH + (size_t)j * (CS * HID), g1Q, tid);
+          const Opd x2P = bounce(s_bnc, x2Q, lane);      // lane = hid, contraction = tok
+          const Opd g1P = bounce(s_bnc, g1Q, lane);
+          const Opd g2T = lds_tr_kappa(s_gz2, lane);     // lane = F, contraction = tok
+          mma(W2s, x2P, g2T);
+          mma(W2t, g2T, x2P);
+          rowsum_mma(b2, g2T, ones);
+          const Opd xkT = lds_tr_kappa(s_xk, lane);      // lane = F, contraction = tok
+          mma(W1s, xkT, g1P);
+          rowsum_mma(b1, g1P, ones);
+        }
+        if (w == 0 && c == 0) rowvec_store_lds(b2, s_b2, h);
+        // post-update forward on XQ
+        {
+          const Opd w1A = cvt_chain(W1s);
+          const Opd xqB = lds_rows_kappa(s_xq, c, h);
+          Acc z1b;
+          acc_init_rowvec(z1b, b1);
+          mma(z1b, w1A, xqB);
+          img_store(p.Z1_bar_group + g_TH + (size_t)j * (CS * HID), z1b, tid);
+#pragma unroll
+          for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+            for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+              for (int i = 0; i < 16; i++) z1b.b[rb][cb][i] = gelu_f(z1b.b[rb][cb][i]);
+          const Opd x2bQ = cvt_chain(z1b);
+          const Opd w2A = cvt_chain(W2s);
+          Acc z2;
+          acc_zero(z2);
+          mma(z2, w2A, x2bQ);
+          lds_store_partial(s_Pw, z2, c, h);
+        }
+        __syncthreads();
+        {
+          float z[4][4];
+          ln_gather(z, s_P, s_b2, tok, fq);
+          float sd;
+          ln_normalize(z, &sd);
+          ln_store(p.x_hat_ln_group + g_TF + (size_t)j * (CS * FD) + tok * FD, z, fq);
+          if (fq == 0) p.std_ln_group[g_T + (size_t)j * CS + tok] = sd;
+        }
+      }
+      // W1t = transpose of W1s through this wave's fp32 partial tile
+      __syncthreads();
+      lds_store_partial(s_Pw, W1s, c, h);  // stored [hid][F]
+      __syncthreads();
+#pragma unroll
+      for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+        for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+          for (int i = 0; i < 16; i++)
+            W1t.b[rb][cb][i] = s_Pw[(32 * rb + 8 * (i >> 2) + 4 * h + (i & 3)) * LDP + 32 * cb + c];
+      // running gradients back into registers
+      acc_load_rows(gW1s, park_W1, HID, 0, 64 * w, c, h);
+      acc_load_rows(gW2s, park_W2, FD, 64 * w, 0, c, h);
+      rowvec_load(gb1, park_b1 + 64 * w, h);
+      rowvec_load(gb2, park_b2, h);
+    }
+
+    // ================================================================= reverse walk
+    for (int j = n_mb - 1; j >= 0; j--) {
+      const int mb = k * cgs + j;
+      const size_t xo = x_base + (size_t)mb * (CS * FD);
+      const size_t so = g_TF + (size_t)j * (CS * FD);
+      const float eta_l = bf2f(p.last_eta[eta_base + (size_t)mb * CS + 32 * 0 + c]);      // token c
+      const float eta_h = bf2f(p.last_eta[eta_base + (size_t)mb * CS + 32 * 1 + c]);      // token 32 + c
+      const float eta_cb[2] = {eta_l, eta_h};  // eta of the token this lane holds in column block cb
+      __syncthreads();
+      stage_tile(s_xq, p.XQ + xo, tid);
+      stage_tile(s_xk, p.XK + xo, tid);
+      stage_tile(s_gz2, p.grad_l_wrt_Z2_group + so, tid);
+      stage_tile(s_e2, p.grad_x_hat_fused_group + so, tid);   // G2 = -eta * dl/dZ2 as used by the weight step
+      if (tid < CS) s_eta[tid] = bf2f(p.last_eta[eta_base + (size_t)mb * CS + tid]);
+
+      // ---- output LayerNorm backward (LayerNorm lanes)
+      float gO[4][4];
+      ln_load(gO, p.grad_L_XQW + xo + tok * FD, fq);
+      {
+        float xh[4][4], gx[4][4];
+        ln_load(xh, p.x_hat_ln_group + so + tok * FD, fq);
+        const float sd = p.std_ln_group[g_T + (size_t)j * CS + tok];
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            dbet[r][e] += gO[r][e];
+            dgam[r][e] = __builtin_fmaf(gO[r][e], xh[r][e], dgam[r][e]);
+            gx[r][e] = gO[r][e] * gam[r][e];
+          }
+        const float s1 = quad_sum(sum16(gx)), s2 = quad_sum(dot16(gx, xh));
+        const float sc = 1.f / (FD * sd);
+        float gz[4][4];
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) gz[r][e] = (FD * gx[r][e] - s1 - xh[r][e] * s2) * sc;
+        ln_store(s_a + tok * LDB, gz, fq);  // gZ2_bar
+      }
+      __syncthreads();
+
+      // ---- post-update forward, backwards (uses the state AFTER this mini-batch)
+      Opd gw1T, gw2T;  // running gradients with lane/contraction swapped, taken after their first update
+      {
+        Acc z1b;
+        img_load(p.Z1_bar_group + g_TH + (size_t)j * (CS * HID), z1b, tid);
+        Acc d1b;
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+          for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+              float g, d;
+              gelu_fd(z1b.b[rb][cb][i], g, d);
+              z1b.b[rb][cb][i] = g;   // X2_bar
+              d1b.b[rb][cb][i] = d;
+            }
+        const Opd x2bQ = cvt_chain(z1b);
+        const Opd gz2bB = lds_rows_kappa(s_a, c, h);     // lane = tok, contraction = F
+        const Opd w2tA = cvt_chain(W2t);                 // lane = hid, contraction = F   (W2 after the step)
+        Acc gz1b;
+        acc_zero(gz1b);
+        mma(gz1b, w2tA, gz2bB);                          // rows hid, lane = tok
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+          for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) gz1b.b[rb][cb][i] *= d1b.b[rb][cb][i];
+        const Opd gz1bQ = cvt_chain(gz1b);               // lane = tok, contraction = hid
+        {
+          const Opd w1tA = cvt_chain(W1t);               // lane = F, contraction = hid   (W1 after the step)
+          Acc dq;
+          acc_zero(dq);
+          mma(dq, w1tA, gz1bQ);                          // rows F, lane = tok
+          lds_store_partial(s_Pw, dq, c, h);
+        }
+        const Opd x2bP = bounce(s_bnc, x2bQ, lane);      // lane = hid, contraction = tok
+        const Opd gz1bP = bounce(s_bnc, gz1bQ, lane);
+        const Opd gz2bT = lds_tr_kappa(s_a, lane);       // lane = F, contraction = tok
+        mma(gW2s, x2bP, gz2bT);
+        rowsum_mma(gb2, gz2bT, ones);
+        const Opd xqT = lds_tr_kappa(s_xq, lane);
+        mma(gW1s, xqT, gz1bP);
+        rowsum_mma(gb1, gz1bP, ones);
+        gw1T = bounce(s_bnc, cvt_chain(gW1s), lane);     // lane = F,   contraction = hid
+        gw2T = bounce(s_bnc, cvt_chain(gW2s), lane);     // lane = hid, contraction = F
+      }
+      __syncthreads();  // partial dXQ tiles complete; gZ2_bar tile no longer needed
+      if (w == 0 && c == 0) rowvec_store_lds(gb2, s_b2, h);  // gb2 after adding sum_t gZ2_bar
+      {
+        float z[4][4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          f32x4 a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int v = 0; v < 4; v++) a += *reinterpret_cast<const f32x4*>(s_P + v * 64 * LDP + tok * LDP + 16 * r + 4 * fq);
+#pragma unroll
+          for (int e = 0; e < 4; e++) z[r][e] = a[e] + gO[r][e];
+        }
+        ln_accumulate(p.grad_L_XQ + xo + tok * FD, z, fq);
+      }
+
+      // ---- the weight step, backwards
+      Acc d1, d2, S, R;
+      Opd x2P;
+      {
+        {
+          Acc z1;
+          img_load(p.Z1_group + g_TH + (size_t)j * (CS * HID), z1, tid);
+#pragma unroll
+          for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+            for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+              for (int i = 0; i < 16; i++) {
+                float g, a, b;
+                gelu_fdd(z1.b[rb][cb][i], g, a, b);
+                d1.b[rb][cb][i] = a;
+                d2.b[rb][cb][i] = b;
+              }
+        }
+        // X2 exactly as the replay fed it to the weight step
+        const Opd x2Q = opd_load(p.X2_group + g_TH + (size_t)j * (CS * HID), tid);   // lane = tok, contraction = hid
+        x2P = bounce(s_bnc, x2Q, lane);                  // lane = hid, contraction = tok
+        // undo the W2 step with the very operands that made it: W2 before = W2 after - X2^T G2
+        {
+          const Opd g2Tn = opd_neg(lds_tr_kappa(s_e2, lane));   // lane = F, contraction = tok
+          mma(W2t, g2Tn, x2P);
+        }
+        const Opd w2tA = cvt_chain(W2t);                 // W2 before the step: lane = hid, contraction = F
+        const Opd gz2B = lds_rows_kappa(s_gz2, c, h);    // lane = tok, contraction = F
+        acc_zero(R);
+        mma(R, w2tA, gz2B);                              // R = gZ2 W2^T  (rows hid, lane = tok)
+        // S = XK gW1 + gb1
+        {
+          const Opd gw1A = cvt_chain(gW1s);              // lane = hid, contraction = F
+          const Opd xkB = lds_rows_kappa(s_xk, c, h);
+          acc_init_rowvec(S, gb1);
+          mma(S, gw1A, xkB);
+        }
+        // partial ggZ2 / (-eta): gW2^T X2^T + W2^T (S*d1)^T, and the first dEta partial sum
+        Acc pz;
+        acc_zero(pz);
+        {
+          const Opd gw2A = cvt_chain(gW2s);              // lane = F, contraction = hid
+          mma(pz, gw2A, x2Q);                            // rows F, lane = tok
+        }
+        float de1[2] = {0.f, 0.f}, de3[2] = {0.f, 0.f};
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+          for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+              for (int jj = 0; jj < 8; jj++)
+                de1[cb] = __builtin_fmaf((float)gz2B.v[cb][2 * rb + t][jj], pz.b[rb][cb][8 * t + jj], de1[cb]);
+        Acc u;
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+          for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+              const float gz1 = R.b[rb][cb][i] * d1.b[rb][cb][i];        // dl/dZ1 (no eta)
+              de3[cb] = __builtin_fmaf(gz1, S.b[rb][cb][i], de3[cb]);
+              u.b[rb][cb][i] = S.b[rb][cb][i] * d1.b[rb][cb][i];
+            }
+        const Opd uQ = cvt_chain(u);
+        {
+          const Opd w2sA = bounce(s_bnc, w2tA, lane);    // W2 before the step: lane = F, contraction = hid
+          mma(pz, w2sA, uQ);
+        }
+        __syncthreads();  // dXQ readers of the partial tiles are done
+        lds_store_partial(s_Pw, pz, c, h);
+#pragma unroll
+        for (int cb = 0; cb < 2; cb++) {
+          const float a = half_sum(de1[cb]), b = half_sum(de3[cb]);
+          if (h == 0) {
+            s_deta[(0 * 4 + w) * CS + 32 * cb + c] = a;
+            s_deta[(1 * 4 + w) * CS + 32 * cb + c] = b;
+          }
+        }
+        // undo the W1 step with the saved operand G1 = -eta * dl/dZ1: W1 before = W1 after - XK^T G1
+        const Opd g1Q = opd_load(p.grad_l_wrt_Z1_group + g_TH + (size_t)j * (CS * HID), tid);  // lane = tok
+        {
+          const Opd g1Pn = opd_neg(bounce(s_bnc, g1Q, lane));   // lane = hid, contraction = tok
+          const Opd xkT = lds_tr_kappa(s_xk, lane);             // lane = F,   contraction = tok
+          mma(W1t, g1Pn, xkT);
+        }
+        // u <- -eta * S * d1  (the gradient wrt dl/dZ1 times gelu')
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+          for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) u.b[rb][cb][i] *= -eta_cb[cb];
+        const Opd uP = bounce(s_bnc, cvt_chain(u), lane);       // lane = hid, contraction = tok
+        const Opd gz2T = lds_tr_kappa(s_gz2, lane);             // lane = F,   contraction = tok
+        __syncthreads();  // all partial ggZ2 tiles and dEta partial sums are in LDS
+        // (gW2s += u^T gZ2 is applied below, after the old gW2 has served its last product)
+
+        // ---- second-order pass through the fused LayerNorm loss (LayerNorm lanes)
+        float gy[4][4];
+        {
+          float gg[4][4], xh[4][4], go[4][4], gz[4][4];
+          ln_gather(gg, s_P, s_b2, tok, fq);
+          const float neg_eta = -s_eta[tok];
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) gg[r][e] *= neg_eta;                 // grad wrt dl/dZ2
+          ln_load(xh, p.x_hat_fused_group + so + tok * FD, fq);
+          ln_load(go, p.grad_output_fused_group + so + tok * FD, fq);
+          ln_load(gz, s_gz2 + tok * LDB, fq);
+          const float sd = p.std_fused_group[g_T + (size_t)j * CS + tok];
+          const float rsd = 1.f / sd;
+          // dEta: -(sum_F gZ2*(X2 gW2 + gb2) + sum_H gZ1*(XK gW1 + gb1))
+          {
+            float bias_dot = 0.f;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+              const f32x4 bv = *reinterpret_cast<const f32x4*>(s_b2 + 16 * r + 4 * fq);
+#pragma unroll
+              for (int e = 0; e < 4; e++) bias_dot = __builtin_fmaf(gz[r][e], bv[e], bias_dot);
+            }
+            bias_dot = quad_sum(bias_dot);
+            float tot = bias_dot;
+#pragma unroll
+            for (int v = 0; v < 8; v++) tot += s_deta[v * CS + tok];
+            if (fq == 0) {
+              bf16* dst = p.grad_L_last_eta + eta_base + (size_t)mb * CS + tok;
+              *dst = (bf16)((float)*dst - tot);
+            }
+          }
+          float gxh[4][4];
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) gxh[r][e] = go[r][e] * gam[r][e];
+          const float s0 = quad_sum(sum16(gg)), a = quad_sum(dot16(gg, xh)), bb = quad_sum(dot16(gxh, xh));
+          float gx[4][4], gstd[4][4];
+          const float inv = rsd * (1.f / FD);
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              const float ggx = (gg[r][e] - (s0 + xh[r][e] * a) * (1.f / FD)) * rsd;
+              gy[r][e] = gam[r][e] * ggx;
+              dgam[r][e] += go[r][e] * ggx + gy[r][e] * xh[r][e];
+              dbet[r][e] += gy[r][e];
+              gx[r][e] = gy[r][e] * gam[r][e] - (gxh[r][e] * a + gg[r][e] * bb) * inv;
+              gstd[r][e] = (-gx[r][e] * xh[r][e] - gg[r][e] * gz[r][e]) * rsd;
+            }
+          const float sg = quad_sum(sum16(gstd)), sx = quad_sum(sum16(gx));
+          float dz2[4][4], dxv[4][4];
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              dz2[r][e] = gx[r][e] * rsd + (sg * xh[r][e] - sx * rsd) * (1.f / FD);
+              dxv[r][e] = -gy[r][e];
+            }
+          ln_store(s_a + tok * LDB, dz2, fq);
+          ln_accumulate(p.grad_L_XV + xo + tok * FD, dxv, fq);
+        }
+        __syncthreads();  // dZ2 tile complete; partial tiles free again
+
+        // ---- inner MLP, backwards (uses the state BEFORE this mini-batch)
+        {
+          Acc dx2;
+          acc_zero(dx2);
+          mma(dx2, gw2T, gz2B);                          // P2 = gZ2 gW2^T  (rows hid, lane = tok)
+#pragma unroll
+          for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+            for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+              for (int i = 0; i < 16; i++) dx2.b[rb][cb][i] *= -eta_cb[cb];
+          const Opd dz2B = lds_rows_kappa(s_a, c, h);    // lane = tok, contraction = F
+          mma(dx2, w2tA, dz2B);                          // + dZ2 W2^T
+          // dZ1 = dX2*gelu' - eta * R * S * gelu''   with R = gZ2 W2^T, dl/dZ1 = R*gelu'
+#pragma unroll
+          for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+            for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+              for (int i = 0; i < 16; i++) {
+                const float r0 = R.b[rb][cb][i];
+                dx2.b[rb][cb][i] = dx2.b[rb][cb][i] * d1.b[rb][cb][i]
+                                   - eta_cb[cb] * r0 * S.b[rb][cb][i] * d2.b[rb][cb][i];
+              }
+          const Opd dz1Q = cvt_chain(dx2);               // lane = tok, contraction = hid
+          {
+            Acc dk;
+            acc_zero(dk);
+            mma(dk, gw1T, g1Q);                          // -eta * gZ1 gW1^T   (rows F, lane = tok)
+            mma(dk, cvt_chain(W1t), dz1Q);               // + dZ1 W1^T  (W1 before the step)
+            lds_store_partial(s_Pw, dk, c, h);
+          }
+          const Opd dz1P = bounce(s_bnc, dz1Q, lane);    // lane = hid, contraction = tok
+          const Opd dz2T = lds_tr_kappa(s_a, lane);      // lane = F,   contraction = tok
+          mma(gW2s, uP, gz2T);
+          mma(gW2s, x2P, dz2T);
+          rowsum_mma(gb2, dz2T, ones);
+          const Opd xkT = lds_tr_kappa(s_xk, lane);
+          mma(gW1s, xkT, dz1P);
+          rowsum_mma(gb1, dz1P, ones);
+        }
+        __syncthreads();  // partial dXK tiles complete
+        {
+          float z[4][4];
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            f32x4 a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int v = 0; v < 4; v++) a += *reinterpret_cast<const f32x4*>(s_P + v * 64 * LDP + tok * LDP + 16 * r + 4 * fq);
+#pragma unroll
+            for (int e = 0; e < 4; e++) z[r][e] = a[e] + gy[r][e];
+          }
+          ln_accumulate(p.grad_L_XK + xo + tok * FD, z, fq);
+        }
+      }
+    }
+  }
+
+  // ---- outputs that are written once
+  acc_store_rows(gW1s, p.grad_L_W1_init + (size_t)bh * FD * HID, HID, 0, 64 * w, c, h);
+  acc_store_rows(gW2s, p.grad_L_W2_init + (size_t)bh * HID * FD, FD, 64 * w, 0, c, h);
+  if (c == 0) {
+    rowvec_store(gb1, p.grad_L_b1_init + (size_t)bh * HID + 64 * w, h);
+    if (w == 0) rowvec_store(gb2, p.grad_L_b2_init + (size_t)bh * FD, h);
+  }
+  // norm-weight / norm-bias gradients: sum over the 16 tokens of the wave, then over the 4 waves
+#pragma unroll
+  for (int r = 0; r < 4; r++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      float a = dgam[r][e], b = dbet[r][e];
+#pragma unroll
+      for (int m = 4; m < 64; m <<= 1) {
+        a += __shfl_xor(a, m, 64);
+        b += __shfl_xor(b, m, 64);
+      }
+      if (q == 0) {
+        s_red[(w * 2 + 0) * FD + 16 * r + 4 * fq + e] = a;
+        s_red[(w * 2 + 1) * FD + 16 * r + 4 * fq + e] = b;
+      }
+    }
+  __syncthreads();
+  if (tid < 2 * FD) {
+    const int which = tid / FD, f = tid % FD;
+    float s = 0.f;
+#pragma unroll
+    for (int v = 0; v < 4; v++) s += s_red[(v * 2 + which) * FD + f];
+    (which == 0 ? p.grad_L_ttt_norm_weight : p.grad_L_ttt_norm_bias)[(size_t)bh * FD + f] = s;
+  }
+}
+
+}  // namespace ttt
+
+extern "C" int ttt_mlp_bwd_lds_bytes() { return ttt::SM_BWD_BYTES; }
+
+hipError_t ttt_mlp_bwd_enqueue(const ttt::BwdParams& p, hipStream_t stream) {
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(ttt::ttt_mlp_bwd_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, ttt::SM_BWD_BYTES);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(ttt::ttt_mlp_bwd_kernel, dim3(p.B * p.NH), dim3(ttt::NTHREADS), ttt::SM_BWD_BYTES, stream, p);
+  return hipGetLastError();
+}

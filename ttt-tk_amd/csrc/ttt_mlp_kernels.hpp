@@ -14,8 +14,28 @@ struct FwdParams {
   int B, NH, NC, K, cgs;
 };
 
+struct BwdParams {
+  const __bf16 *XQ, *XK, *XV, *last_eta;
+  const float *ttt_norm_weight, *ttt_norm_bias;
+  const float *W1_ck, *b1_ck, *W2_ck, *b2_ck;
+  float *W1_init_group, *b1_init_group, *W2_init_group, *b2_init_group;
+  __bf16* x_hat_ln_group;
+  float* std_ln_group;
+  __bf16 *X2_group, *Z1_group, *Z1_bar_group, *X2_bar_group;
+  __bf16 *grad_l_wrt_Z2_group, *grad_l_wrt_Z1_group;
+  __bf16 *x_hat_fused_group, *grad_x_hat_fused_group, *grad_output_fused_group;
+  float* std_fused_group;
+  const float *grad_L_W1_last, *grad_L_b1_last, *grad_L_W2_last, *grad_L_b2_last;
+  const __bf16* grad_L_XQW;
+  float *grad_L_ttt_norm_weight, *grad_L_ttt_norm_bias;
+  float *grad_L_W1_init, *grad_L_b1_init, *grad_L_W2_init, *grad_L_b2_init;
+  __bf16 *grad_L_last_eta, *grad_L_XQ, *grad_L_XK, *grad_L_XV;
+  int B, NH, NC, K, cgs;
+};
+
 }  // namespace ttt
 
 hipError_t ttt_mlp_fwd_enqueue(const ttt::FwdParams& p, hipStream_t stream);
+hipError_t ttt_mlp_bwd_enqueue(const ttt::BwdParams& p, hipStream_t stream);
 extern "C" int ttt_mlp_fwd_lds_bytes();
 extern "C" int ttt_mlp_bwd_lds_bytes();
