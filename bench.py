@@ -1,0 +1,163 @@
+#!/usr/bin/env python3
+"""Benchmark of the TTT-MLP forward + remat-backward hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c5|c3] [--no-cpu-baseline]
+
+A "step" is one forward + one remat backward over one batch of synthetic input that is already
+resident in HBM (zero-filling the four accumulating gradient outputs is part of the step, as the
+operator's contract makes the caller do it).  Prints ONE JSON line:
+  value      tokens/s for forward + backward, whole job
+  roofline   the dominant kernel (the backward) against the dense bf16 MFMA peak, its duration
+             measured with events on the launch stream inside the timed region
+  cpu_baseline  the fp32 PyTorch oracle of the same math on the host cores, on a bounded sample
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "ttt-tk_amd"))
+
+G_FLOP = 2 * 64 * 64 * 256                 # one 64x64x256 contraction
+FWD_G, BWD_G = 7, 21                        # contractions per mini-batch per (batch, head): forward; replay 7 + reverse 14
+PEAK_BF16_TFLOPS = 2516.6                   # MI355X dense bf16 MFMA: 256 CU x 4096 FLOP/clk x 2.4 GHz
+WORKLOADS = {
+    # name: (B, NH, NC, checkpoint_group_size, eta logit std, description)
+    "c3": (1, 48, 256, 16, 1.0, "fwd+bwd B=1 NH=48 16,384 tokens cgs=16"),
+    "c4": (1, 48, 4096, 64, 1.0, "fwd+bwd B=1 NH=48 262,144 tokens cgs=64 (the configuration the metric is quoted on)"),
+    "c5": (8, 48, 512, 32, 2.0, "fwd+bwd B=8 NH=48 32,768 tokens/sequence cgs=32 (fill-the-chip)"),
+}
+# HBM bytes per backward launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/), or None.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def make_device_inputs(B, NH, NC, eta_std, dev):
+    """Synthetic inputs of the operator's shapes and dtypes, generated on the device (seed 0)."""
+    import torch
+    g = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *s: torch.randn(*s, generator=g, device=dev, dtype=torch.float32)
+    t = {}
+    for name in ("XQ", "XK", "XV", "grad_L_XQW_mini_batch"):
+        t[name] = torch.empty(B, NH, NC, 64, 64, device=dev, dtype=torch.bfloat16)
+        for b in range(B):                      # generated per batch element to bound the fp32 temporary
+            t[name][b] = rn(NH, NC, 64, 64).to(torch.bfloat16)
+    t["W1"] = rn(B, NH, 64, 256) * 0.02
+    t["W2"] = rn(B, NH, 256, 64) * 0.02
+    t["b1"] = torch.zeros(B, NH, 1, 256, device=dev)
+    t["b2"] = torch.zeros(B, NH, 1, 64, device=dev)
+    t["ttt_norm_weight"] = torch.ones(1, NH, 1, 64, device=dev)
+    t["ttt_norm_bias"] = torch.zeros(1, NH, 1, 64, device=dev)
+    t["last_eta"] = (torch.sigmoid(rn(B, NH, NC, 64, 1) * eta_std) / 64).to(torch.bfloat16)
+    t["grad_L_W1_last"] = rn(B, NH, 64, 256) * 1e-3
+    t["grad_L_b1_last"] = rn(B, NH, 1, 256) * 1e-3
+    t["grad_L_W2_last"] = rn(B, NH, 256, 64) * 1e-3
+    t["grad_L_b2_last"] = rn(B, NH, 1, 64) * 1e-3
+    return t
+
+
+def cpu_baseline(NH, cgs, nc_sample):
+    """fp32 oracle forward + backward on the host cores over the first nc_sample mini-batches."""
+    import torch
+    from oracle import ttt_mlp_oracle as orc
+    threads = os.cpu_count() or 1
+    env = os.environ.get("OMP_NUM_THREADS")
+    if env and env.isdigit():
+        threads = min(threads, int(env))
+    torch.set_num_threads(threads)
+    d = orc.make_inputs(1, NH, nc_sample, seed=0)
+    keys = ("XQ", "XK", "XV", "last_eta", "ttt_norm_weight", "ttt_norm_bias", "W1", "b1", "W2", "b2")
+    t0 = time.perf_counter()
+    with torch.no_grad():
+        _, ck, _ = orc.ttt_forward(*[d[k] for k in keys], cgs)
+        orc.ttt_backward(d["XQ"], d["XK"], d["XV"], d["last_eta"], d["ttt_norm_weight"], d["ttt_norm_bias"], ck,
+                         orc.State(d["grad_L_W1_last"], d["grad_L_b1_last"], d["grad_L_W2_last"], d["grad_L_b2_last"]),
+                         d["grad_L_XQW_mini_batch"], cgs)
+    dt = time.perf_counter() - t0
+    return {"value": nc_sample * 64 / dt, "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": f"fp32 PyTorch oracle, forward + backward, B=1 NH={NH} first {nc_sample} mini-batches "
+                      f"({nc_sample * 64} tokens) cgs={cgs}, {dt:.1f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c4")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-mb", type=int, default=1536, help="mini-batches in the CPU baseline sample")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (every (batch, head) recurrence is independent and no "
+                 "collective is involved); --gpus must be 1")
+
+    import torch
+    import ttt_mlp_host as host          # fails loudly if the HIP extension is not built
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = torch.device("cuda:0")
+    B, NH, NC, cgs, eta_std, desc = WORKLOADS[a.workload]
+    t = make_device_inputs(B, NH, NC, eta_std, dev)
+    t.update(host.alloc_forward_buffers(B, NH, NC, cgs, dev))
+    t.update(host.alloc_backward_buffers(B, NH, NC, cgs, dev))
+    host.set_synchronize(False)           # time with events; the operator's default host sync is not part of the kernel
+
+    def step(ev=None):
+        host.zero_accumulating_grads(t)
+        if ev:
+            ev[0].record()
+        host.forward(t, cgs)
+        if ev:
+            ev[1].record()
+        host.backward(t, cgs)
+        if ev:
+            ev[2].record()
+
+    for _ in range(a.warmup):
+        step()
+    torch.cuda.synchronize()
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(a.steps)]
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        step(events[i])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    host.set_synchronize(True)
+    assert bool(torch.isfinite(t["grad_L_W1_init"]).all()) and bool(torch.isfinite(t["Out"].float()).all())
+
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in events) / a.steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in events) / a.steps
+    ms_per_step = wall * 1e3 / a.steps
+    tokens = B * NC * 64
+    value = tokens / (ms_per_step * 1e-3)
+    mb_steps = B * NH * NC
+    bwd_tflops = BWD_G * G_FLOP * mb_steps / (bwd_ms * 1e-3) / 1e12
+    fwd_tflops = FWD_G * G_FLOP * mb_steps / (fwd_ms * 1e-3) / 1e12
+    all_tflops = (FWD_G + BWD_G) * G_FLOP * mb_steps / (ms_per_step * 1e-3) / 1e12
+    out = {
+        "metric": "TTT-MLP fwd+bwd tokens/sec on 1 MI355X (B=1,NH=48,256K tok); % bf16 MFMA peak",
+        "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{a.workload}: {desc}", "B": B, "NH": NH, "NC": NC, "tokens": tokens,
+                   "checkpoint_group_size": cgs},
+        "fwd_ms": fwd_ms, "bwd_ms": bwd_ms, "fwd_tflops": fwd_tflops, "fwd_bwd_tflops": all_tflops,
+        "pct_of_bf16_mfma_peak": 100.0 * all_tflops / PEAK_BF16_TFLOPS,
+        "roofline": {"bound": "mfma", "kernel": "ttt_mlp_bwd_kernel", "achieved": bwd_tflops, "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": bwd_tflops / PEAK_BF16_TFLOPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload),
+                     "flop_per_launch": BWD_G * G_FLOP * mb_steps, "avg_launch_ms": bwd_ms},
+    }
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(NH, cgs, min(a.cpu_sample_mb, NC))
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,137 @@
+"""CPU-side checks of the drop-in boundary: the C ABI library loads and exports every symbol the
+header declares, argument validation behaves, and the Python operator module mirrors the reference
+interface (names, positional arity, error behaviour).  No kernel is launched here."""
+import ctypes
+import inspect
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG = os.path.join(ROOT, "ttt-tk_amd")
+LIB = os.path.join(PKG, "libttt_mlp.so")
+HEADER = os.path.join(ROOT, "include", "ttt_mlp.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(LIB):
+        import sys
+        sys.path.insert(0, ROOT)
+        import __graft_entry__ as ge
+        ge.build()
+    return ctypes.CDLL(LIB)
+
+
+def declared_functions():
+    src = open(HEADER).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return sorted(set(re.findall(r"\b(ttt_mlp_[a-z_]+)\s*\(", src)))
+
+
+def test_header_declares_the_expected_entry_points():
+    assert declared_functions() == ["ttt_mlp_abi_version", "ttt_mlp_bwd_launch", "ttt_mlp_error_string",
+                                    "ttt_mlp_fwd_launch", "ttt_mlp_kernel_info"]
+
+
+def test_library_exports_every_declared_symbol(lib):
+    for name in declared_functions():
+        assert hasattr(lib, name), name
+    assert lib.ttt_mlp_abi_version() == 1
+
+
+def test_kernel_info_reports_lds_within_one_cu(lib):
+    for which in (0, 1):
+        lds, thr = ctypes.c_int(), ctypes.c_int()
+        assert lib.ttt_mlp_kernel_info(which, ctypes.byref(lds), ctypes.byref(thr)) == 0
+        assert thr.value == 256 and 0 < lds.value <= 160 * 1024
+    assert lib.ttt_mlp_kernel_info(2, ctypes.byref(lds), ctypes.byref(thr)) != 0
+
+
+class FwdArgs(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_void_p) for n in
+                ("XQ", "XK", "XV", "last_eta", "ttt_norm_weight", "ttt_norm_bias", "W1", "b1", "W2", "b2",
+                 "W1_checkpoints", "b1_checkpoints", "W2_checkpoints", "b2_checkpoints", "Out")] + \
+               [(n, ctypes.c_int32) for n in ("checkpoint_group_size", "B", "NH", "NC", "K")]
+
+
+def test_forward_launch_rejects_bad_arguments_before_touching_the_gpu(lib):
+    lib.ttt_mlp_error_string.restype = ctypes.c_char_p
+    assert lib.ttt_mlp_fwd_launch(None, None) == 1001
+    a = FwdArgs()
+    assert lib.ttt_mlp_fwd_launch(ctypes.byref(a), None) == 1001          # null pointers
+    for f, _ in FwdArgs._fields_[:15]:
+        setattr(a, f, 0x1000)
+    a.B, a.NH, a.NC, a.K, a.checkpoint_group_size = 1, 2, 9, 2, 4
+    assert lib.ttt_mlp_fwd_launch(ctypes.byref(a), None) == 1002          # K must be ceil(9/4) = 3
+    assert b"ceil" in lib.ttt_mlp_error_string(1002)
+    a.K = 3
+    a.XK = 0x1008
+    assert lib.ttt_mlp_fwd_launch(ctypes.byref(a), None) == 1003          # misaligned
+    a.XK = 0x1000
+    a.NC = 0
+    assert lib.ttt_mlp_fwd_launch(ctypes.byref(a), None) == 1001
+    assert lib.ttt_mlp_bwd_launch(None, None) == 1001
+
+
+def test_struct_layout_matches_header_field_order():
+    src = open(HEADER).read()
+    body = src[src.index("typedef struct ttt_mlp_fwd_args"):src.index("} ttt_mlp_fwd_args;")]
+    names = re.findall(r"\b(?:const\s+)?(?:uint16_t|float)\s*\*\s*(\w+);", body)
+    assert names == [f for f, _ in FwdArgs._fields_[:15]]
+    body = src[src.index("typedef struct ttt_mlp_bwd_args"):src.index("} ttt_mlp_bwd_args;")]
+    names = re.findall(r"\b(?:const\s+)?(?:uint16_t|float)\s*\*\s*(\w+);", body)
+    import sys
+    sys.path.insert(0, PKG)
+    import ttt_mlp_host as host
+    assert tuple(names) == host.BWD_ORDER         # 42 tensors in the operator's positional order
+    assert len(host.FWD_ORDER) == 15 and len(host.BWD_ORDER) == 42
+
+
+def test_operator_module_mirrors_reference_interface(lib):
+    import sys
+    sys.path.insert(0, PKG)
+    import test_time_training as ttt
+    assert ttt.__doc__ == "Test Time Training Kernels"
+    assert ttt.ttt_forward.__doc__.strip().endswith("TTT Forward.")
+    assert ttt.ttt_backward.__doc__.strip().endswith("TTT Backward.")
+    sig = ttt.ttt_forward.__doc__.splitlines()[0]
+    assert sig.count("arg") == 16                  # 15 tensors + checkpoint_group_size, positional only
+    sig = ttt.ttt_backward.__doc__.splitlines()[0]
+    assert sig.count("arg") == 43
+
+
+def test_operator_raises_on_cpu_tensors_and_bad_shapes(lib):
+    import sys
+    sys.path.insert(0, PKG)
+    import ttt_mlp_host as host
+    B, NH, NC, cgs = 1, 2, 3, 2
+    from oracle import ttt_mlp_oracle as orc
+    d = orc.make_inputs(B, NH, NC, seed=0, with_grads=False)
+    t = dict(d)
+    t.update(host.alloc_forward_buffers(B, NH, NC, cgs, "cpu"))
+    with pytest.raises(RuntimeError, match="XQ"):
+        host.forward(t, cgs)                       # CPU tensors: no silent fallback
+    t["XQ"] = t["XQ"][..., :32]
+    with pytest.raises(RuntimeError, match="XQ"):
+        host.forward(t, cgs)
+    t = dict(d)
+    t.update(host.alloc_forward_buffers(B, NH, NC, 3, "cpu"))      # K = 1, but cgs = 2 needs 2
+    with pytest.raises(RuntimeError, match="checkpoints"):
+        host.forward(t, cgs)
+
+
+def test_host_allocator_shapes():
+    import sys
+    sys.path.insert(0, PKG)
+    import ttt_mlp_host as host
+    assert host.num_checkpoints(9, 4) == 3 and host.num_checkpoints(8, 4) == 2
+    f = host.alloc_forward_buffers(2, 3, 9, 4, "cpu")
+    assert f["W1_checkpoints"].shape == (2, 3, 3, 64, 256) and f["Out"].dtype == torch.bfloat16
+    b = host.alloc_backward_buffers(2, 3, 9, 4, "cpu")
+    assert b["Z1_group"].shape == (2, 3, 4, 64, 256) and b["std_ln_group"].shape == (2, 3, 4, 64, 1)
+    assert b["grad_L_ttt_norm_weight"].shape == (2, 3, 1, 64)      # per batch element
+    for k in ("grad_L_last_eta", "grad_L_XQ", "grad_L_XK", "grad_L_XV"):
+        assert b[k].abs().max() == 0

@@ -82,3 +82,30 @@ def test_backward_matches_oracle(B, NH, NC, cgs, seed, rand_affine):
     for name, r in ref.items():
         check(name, hw[name], r, failures)
     assert not failures, failures
+
+
+def test_matches_committed_golden_samples():
+    """The CPU-runnable reference configuration against tests/golden/c1_oracle_samples.json."""
+    import json
+    import os
+    here = os.path.dirname(os.path.abspath(__file__))
+    with open(os.path.join(here, "golden", "c1_oracle_samples.json")) as f:
+        doc = json.load(f)
+    cfg = doc["config"]
+    d = orc.make_inputs(cfg["B"], cfg["NH"], cfg["NC"], seed=cfg["seed"])
+    for k, v in d.items():
+        if abs(v.double().sum().item() - doc["inputs"][k]["sum"]) > 1e-6 * max(1.0, abs(doc["inputs"][k]["sum"])):
+            pytest.skip("random stream differs from the one the fixture was written with")
+    hw = run_fwd_bwd(d, cfg["checkpoint_group_size"])
+    failures = []
+    for name, ref in doc["outputs"].items():
+        if name not in hw:
+            continue                                   # final state is not an operator output
+        got = hw[name].flatten()[::cfg["stride"]]
+        want = torch.tensor(ref["samples"])
+        scale = ref["l2"] / max(1, torch.tensor(ref["shape"]).prod().item()) ** 0.5   # rms of the full tensor
+        err = (got - want).abs().max().item() / max(scale, 1e-30)
+        print(f"{name:24s} sample max err / rms = {err:.3e}", flush=True)
+        if not err <= 6e-2:                            # 2e-2 of max|ref| is about 6e-2 of the rms here
+            failures.append((name, err))
+    assert not failures, failures
