@@ -37,16 +37,26 @@ constexpr int SB_A = SB_E2 + SB_TILE;     // reverse: gZ2_bar, later dZ2
 constexpr int SB_P = SB_A + SB_TILE;      // 4 fp32 partial tiles
 constexpr int SB_PTILE = 64 * LDP * 4;
 constexpr int SB_BNC = SB_P + 4 * SB_PTILE;   // 4 wave-private bounce tiles
-constexpr int SB_B2 = SB_BNC + 4 * SB_TILE;   // b2 (replay) / gb2 (reverse), 64 floats
-constexpr int SB_ETA = SB_B2 + FD * 4;
+constexpr int SB_B1 = SB_BNC + 4 * SB_TILE;   // b1 during a replay, 256 floats
+constexpr int SB_B2 = SB_B1 + HID * 4;        // b2 during a replay, 64 floats
+constexpr int SB_GB1 = SB_B2 + FD * 4;        // running gradient wrt b1
+constexpr int SB_GB2 = SB_GB1 + HID * 4;      // running gradient wrt b2
+constexpr int SB_GAM = SB_GB2 + FD * 4;       // ttt_norm_weight of this head
+constexpr int SB_BET = SB_GAM + FD * 4;       // ttt_norm_bias of this head
+constexpr int SB_ETA = SB_BET + FD * 4;
 constexpr int SB_DETA = SB_ETA + CS * 4;      // [2][4 waves][64 tokens] partial dEta sums
 constexpr int SB_RED = SB_DETA + 2 * 4 * CS * 4;  // [4 waves][2][64] final norm-grad reduction
 constexpr int SM_BWD_BYTES = SB_RED + 4 * 2 * FD * 4;
 static_assert(SM_BWD_BYTES <= 160 * 1024, "LDS budget of one gfx950 CU exceeded");
 
-// All waves run the same straight-line code, so a workgroup barrier is a valid (if heavier than
-// needed) way to order a wave-private LDS store against the transposing read that follows it.
-#define WAVE_SYNC() __syncthreads()
+// Orders a wave-private LDS store against the transposing read that follows it.  LDS operations of
+// one wave execute in issue order, so only the compiler has to be kept from reordering them.
+#define WAVE_SYNC()                                        \
+  do {                                                     \
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); \
+    __builtin_amdgcn_wave_barrier();                       \
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront"); \
+  } while (0)
 
 // ------------------------------------------------------------------ register images in HBM
 // A 64x64 tile as 8 chunks of 8 bf16 per lane; chunk n of thread tid sits at (n*256 + tid)*16 bytes,
@@ -254,6 +264,64 @@ TTT_DEV void stage_tile(bf16* s_tile, const bf16* g_tile, int tid) {
   }
 }
 
+// C-init of a Q-orientation tile from an LDS vector indexed by accumulator row (64 floats).
+TTT_DEV void acc_init_rows_lds(Acc& a, const float* s_vec, int h) {
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(s_vec + 32 * rb + 8 * g + 4 * h);
+#pragma unroll
+      for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) a.b[rb][cb][4 * g + e] = v[e];
+    }
+}
+// s_vec[row] += sum over the contraction of operand `a` (lane = row index); the sum is formed on the
+// matrix cores, lanes with c == 0 fold it into the LDS vector.
+TTT_DEV void lds_rowsum_add(float* s_vec, const Opd& a, bf16x8 ones, int c, int h) {
+  f32x16 t[2];
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) t[rb][i] = 0.f;
+  rowsum_mma(t, a, ones);
+  if (c == 0) {
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        f32x4* q = reinterpret_cast<f32x4*>(s_vec + 32 * rb + 8 * g + 4 * h);
+        f32x4 v = *q;
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] += t[rb][4 * g + e];
+        *q = v;
+      }
+  }
+  // Other lanes of this wave read the vector next; without a fence the compiler may forward the
+  // values each lane saw before the update.
+  WAVE_SYNC();
+}
+TTT_DEV void ln_load_f32(float (&x)[4][4], const float* s_vec, int fq) {
+#pragma unroll
+  for (int r = 0; r < 4; r++) {
+    const f32x4 v = *reinterpret_cast<const f32x4*>(s_vec + 16 * r + 4 * fq);
+#pragma unroll
+    for (int e = 0; e < 4; e++) x[r][e] = v[e];
+  }
+}
+// Sum of the 4 shard partial tiles for this lane's 16 features.
+TTT_DEV void ln_gather0(float (&z)[4][4], const float* s_P, int tok, int fq) {
+#pragma unroll
+  for (int r = 0; r < 4; r++) {
+    f32x4 a = *reinterpret_cast<const f32x4*>(s_P + tok * LDP + 16 * r + 4 * fq);
+#pragma unroll
+    for (int v = 1; v < 4; v++) a += *reinterpret_cast<const f32x4*>(s_P + v * 64 * LDP + tok * LDP + 16 * r + 4 * fq);
+#pragma unroll
+    for (int e = 0; e < 4; e++) z[r][e] = a[e];
+  }
+}
+
 __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   bf16* s_xq = reinterpret_cast<bf16*>(smem + SB_XQ);
@@ -262,7 +330,12 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
   bf16* s_e2 = reinterpret_cast<bf16*>(smem + SB_E2);
   bf16* s_a = reinterpret_cast<bf16*>(smem + SB_A);
   float* s_P = reinterpret_cast<float*>(smem + SB_P);
-  float* s_b2 = reinterpret_cast<float*>(smem + SB_B2);
+  float* s_b1 = reinterpret_cast<float*>(smem + SB_B1);     // replay: b1
+  float* s_b2 = reinterpret_cast<float*>(smem + SB_B2);     // replay: b2
+  float* s_gb1 = reinterpret_cast<float*>(smem + SB_GB1);   // running gradient wrt b1
+  float* s_gb2 = reinterpret_cast<float*>(smem + SB_GB2);   // running gradient wrt b2
+  float* s_gam = reinterpret_cast<float*>(smem + SB_GAM);
+  float* s_bet = reinterpret_cast<float*>(smem + SB_BET);
   float* s_eta = reinterpret_cast<float*>(smem + SB_ETA);
   float* s_deta = reinterpret_cast<float*>(smem + SB_DETA);
   float* s_red = reinterpret_cast<float*>(smem + SB_RED);
@@ -272,16 +345,16 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
   const int bh = blockIdx.x, head = bh % p.NH;
   float* s_Pw = s_P + w * 64 * LDP;
   bf16* s_bnc = reinterpret_cast<bf16*>(smem + SB_BNC) + w * 64 * LDB;
+  float* s_b1w = s_b1 + 64 * w;
+  float* s_gb1w = s_gb1 + 64 * w;
   const int cgs = p.cgs;
 
-  float gam[4][4], bet[4][4];
-#pragma unroll
-  for (int r = 0; r < 4; r++)
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-      gam[r][e] = p.ttt_norm_weight[head * FD + 16 * r + 4 * fq + e];
-      bet[r][e] = p.ttt_norm_bias[head * FD + 16 * r + 4 * fq + e];
-    }
+  if (tid < FD) {
+    s_gam[tid] = p.ttt_norm_weight[head * FD + tid];
+    s_bet[tid] = p.ttt_norm_bias[head * FD + tid];
+    s_gb2[tid] = p.grad_L_b2_last[(size_t)bh * FD + tid];
+  }
+  s_gb1[tid] = p.grad_L_b1_last[(size_t)bh * HID + tid];
   float dgam[4][4], dbet[4][4];
 #pragma unroll
   for (int r = 0; r < 4; r++)
@@ -299,16 +372,11 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
   const size_t g_T = (size_t)bh * cgs * CS;             // [cgs][64] vectors
   float* park_W1 = p.W1_init_group + (size_t)bh * cgs * FD * HID;
   float* park_W2 = p.W2_init_group + (size_t)bh * cgs * HID * FD;
-  float* park_b1 = p.b1_init_group + (size_t)bh * cgs * HID;
-  float* park_b2 = p.b2_init_group + (size_t)bh * cgs * FD;
 
   // running gradients wrt the state after the last mini-batch
   Acc gW1s, gW2s;
-  f32x16 gb1[2], gb2[2];
   acc_load_rows(gW1s, p.grad_L_W1_last + (size_t)bh * FD * HID, HID, 0, 64 * w, c, h);
   acc_load_rows(gW2s, p.grad_L_W2_last + (size_t)bh * HID * FD, FD, 64 * w, 0, c, h);
-  rowvec_load(gb1, p.grad_L_b1_last + (size_t)bh * HID + 64 * w, h);
-  rowvec_load(gb2, p.grad_L_b2_last + (size_t)bh * FD, h);
 
   for (int k = p.K - 1; k >= 0; k--) {
     const int n_mb = min(cgs, p.NC - k * cgs);
@@ -316,22 +384,16 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
     Acc W1t;
     // ================================================================= replay
     {
-      // park the running gradients
+      // park the running gradients while the forward state needs the registers
       acc_store_rows(gW1s, park_W1, HID, 0, 64 * w, c, h);
       acc_store_rows(gW2s, park_W2, FD, 64 * w, 0, c, h);
-      if (c == 0) {
-        rowvec_store(gb1, park_b1 + 64 * w, h);
-        if (w == 0) rowvec_store(gb2, park_b2, h);
-      }
       Acc W1s, W2s;
-      f32x16 b1[2], b2[2];
       const size_t slot = (size_t)bh * p.K + k;
       acc_load_rows(W1s, p.W1_ck + slot * FD * HID, HID, 0, 64 * w, c, h);
       acc_load_rows(W2s, p.W2_ck + slot * HID * FD, FD, 64 * w, 0, c, h);
       acc_load_cols(W2t, p.W2_ck + slot * HID * FD, FD, 64 * w, 0, c, h);
-      rowvec_load(b1, p.b1_ck + slot * HID + 64 * w, h);
-      rowvec_load(b2, p.b2_ck + slot * FD, h);
-      __syncthreads();  // previous group's readers of s_b2 are done
+      __syncthreads();  // previous group's readers of the bias vectors are done
+      s_b1[tid] = p.b1_ck[slot * HID + tid];
       if (tid < FD) s_b2[tid] = p.b2_ck[slot * FD + tid];
 
       for (int j = 0; j < n_mb; j++) {
@@ -345,12 +407,16 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
         __syncthreads();
 
         // Z1^T = W1s^T XK^T + b1  (rows hid, lane = tok)
-        Acc x2, d1;
+        Acc d1;
+        Opd x2Q;  // lane = tok, contraction = hid
         {
-          const Opd w1A = cvt_chain(W1s);
-          const Opd xkB = lds_rows_kappa(s_xk, c, h);
-          acc_init_rowvec(x2, b1);
-          mma(x2, w1A, xkB);
+          Acc x2;
+          acc_init_rows_lds(x2, s_b1w, h);
+          {
+            const Opd w1A = cvt_chain(W1s);
+            const Opd xkB = lds_rows_kappa(s_xk, c, h);
+            mma(x2, w1A, xkB);
+          }
           img_store(p.Z1_group + g_TH + (size_t)j * (CS * HID), x2, tid);
 #pragma unroll
           for (int rb = 0; rb < 2; rb++)
@@ -363,8 +429,8 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
                 x2.b[rb][cb][i] = g;
                 d1.b[rb][cb][i] = d;
               }
+          x2Q = cvt_chain(x2);
         }
-        const Opd x2Q = cvt_chain(x2);  // lane = tok, contraction = hid
         opd_store(p.X2_group + g_TH + (size_t)j * (CS * HID), x2Q, tid);
         {
           const Opd w2A = cvt_chain(W2s);
@@ -376,72 +442,87 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
         __syncthreads();
         // fused LayerNorm + reconstruction-loss gradient; saves for the reverse walk
         {
-          float z[4][4], kv[4][4], vv[4][4];
+          float z[4][4], gam[4][4];
           ln_gather(z, s_P, s_b2, tok, fq);
+          ln_load_f32(gam, s_gam, fq);
           float sd;
           const float rstd = ln_normalize(z, &sd);
-          ln_load(kv, s_xk + tok * LDB, fq);
-          ln_load(vv, s_e2 + tok * LDB, fq);
           float go[4][4], gx[4][4];
+          {
+            float kv[4][4], vv[4][4], bet[4][4];
+            ln_load(kv, s_xk + tok * LDB, fq);
+            ln_load(vv, s_e2 + tok * LDB, fq);
+            ln_load_f32(bet, s_bet, fq);
 #pragma unroll
-          for (int r = 0; r < 4; r++)
+            for (int r = 0; r < 4; r++)
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-              go[r][e] = __builtin_fmaf(gam[r][e], z[r][e], bet[r][e]) - (vv[r][e] - kv[r][e]);
-              gx[r][e] = go[r][e] * gam[r][e];
-            }
-          const float s1 = quad_sum(sum16(gx)), s2 = quad_sum(dot16(gx, z));
-          const float sc = rstd * (1.f / FD), neg_eta = -s_eta[tok];
-          float gz[4][4], g2[4][4];
-#pragma unroll
-          for (int r = 0; r < 4; r++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-              gz[r][e] = (FD * gx[r][e] - s1 - z[r][e] * s2) * sc;
-              g2[r][e] = neg_eta * gz[r][e];
-            }
-          ln_store(s_gz2 + tok * LDB, g2, fq);
+              for (int e = 0; e < 4; e++) {
+                go[r][e] = __builtin_fmaf(gam[r][e], z[r][e], bet[r][e]) - (vv[r][e] - kv[r][e]);
+                gx[r][e] = go[r][e] * gam[r][e];
+              }
+          }
           const size_t so = g_TF + (size_t)j * (CS * FD) + tok * FD;
           ln_store(p.x_hat_fused_group + so, z, fq);
           ln_store(p.grad_output_fused_group + so, go, fq);
-          ln_store(p.grad_l_wrt_Z2_group + so, gz, fq);
-          ln_store(p.grad_x_hat_fused_group + so, g2, fq);   // the exact bf16 operand of the weight step
+          const float s1 = quad_sum(sum16(gx)), s2 = quad_sum(dot16(gx, z));
+          const float sc = rstd * (1.f / FD), neg_eta = -s_eta[tok];
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) gx[r][e] = (FD * gx[r][e] - s1 - z[r][e] * s2) * sc;   // dl/dZ2
+          ln_store(p.grad_l_wrt_Z2_group + so, gx, fq);
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) gx[r][e] *= neg_eta;                                   // G2
+          ln_store(s_gz2 + tok * LDB, gx, fq);
+          ln_store(p.grad_x_hat_fused_group + so, gx, fq);   // the exact bf16 operand of the weight step
           if (fq == 0) p.std_fused_group[g_T + (size_t)j * CS + tok] = sd;
         }
         __syncthreads();
-        // G1^T = (W2t^T... rows hid, lane = tok) * gelu'(Z1); weight step
+        // G1 = (W2 G2^T) * gelu'(Z1)  (rows hid, lane = tok); weight step
         {
-          const Opd g2B = lds_rows_kappa(s_gz2, c, h);   // lane = tok, contraction = F
-          const Opd w2tA = cvt_chain(W2t);               // lane = hid, contraction = F
-          Acc g1;
-          acc_zero(g1);
-          mma(g1, w2tA, g2B);
+          Opd g1Q;
+          {
+            Acc g1;
+            acc_zero(g1);
+            {
+              const Opd g2B = lds_rows_kappa(s_gz2, c, h);   // lane = tok, contraction = F
+              const Opd w2tA = cvt_chain(W2t);               // lane = hid, contraction = F
+              mma(g1, w2tA, g2B);
+            }
 #pragma unroll
-          for (int rb = 0; rb < 2; rb++)
+            for (int rb = 0; rb < 2; rb++)
 #pragma unroll
-            for (int cb = 0; cb < 2; cb++)
+              for (int cb = 0; cb < 2; cb++)
 #pragma unroll
-              for (int i = 0; i < 16; i++) g1.b[rb][cb][i] *= d1.b[rb][cb][i];
-          const Opd g1Q = cvt_chain(g1);
+                for (int i = 0; i < 16; i++) g1.b[rb][cb][i] *= d1.b[rb][cb][i];
+            g1Q = cvt_chain(g1);
+          }
           opd_store(p.grad_l_wrt_Z1_group + g_TH + (size_t)j * (CS * HID), g1Q, tid);
-          const Opd x2P = bounce(s_bnc, x2Q, lane);      // lane = hid, contraction = tok
-          const Opd g1P = bounce(s_bnc, g1Q, lane);
-          const Opd g2T = lds_tr_kappa(s_gz2, lane);     // lane = F, contraction = tok
-          mma(W2s, x2P, g2T);
-          mma(W2t, g2T, x2P);
-          rowsum_mma(b2, g2T, ones);
-          const Opd xkT = lds_tr_kappa(s_xk, lane);      // lane = F, contraction = tok
-          mma(W1s, xkT, g1P);
-          rowsum_mma(b1, g1P, ones);
+          {
+            const Opd g2T = lds_tr_kappa(s_gz2, lane);       // lane = F, contraction = tok
+            const Opd x2P = bounce(s_bnc, x2Q, lane);        // lane = hid, contraction = tok
+            mma(W2s, x2P, g2T);
+            mma(W2t, g2T, x2P);
+            if (w == 0) lds_rowsum_add(s_b2, g2T, ones, c, h);
+          }
+          {
+            const Opd g1P = bounce(s_bnc, g1Q, lane);
+            const Opd xkT = lds_tr_kappa(s_xk, lane);        // lane = F, contraction = tok
+            mma(W1s, xkT, g1P);
+            lds_rowsum_add(s_b1w, g1P, ones, c, h);
+          }
         }
-        if (w == 0 && c == 0) rowvec_store_lds(b2, s_b2, h);
         // post-update forward on XQ
         {
-          const Opd w1A = cvt_chain(W1s);
-          const Opd xqB = lds_rows_kappa(s_xq, c, h);
           Acc z1b;
-          acc_init_rowvec(z1b, b1);
-          mma(z1b, w1A, xqB);
+          acc_init_rows_lds(z1b, s_b1w, h);
+          {
+            const Opd w1A = cvt_chain(W1s);
+            const Opd xqB = lds_rows_kappa(s_xq, c, h);
+            mma(z1b, w1A, xqB);
+          }
           img_store(p.Z1_bar_group + g_TH + (size_t)j * (CS * HID), z1b, tid);
 #pragma unroll
           for (int rb = 0; rb < 2; rb++)
@@ -480,8 +561,6 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
       // running gradients back into registers
       acc_load_rows(gW1s, park_W1, HID, 0, 64 * w, c, h);
       acc_load_rows(gW2s, park_W2, FD, 64 * w, 0, c, h);
-      rowvec_load(gb1, park_b1 + 64 * w, h);
-      rowvec_load(gb2, park_b2, h);
     }
 
     // ================================================================= reverse walk
@@ -489,9 +568,10 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
       const int mb = k * cgs + j;
       const size_t xo = x_base + (size_t)mb * (CS * FD);
       const size_t so = g_TF + (size_t)j * (CS * FD);
-      const float eta_l = bf2f(p.last_eta[eta_base + (size_t)mb * CS + 32 * 0 + c]);      // token c
-      const float eta_h = bf2f(p.last_eta[eta_base + (size_t)mb * CS + 32 * 1 + c]);      // token 32 + c
-      const float eta_cb[2] = {eta_l, eta_h};  // eta of the token this lane holds in column block cb
+      const size_t ho = g_TH + (size_t)j * (CS * HID);
+      // eta of the token this lane holds in column block cb of a Q-orientation tile
+      const float eta_cb[2] = {bf2f(p.last_eta[eta_base + (size_t)mb * CS + c]),
+                               bf2f(p.last_eta[eta_base + (size_t)mb * CS + 32 + c])};
       __syncthreads();
       stage_tile(s_xq, p.XQ + xo, tid);
       stage_tile(s_xk, p.XK + xo, tid);
@@ -500,11 +580,11 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
       if (tid < CS) s_eta[tid] = bf2f(p.last_eta[eta_base + (size_t)mb * CS + tid]);
 
       // ---- output LayerNorm backward (LayerNorm lanes)
-      float gO[4][4];
-      ln_load(gO, p.grad_L_XQW + xo + tok * FD, fq);
       {
-        float xh[4][4], gx[4][4];
+        float gO[4][4], xh[4][4], gx[4][4], gam[4][4];
+        ln_load(gO, p.grad_L_XQW + xo + tok * FD, fq);
         ln_load(xh, p.x_hat_ln_group + so + tok * FD, fq);
+        ln_load_f32(gam, s_gam, fq);
         const float sd = p.std_ln_group[g_T + (size_t)j * CS + tok];
 #pragma unroll
         for (int r = 0; r < 4; r++)
@@ -516,298 +596,322 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
           }
         const float s1 = quad_sum(sum16(gx)), s2 = quad_sum(dot16(gx, xh));
         const float sc = 1.f / (FD * sd);
-        float gz[4][4];
 #pragma unroll
         for (int r = 0; r < 4; r++)
 #pragma unroll
-          for (int e = 0; e < 4; e++) gz[r][e] = (FD * gx[r][e] - s1 - xh[r][e] * s2) * sc;
-        ln_store(s_a + tok * LDB, gz, fq);  // gZ2_bar
+          for (int e = 0; e < 4; e++) gx[r][e] = (FD * gx[r][e] - s1 - xh[r][e] * s2) * sc;
+        ln_store(s_a + tok * LDB, gx, fq);  // gZ2_bar
       }
       __syncthreads();
 
       // ---- post-update forward, backwards (uses the state AFTER this mini-batch)
-      Opd gw1T, gw2T;  // running gradients with lane/contraction swapped, taken after their first update
       {
-        Acc z1b;
-        img_load(p.Z1_bar_group + g_TH + (size_t)j * (CS * HID), z1b, tid);
-        Acc d1b;
-#pragma unroll
-        for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-          for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-              float g, d;
-              gelu_fd(z1b.b[rb][cb][i], g, d);
-              z1b.b[rb][cb][i] = g;   // X2_bar
-              d1b.b[rb][cb][i] = d;
-            }
-        const Opd x2bQ = cvt_chain(z1b);
-        const Opd gz2bB = lds_rows_kappa(s_a, c, h);     // lane = tok, contraction = F
-        const Opd w2tA = cvt_chain(W2t);                 // lane = hid, contraction = F   (W2 after the step)
-        Acc gz1b;
-        acc_zero(gz1b);
-        mma(gz1b, w2tA, gz2bB);                          // rows hid, lane = tok
-#pragma unroll
-        for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-          for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) gz1b.b[rb][cb][i] *= d1b.b[rb][cb][i];
-        const Opd gz1bQ = cvt_chain(gz1b);               // lane = tok, contraction = hid
+        Opd x2bQ, gz1bQ;  // lane = tok, contraction = hid
         {
-          const Opd w1tA = cvt_chain(W1t);               // lane = F, contraction = hid   (W1 after the step)
+          Acc gz1b;
+          acc_zero(gz1b);
+          {
+            const Opd gz2bB = lds_rows_kappa(s_a, c, h);   // lane = tok, contraction = F
+            const Opd w2tA = cvt_chain(W2t);               // lane = hid, contraction = F   (W2 after the step)
+            mma(gz1b, w2tA, gz2bB);                        // rows hid, lane = tok
+          }
+          const Opd zimg = opd_load(p.Z1_bar_group + ho, tid);
+#pragma unroll
+          for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+#pragma unroll
+              for (int jj = 0; jj < 8; jj++) {
+                float g, d;
+                gelu_fd((float)zimg.v[cb][s][jj], g, d);
+                gz1b.b[s >> 1][cb][8 * (s & 1) + jj] *= d;
+                x2bQ.v[cb][s][jj] = (bf16)g;
+              }
+          gz1bQ = cvt_chain(gz1b);
+        }
+        {
+          const Opd w1tA = cvt_chain(W1t);                 // lane = F, contraction = hid   (W1 after the step)
           Acc dq;
           acc_zero(dq);
-          mma(dq, w1tA, gz1bQ);                          // rows F, lane = tok
+          mma(dq, w1tA, gz1bQ);                            // rows F, lane = tok
           lds_store_partial(s_Pw, dq, c, h);
         }
-        const Opd x2bP = bounce(s_bnc, x2bQ, lane);      // lane = hid, contraction = tok
-        const Opd gz1bP = bounce(s_bnc, gz1bQ, lane);
-        const Opd gz2bT = lds_tr_kappa(s_a, lane);       // lane = F, contraction = tok
-        mma(gW2s, x2bP, gz2bT);
-        rowsum_mma(gb2, gz2bT, ones);
-        const Opd xqT = lds_tr_kappa(s_xq, lane);
-        mma(gW1s, xqT, gz1bP);
-        rowsum_mma(gb1, gz1bP, ones);
-        gw1T = bounce(s_bnc, cvt_chain(gW1s), lane);     // lane = F,   contraction = hid
-        gw2T = bounce(s_bnc, cvt_chain(gW2s), lane);     // lane = hid, contraction = F
-      }
-      __syncthreads();  // partial dXQ tiles complete; gZ2_bar tile no longer needed
-      if (w == 0 && c == 0) rowvec_store_lds(gb2, s_b2, h);  // gb2 after adding sum_t gZ2_bar
-      {
-        float z[4][4];
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-          f32x4 a = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int v = 0; v < 4; v++) a += *reinterpret_cast<const f32x4*>(s_P + v * 64 * LDP + tok * LDP + 16 * r + 4 * fq);
-#pragma unroll
-          for (int e = 0; e < 4; e++) z[r][e] = a[e] + gO[r][e];
+        {
+          const Opd gz2bT = lds_tr_kappa(s_a, lane);       // lane = F, contraction = tok
+          {
+            const Opd x2bP = bounce(s_bnc, x2bQ, lane);    // lane = hid, contraction = tok
+            mma(gW2s, x2bP, gz2bT);
+          }
+          if (w == 0) lds_rowsum_add(s_gb2, gz2bT, ones, c, h);
         }
+        {
+          const Opd gz1bP = bounce(s_bnc, gz1bQ, lane);
+          const Opd xqT = lds_tr_kappa(s_xq, lane);
+          mma(gW1s, xqT, gz1bP);
+          lds_rowsum_add(s_gb1w, gz1bP, ones, c, h);
+        }
+      }
+      __syncthreads();  // partial dXQ tiles complete; gb2 holds its value after the first update
+      {
+        float z[4][4], gO[4][4];
+        ln_gather0(z, s_P, tok, fq);
+        ln_load(gO, p.grad_L_XQW + xo + tok * FD, fq);
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) z[r][e] += gO[r][e];
         ln_accumulate(p.grad_L_XQ + xo + tok * FD, z, fq);
       }
 
-      // ---- the weight step, backwards
-      Acc d1, d2, S, R;
-      Opd x2P;
+      // ---- the weight step, backwards.  Two packed tiles survive the LayerNorm stage:
+      //      d1p = gelu'(Z1) and t2p = -eta * (gZ2 W2^T) * (XK gW1 + gb1) * gelu''(Z1).
+      Opd d1p, t2p;
       {
+        const Opd x2Q = opd_load(p.X2_group + ho, tid);      // X2 exactly as the replay fed it to the weight step
         {
-          Acc z1;
-          img_load(p.Z1_group + g_TH + (size_t)j * (CS * HID), z1, tid);
-#pragma unroll
-          for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-            for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-              for (int i = 0; i < 16; i++) {
-                float g, a, b;
-                gelu_fdd(z1.b[rb][cb][i], g, a, b);
-                d1.b[rb][cb][i] = a;
-                d2.b[rb][cb][i] = b;
-              }
-        }
-        // X2 exactly as the replay fed it to the weight step
-        const Opd x2Q = opd_load(p.X2_group + g_TH + (size_t)j * (CS * HID), tid);   // lane = tok, contraction = hid
-        x2P = bounce(s_bnc, x2Q, lane);                  // lane = hid, contraction = tok
-        // undo the W2 step with the very operands that made it: W2 before = W2 after - X2^T G2
-        {
+          // undo the W2 step with the very operands that made it: W2 before = W2 after - X2^T G2
+          const Opd x2P = bounce(s_bnc, x2Q, lane);          // lane = hid, contraction = tok
           const Opd g2Tn = opd_neg(lds_tr_kappa(s_e2, lane));   // lane = F, contraction = tok
           mma(W2t, g2Tn, x2P);
         }
-        const Opd w2tA = cvt_chain(W2t);                 // W2 before the step: lane = hid, contraction = F
-        const Opd gz2B = lds_rows_kappa(s_gz2, c, h);    // lane = tok, contraction = F
-        acc_zero(R);
-        mma(R, w2tA, gz2B);                              // R = gZ2 W2^T  (rows hid, lane = tok)
-        // S = XK gW1 + gb1
+        Opd uQ;   // (XK gW1 + gb1) * gelu'(Z1), lane = tok
+        float de3[2] = {0.f, 0.f};
         {
-          const Opd gw1A = cvt_chain(gW1s);              // lane = hid, contraction = F
+          const Opd w2tA = cvt_chain(W2t);                   // W2 before the step: lane = hid, contraction = F
+          const Opd gz2B = lds_rows_kappa(s_gz2, c, h);      // lane = tok, contraction = F
+          const Opd gw1A = cvt_chain(gW1s);                  // lane = hid, contraction = F
           const Opd xkB = lds_rows_kappa(s_xk, c, h);
-          acc_init_rowvec(S, gb1);
-          mma(S, gw1A, xkB);
-        }
-        // partial ggZ2 / (-eta): gW2^T X2^T + W2^T (S*d1)^T, and the first dEta partial sum
-        Acc pz;
-        acc_zero(pz);
-        {
-          const Opd gw2A = cvt_chain(gW2s);              // lane = F, contraction = hid
-          mma(pz, gw2A, x2Q);                            // rows F, lane = tok
-        }
-        float de1[2] = {0.f, 0.f}, de3[2] = {0.f, 0.f};
+          const Opd zimg = opd_load(p.Z1_group + ho, tid);
 #pragma unroll
-        for (int rb = 0; rb < 2; rb++)
+          for (int cb = 0; cb < 2; cb++) {
+            f32x16 R[2], S[2];   // R = gZ2 W2^T, S = XK gW1 + gb1 for tokens 32cb..32cb+31
 #pragma unroll
-          for (int cb = 0; cb < 2; cb++)
+            for (int rb = 0; rb < 2; rb++)
 #pragma unroll
-            for (int t = 0; t < 2; t++)
+              for (int g = 0; g < 4; g++) {
+                const f32x4 v = *reinterpret_cast<const f32x4*>(s_gb1w + 32 * rb + 8 * g + 4 * h);
 #pragma unroll
-              for (int jj = 0; jj < 8; jj++)
-                de1[cb] = __builtin_fmaf((float)gz2B.v[cb][2 * rb + t][jj], pz.b[rb][cb][8 * t + jj], de1[cb]);
-        Acc u;
+                for (int e = 0; e < 4; e++) { S[rb][4 * g + e] = v[e]; R[rb][4 * g + e] = 0.f; }
+              }
 #pragma unroll
-        for (int rb = 0; rb < 2; rb++)
+            for (int s = 0; s < 4; s++)
 #pragma unroll
-          for (int cb = 0; cb < 2; cb++)
+              for (int rb = 0; rb < 2; rb++) {
+                R[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w2tA.v[rb][s], gz2B.v[cb][s], R[rb], 0, 0, 0);
+                S[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gw1A.v[rb][s], xkB.v[cb][s], S[rb], 0, 0, 0);
+              }
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-              const float gz1 = R.b[rb][cb][i] * d1.b[rb][cb][i];        // dl/dZ1 (no eta)
-              de3[cb] = __builtin_fmaf(gz1, S.b[rb][cb][i], de3[cb]);
-              u.b[rb][cb][i] = S.b[rb][cb][i] * d1.b[rb][cb][i];
-            }
-        const Opd uQ = cvt_chain(u);
-        {
-          const Opd w2sA = bounce(s_bnc, w2tA, lane);    // W2 before the step: lane = F, contraction = hid
-          mma(pz, w2sA, uQ);
-        }
-        __syncthreads();  // dXQ readers of the partial tiles are done
-        lds_store_partial(s_Pw, pz, c, h);
+            for (int s = 0; s < 4; s++)
 #pragma unroll
-        for (int cb = 0; cb < 2; cb++) {
-          const float a = half_sum(de1[cb]), b = half_sum(de3[cb]);
-          if (h == 0) {
-            s_deta[(0 * 4 + w) * CS + 32 * cb + c] = a;
-            s_deta[(1 * 4 + w) * CS + 32 * cb + c] = b;
+              for (int jj = 0; jj < 8; jj++) {
+                float g, a, b;
+                gelu_fdd((float)zimg.v[cb][s][jj], g, a, b);
+                const float r0 = R[s >> 1][8 * (s & 1) + jj], sv = S[s >> 1][8 * (s & 1) + jj];
+                de3[cb] = __builtin_fmaf(r0 * a, sv, de3[cb]);          // dl/dZ1 * S
+                uQ.v[cb][s][jj] = (bf16)(sv * a);
+                d1p.v[cb][s][jj] = (bf16)a;
+                t2p.v[cb][s][jj] = (bf16)(-eta_cb[cb] * r0 * sv * b);
+              }
           }
         }
-        // undo the W1 step with the saved operand G1 = -eta * dl/dZ1: W1 before = W1 after - XK^T G1
-        const Opd g1Q = opd_load(p.grad_l_wrt_Z1_group + g_TH + (size_t)j * (CS * HID), tid);  // lane = tok
+        // partial ggZ2 / (-eta): gW2^T X2^T + W2^T uQ^T, and the first dEta partial sum
         {
-          const Opd g1Pn = opd_neg(bounce(s_bnc, g1Q, lane));   // lane = hid, contraction = tok
-          const Opd xkT = lds_tr_kappa(s_xk, lane);             // lane = F,   contraction = tok
-          mma(W1t, g1Pn, xkT);
-        }
-        // u <- -eta * S * d1  (the gradient wrt dl/dZ1 times gelu')
-#pragma unroll
-        for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-          for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) u.b[rb][cb][i] *= -eta_cb[cb];
-        const Opd uP = bounce(s_bnc, cvt_chain(u), lane);       // lane = hid, contraction = tok
-        const Opd gz2T = lds_tr_kappa(s_gz2, lane);             // lane = F,   contraction = tok
-        __syncthreads();  // all partial ggZ2 tiles and dEta partial sums are in LDS
-        // (gW2s += u^T gZ2 is applied below, after the old gW2 has served its last product)
-
-        // ---- second-order pass through the fused LayerNorm loss (LayerNorm lanes)
-        float gy[4][4];
-        {
-          float gg[4][4], xh[4][4], go[4][4], gz[4][4];
-          ln_gather(gg, s_P, s_b2, tok, fq);
-          const float neg_eta = -s_eta[tok];
-#pragma unroll
-          for (int r = 0; r < 4; r++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) gg[r][e] *= neg_eta;                 // grad wrt dl/dZ2
-          ln_load(xh, p.x_hat_fused_group + so + tok * FD, fq);
-          ln_load(go, p.grad_output_fused_group + so + tok * FD, fq);
-          ln_load(gz, s_gz2 + tok * LDB, fq);
-          const float sd = p.std_fused_group[g_T + (size_t)j * CS + tok];
-          const float rsd = 1.f / sd;
-          // dEta: -(sum_F gZ2*(X2 gW2 + gb2) + sum_H gZ1*(XK gW1 + gb1))
+          Acc pz;
+          acc_zero(pz);
           {
-            float bias_dot = 0.f;
+            const Opd gw2A = cvt_chain(gW2s);                // lane = F, contraction = hid
+            mma(pz, gw2A, x2Q);                              // rows F, lane = tok
+          }
+          float de1[2] = {0.f, 0.f};
+          {
+            const Opd gz2B = lds_rows_kappa(s_gz2, c, h);
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-              const f32x4 bv = *reinterpret_cast<const f32x4*>(s_b2 + 16 * r + 4 * fq);
+            for (int rb = 0; rb < 2; rb++)
 #pragma unroll
-              for (int e = 0; e < 4; e++) bias_dot = __builtin_fmaf(gz[r][e], bv[e], bias_dot);
-            }
-            bias_dot = quad_sum(bias_dot);
-            float tot = bias_dot;
+              for (int cb = 0; cb < 2; cb++)
 #pragma unroll
-            for (int v = 0; v < 8; v++) tot += s_deta[v * CS + tok];
-            if (fq == 0) {
-              bf16* dst = p.grad_L_last_eta + eta_base + (size_t)mb * CS + tok;
-              *dst = (bf16)((float)*dst - tot);
+                for (int t = 0; t < 2; t++)
+#pragma unroll
+                  for (int jj = 0; jj < 8; jj++)
+                    de1[cb] = __builtin_fmaf((float)gz2B.v[cb][2 * rb + t][jj], pz.b[rb][cb][8 * t + jj], de1[cb]);
+          }
+          {
+            const Opd w2sA = bounce(s_bnc, cvt_chain(W2t), lane);   // W2 before the step: lane = F, contraction = hid
+            mma(pz, w2sA, uQ);
+          }
+          __syncthreads();  // dXQ readers of the partial tiles are done
+          lds_store_partial(s_Pw, pz, c, h);
+#pragma unroll
+          for (int cb = 0; cb < 2; cb++) {
+            const float a = half_sum(de1[cb]), b = half_sum(de3[cb]);
+            if (h == 0) {
+              s_deta[(0 * 4 + w) * CS + 32 * cb + c] = a;
+              s_deta[(1 * 4 + w) * CS + 32 * cb + c] = b;
             }
           }
-          float gxh[4][4];
-#pragma unroll
-          for (int r = 0; r < 4; r++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) gxh[r][e] = go[r][e] * gam[r][e];
-          const float s0 = quad_sum(sum16(gg)), a = quad_sum(dot16(gg, xh)), bb = quad_sum(dot16(gxh, xh));
-          float gx[4][4], gstd[4][4];
-          const float inv = rsd * (1.f / FD);
-#pragma unroll
-          for (int r = 0; r < 4; r++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-              const float ggx = (gg[r][e] - (s0 + xh[r][e] * a) * (1.f / FD)) * rsd;
-              gy[r][e] = gam[r][e] * ggx;
-              dgam[r][e] += go[r][e] * ggx + gy[r][e] * xh[r][e];
-              dbet[r][e] += gy[r][e];
-              gx[r][e] = gy[r][e] * gam[r][e] - (gxh[r][e] * a + gg[r][e] * bb) * inv;
-              gstd[r][e] = (-gx[r][e] * xh[r][e] - gg[r][e] * gz[r][e]) * rsd;
-            }
-          const float sg = quad_sum(sum16(gstd)), sx = quad_sum(sum16(gx));
-          float dz2[4][4], dxv[4][4];
-#pragma unroll
-          for (int r = 0; r < 4; r++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-              dz2[r][e] = gx[r][e] * rsd + (sg * xh[r][e] - sx * rsd) * (1.f / FD);
-              dxv[r][e] = -gy[r][e];
-            }
-          ln_store(s_a + tok * LDB, dz2, fq);
-          ln_accumulate(p.grad_L_XV + xo + tok * FD, dxv, fq);
         }
-        __syncthreads();  // dZ2 tile complete; partial tiles free again
+        // park -eta * uQ in the bounce tile; it is read back transposed after the LayerNorm stage
+        {
+          Opd uh;
+#pragma unroll
+          for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+#pragma unroll
+              for (int jj = 0; jj < 8; jj++) uh.v[cb][s][jj] = (bf16)(-eta_cb[cb] * (float)uQ.v[cb][s][jj]);
+          WAVE_SYNC();
+          lds_store_rows_kappa(s_bnc, uh, c, h);
+        }
+      }
+      __syncthreads();  // all partial ggZ2 tiles and dEta partial sums are in LDS
 
-        // ---- inner MLP, backwards (uses the state BEFORE this mini-batch)
+      // ---- second-order pass through the fused LayerNorm loss (LayerNorm lanes)
+      float gy[4][4];
+      {
+        float gg[4][4], xh[4][4], go[4][4], gz[4][4], gam[4][4];
+        ln_gather(gg, s_P, s_gb2, tok, fq);
+        const float neg_eta = -s_eta[tok];
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) gg[r][e] *= neg_eta;                 // grad wrt dl/dZ2
+        ln_load(xh, p.x_hat_fused_group + so + tok * FD, fq);
+        ln_load(go, p.grad_output_fused_group + so + tok * FD, fq);
+        ln_load(gz, s_gz2 + tok * LDB, fq);
+        ln_load_f32(gam, s_gam, fq);
+        const float sd = p.std_fused_group[g_T + (size_t)j * CS + tok];
+        const float rsd = 1.f / sd;
+        // dEta: -(sum_F gZ2*(X2 gW2 + gb2) + sum_H gZ1*(XK gW1 + gb1))
+        {
+          float gb[4][4];
+          ln_load_f32(gb, s_gb2, fq);
+          float tot = quad_sum(dot16(gz, gb));
+#pragma unroll
+          for (int v = 0; v < 8; v++) tot += s_deta[v * CS + tok];
+          if (fq == 0) {
+            bf16* dst = p.grad_L_last_eta + eta_base + (size_t)mb * CS + tok;
+            *dst = (bf16)((float)*dst - tot);
+          }
+        }
+        const float s0 = quad_sum(sum16(gg)), a = quad_sum(dot16(gg, xh));
+        float bb = 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) bb = __builtin_fmaf(go[r][e] * gam[r][e], xh[r][e], bb);
+        bb = quad_sum(bb);
+        float gx[4][4];
+        const float inv = rsd * (1.f / FD);
+        float sg = 0.f, sx = 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const float ggx = (gg[r][e] - (s0 + xh[r][e] * a) * (1.f / FD)) * rsd;
+            gy[r][e] = gam[r][e] * ggx;
+            dgam[r][e] += go[r][e] * ggx + gy[r][e] * xh[r][e];
+            dbet[r][e] += gy[r][e];
+            gx[r][e] = gy[r][e] * gam[r][e] - (go[r][e] * gam[r][e] * a + gg[r][e] * bb) * inv;
+            sg += (-gx[r][e] * xh[r][e] - gg[r][e] * gz[r][e]) * rsd;
+            sx += gx[r][e];
+          }
+        sg = quad_sum(sg);
+        sx = quad_sum(sx);
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            gx[r][e] = gx[r][e] * rsd + (sg * xh[r][e] - sx * rsd) * (1.f / FD);   // dZ2
+            xh[r][e] = -gy[r][e];                                                   // dXV
+          }
+        ln_store(s_a + tok * LDB, gx, fq);
+        ln_accumulate(p.grad_L_XV + xo + tok * FD, xh, fq);
+      }
+      __syncthreads();  // dZ2 tile complete; partial tiles free again
+
+      // ---- inner MLP, backwards (uses the state BEFORE this mini-batch)
+      {
+        WAVE_SYNC();
+        const Opd uP = lds_tr_kappa(s_bnc, lane);          // -eta*u: lane = hid, contraction = tok
+        Opd dz1Q;                                          // lane = tok, contraction = hid
         {
           Acc dx2;
           acc_zero(dx2);
-          mma(dx2, gw2T, gz2B);                          // P2 = gZ2 gW2^T  (rows hid, lane = tok)
+          {
+            const Opd gw2T = bounce(s_bnc, cvt_chain(gW2s), lane);   // lane = hid, contraction = F
+            const Opd gz2B = lds_rows_kappa(s_gz2, c, h);            // lane = tok, contraction = F
+            mma(dx2, gw2T, gz2B);                                    // P2 = gZ2 gW2^T  (rows hid, lane = tok)
+          }
 #pragma unroll
           for (int rb = 0; rb < 2; rb++)
 #pragma unroll
             for (int cb = 0; cb < 2; cb++)
 #pragma unroll
               for (int i = 0; i < 16; i++) dx2.b[rb][cb][i] *= -eta_cb[cb];
-          const Opd dz2B = lds_rows_kappa(s_a, c, h);    // lane = tok, contraction = F
-          mma(dx2, w2tA, dz2B);                          // + dZ2 W2^T
-          // dZ1 = dX2*gelu' - eta * R * S * gelu''   with R = gZ2 W2^T, dl/dZ1 = R*gelu'
-#pragma unroll
-          for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-            for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-              for (int i = 0; i < 16; i++) {
-                const float r0 = R.b[rb][cb][i];
-                dx2.b[rb][cb][i] = dx2.b[rb][cb][i] * d1.b[rb][cb][i]
-                                   - eta_cb[cb] * r0 * S.b[rb][cb][i] * d2.b[rb][cb][i];
-              }
-          const Opd dz1Q = cvt_chain(dx2);               // lane = tok, contraction = hid
           {
-            Acc dk;
-            acc_zero(dk);
-            mma(dk, gw1T, g1Q);                          // -eta * gZ1 gW1^T   (rows F, lane = tok)
-            mma(dk, cvt_chain(W1t), dz1Q);               // + dZ1 W1^T  (W1 before the step)
-            lds_store_partial(s_Pw, dk, c, h);
+            const Opd dz2B = lds_rows_kappa(s_a, c, h);    // lane = tok, contraction = F
+            const Opd w2tA = cvt_chain(W2t);               // W2 before the step
+            mma(dx2, w2tA, dz2B);                          // + dZ2 W2^T
           }
-          const Opd dz1P = bounce(s_bnc, dz1Q, lane);    // lane = hid, contraction = tok
-          const Opd dz2T = lds_tr_kappa(s_a, lane);      // lane = F,   contraction = tok
+          // dZ1 = dX2*gelu' - eta * R * S * gelu''
+#pragma unroll
+          for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+#pragma unroll
+              for (int jj = 0; jj < 8; jj++)
+                dz1Q.v[cb][s][jj] = (bf16)__builtin_fmaf(dx2.b[s >> 1][cb][8 * (s & 1) + jj], (float)d1p.v[cb][s][jj],
+                                                         (float)t2p.v[cb][s][jj]);
+        }
+        {
+          // G1 = -eta * dl/dZ1 exactly as the replay fed it to the weight step (lane = tok)
+          const Opd g1Q = opd_load(p.grad_l_wrt_Z1_group + ho, tid);
+          Acc dk;
+          acc_zero(dk);
+          {
+            const Opd gw1T = bounce(s_bnc, cvt_chain(gW1s), lane);   // lane = F, contraction = hid
+            mma(dk, gw1T, g1Q);                                      // -eta * gZ1 gW1^T   (rows F, lane = tok)
+          }
+          {
+            // undo the W1 step: W1 before = W1 after - XK^T G1
+            const Opd g1Pn = opd_neg(bounce(s_bnc, g1Q, lane));      // lane = hid, contraction = tok
+            const Opd xkT = lds_tr_kappa(s_xk, lane);                // lane = F,   contraction = tok
+            mma(W1t, g1Pn, xkT);
+          }
+          {
+            const Opd w1tA = cvt_chain(W1t);                         // W1 before the step
+            mma(dk, w1tA, dz1Q);                                     // + dZ1 W1^T
+          }
+          lds_store_partial(s_Pw, dk, c, h);
+        }
+        {
+          const Opd gz2T = lds_tr_kappa(s_gz2, lane);                // lane = F, contraction = tok
           mma(gW2s, uP, gz2T);
-          mma(gW2s, x2P, dz2T);
-          rowsum_mma(gb2, dz2T, ones);
+        }
+        {
+          const Opd dz2T = lds_tr_kappa(s_a, lane);                  // lane = F, contraction = tok
+          {
+            const Opd x2P = bounce(s_bnc, opd_load(p.X2_group + ho, tid), lane);
+            mma(gW2s, x2P, dz2T);
+          }
+          if (w == 0) lds_rowsum_add(s_gb2, dz2T, ones, c, h);
+        }
+        {
+          const Opd dz1P = bounce(s_bnc, dz1Q, lane);                // lane = hid, contraction = tok
           const Opd xkT = lds_tr_kappa(s_xk, lane);
           mma(gW1s, xkT, dz1P);
-          rowsum_mma(gb1, dz1P, ones);
+          lds_rowsum_add(s_gb1w, dz1P, ones, c, h);
         }
-        __syncthreads();  // partial dXK tiles complete
-        {
-          float z[4][4];
+      }
+      __syncthreads();  // partial dXK tiles complete
+      {
+        float z[4][4];
+        ln_gather0(z, s_P, tok, fq);
 #pragma unroll
-          for (int r = 0; r < 4; r++) {
-            f32x4 a = {0.f, 0.f, 0.f, 0.f};
+        for (int r = 0; r < 4; r++)
 #pragma unroll
-            for (int v = 0; v < 4; v++) a += *reinterpret_cast<const f32x4*>(s_P + v * 64 * LDP + tok * LDP + 16 * r + 4 * fq);
-#pragma unroll
-            for (int e = 0; e < 4; e++) z[r][e] = a[e] + gy[r][e];
-          }
-          ln_accumulate(p.grad_L_XK + xo + tok * FD, z, fq);
-        }
+          for (int e = 0; e < 4; e++) z[r][e] += gy[r][e];
+        ln_accumulate(p.grad_L_XK + xo + tok * FD, z, fq);
       }
     }
   }
@@ -815,10 +919,9 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
   // ---- outputs that are written once
   acc_store_rows(gW1s, p.grad_L_W1_init + (size_t)bh * FD * HID, HID, 0, 64 * w, c, h);
   acc_store_rows(gW2s, p.grad_L_W2_init + (size_t)bh * HID * FD, FD, 64 * w, 0, c, h);
-  if (c == 0) {
-    rowvec_store(gb1, p.grad_L_b1_init + (size_t)bh * HID + 64 * w, h);
-    if (w == 0) rowvec_store(gb2, p.grad_L_b2_init + (size_t)bh * FD, h);
-  }
+  __syncthreads();
+  p.grad_L_b1_init[(size_t)bh * HID + tid] = s_gb1[tid];
+  if (tid < FD) p.grad_L_b2_init[(size_t)bh * FD + tid] = s_gb2[tid];
   // norm-weight / norm-bias gradients: sum over the 16 tokens of the wave, then over the 4 waves
 #pragma unroll
   for (int r = 0; r < 4; r++)
