@@ -116,6 +116,22 @@ def _rb(x):
     return x.to(torch.bfloat16).to(x.dtype)
 
 
+class OperandRounding:
+    """Which matrix-product operands are rounded to bf16: ``w`` weights and weight gradients,
+    ``a`` activations, ``g`` activation gradients.  Used to study where the operand precision matters."""
+
+    def __init__(self, w=True, a=True, g=True):
+        self.w = _rb if w else _ident
+        self.a = _rb if a else _ident
+        self.g = _rb if g else _ident
+
+
+def _cat(rnd):
+    if isinstance(rnd, OperandRounding):
+        return rnd.w, rnd.a, rnd.g
+    return rnd, rnd, rnd
+
+
 class State(NamedTuple):
     W1: torch.Tensor
     b1: torch.Tensor
@@ -134,18 +150,19 @@ def forward_step(state: State, xq, xk, xv, eta, gamma, beta, *, rnd=_ident,
     """
     W1, b1, W2, b2 = state
     T = lambda a: a.transpose(-1, -2)
-    Z1 = rnd(xk) @ rnd(W1) + b1
+    rw, ra, rg = _cat(rnd)
+    Z1 = ra(xk) @ rw(W1) + b1
     X2 = gelu(Z1)
-    Z2 = rnd(X2) @ rnd(W2) + b2
+    Z2 = ra(X2) @ rw(W2) + b2
     gZ2, xhat_f, std_f, g_out, g_xhat = ln_l2_grad(Z2, xv - xk, gamma, beta)
-    gZ1 = (rnd(gZ2) @ T(rnd(W2))) * gelu_tanh_d1(Z1)
-    W1n = W1 - T(rnd(xk)) @ rnd(eta * gZ1)
+    gZ1 = (rg(gZ2) @ T(rw(W2))) * gelu_tanh_d1(Z1)
+    W1n = W1 - T(ra(xk)) @ rg(eta * gZ1)
     b1n = b1 - (eta * gZ1).sum(dim=-2, keepdim=True)
-    W2n = W2 - T(rnd(X2)) @ rnd(eta * gZ2)
+    W2n = W2 - T(ra(X2)) @ rg(eta * gZ2)
     b2n = b2 - (eta * gZ2).sum(dim=-2, keepdim=True)
-    Z1b = rnd(xq) @ rnd(W1n) + b1n
+    Z1b = ra(xq) @ rw(W1n) + b1n
     X2b = gelu(Z1b)
-    Z2b = rnd(X2b) @ rnd(W2n) + b2n
+    Z2b = ra(X2b) @ rw(W2n) + b2n
     xhat_l, std_l = ln_fwd(Z2b)
     out = xq + gamma * xhat_l + beta
     saved = dict(Z1=Z1, X2=X2, xhat_f=xhat_f, std_f=std_f, g_out=g_out, g_xhat=g_xhat,
@@ -167,7 +184,8 @@ def ttt_forward(XQ, XK, XV, last_eta, ttt_norm_weight, ttt_norm_bias, W1, b1, W2
                 checkpoint_group_size: int, *, dtype=torch.float32, emulate_bf16_operands=False,
                 gelu=gelu_tanh):
     """Forward scan.  Returns (Out [B,NH,NC,CS,F], checkpoints State of [B,NH,K,..], final State)."""
-    rnd = _rb if emulate_bf16_operands else _ident
+    rnd = emulate_bf16_operands if isinstance(emulate_bf16_operands, OperandRounding) else \
+        (_rb if emulate_bf16_operands else _ident)
     XQ, XK, XV = XQ.to(dtype), XK.to(dtype), XV.to(dtype)
     eta = _eta5(last_eta).to(dtype)
     gamma, beta = _norm_params(ttt_norm_weight, ttt_norm_bias, dtype)
@@ -242,23 +260,24 @@ def backward_step(gO, g: State, init: State, last: State, s: Dict[str, torch.Ten
     # output LayerNorm + residual
     d_beta = sT(gO)
     d_gamma = sT(gO * s["xhat_l"])
+    rw, ra, rg = _cat(rnd)
     gZ2b = ln_bwd(gO * gamma, s["xhat_l"], s["std_l"])
     # post-update forward
-    gZ1b = (rnd(gZ2b) @ T(rnd(last.W2))) * gelu_tanh_d1(s["Z1b"])
+    gZ1b = (rg(gZ2b) @ T(rw(last.W2))) * gelu_tanh_d1(s["Z1b"])
     gb2 = gb2 + sT(gZ2b)
-    gW2 = gW2 + T(rnd(s["X2b"])) @ rnd(gZ2b)
+    gW2 = gW2 + T(ra(s["X2b"])) @ rg(gZ2b)
     gb1 = gb1 + sT(gZ1b)
-    gW1 = gW1 + T(rnd(xq)) @ rnd(gZ1b)
-    dXQ = gO + rnd(gZ1b) @ T(rnd(last.W1))
+    gW1 = gW1 + T(ra(xq)) @ rg(gZ1b)
+    dXQ = gO + rg(gZ1b) @ T(rw(last.W1))
     # the weight step: W_next = W - (eta x)^T g
     d1 = gelu_tanh_d1(s["Z1"])
-    ggZ1 = -(rnd(eta * xk) @ rnd(gW1)) - eta * gb1
+    ggZ1 = -(ra(eta * xk) @ rw(gW1)) - eta * gb1
     u = ggZ1 * d1
-    ggZ2 = -(rnd(eta * s["X2"]) @ rnd(gW2)) - eta * gb2 + rnd(u) @ rnd(init.W2)
-    P1 = rnd(s["gZ1"]) @ T(rnd(gW1))
-    P2 = rnd(s["gZ2"]) @ T(rnd(gW2))
+    ggZ2 = -(ra(eta * s["X2"]) @ rw(gW2)) - eta * gb2 + rg(u) @ rw(init.W2)
+    P1 = rg(s["gZ1"]) @ T(rw(gW1))
+    P2 = rg(s["gZ2"]) @ T(rw(gW2))
     d_eta = -sF(P2 * s["X2"]) - sF(gb2 * s["gZ2"]) - sF(P1 * xk) - sF(gb1 * s["gZ1"])
-    gW2_via_gZ1 = T(rnd(u)) @ rnd(s["gZ2"])
+    gW2_via_gZ1 = T(rg(u)) @ rg(s["gZ2"])
     # second-order pass through the LayerNorm-fused loss gradient
     xh, sd = s["xhat_f"], s["std_f"]
     a = sF(ggZ2 * xh)
@@ -271,14 +290,14 @@ def backward_step(gO, g: State, init: State, last: State, s: Dict[str, torch.Ten
     g_std = (-gx * xh - ggZ2 * s["gZ2"]) / sd
     dZ2 = gx / sd + (sF(g_std) * xh - sF(gx) / sd) / n
     # inner MLP
-    R = rnd(s["gZ2"]) @ T(rnd(init.W2))            # = gZ1 before the GELU' factor
-    dX2 = rnd(dZ2) @ T(rnd(init.W2)) - eta * P2
+    R = rg(s["gZ2"]) @ T(rw(init.W2))              # = gZ1 before the GELU' factor
+    dX2 = rg(dZ2) @ T(rw(init.W2)) - eta * P2
     dZ1 = dX2 * d1 + R * ggZ1 * gelu_tanh_d2(s["Z1"])
-    dXK = g_y - eta * P1 + rnd(dZ1) @ T(rnd(init.W1))
+    dXK = g_y - eta * P1 + rg(dZ1) @ T(rw(init.W1))
     dXV = -g_y
-    gW2 = gW2 + gW2_via_gZ1 + T(rnd(s["X2"])) @ rnd(dZ2)
+    gW2 = gW2 + gW2_via_gZ1 + T(ra(s["X2"])) @ rg(dZ2)
     gb2 = gb2 + sT(dZ2)
-    gW1 = gW1 + T(rnd(xk)) @ rnd(dZ1)
+    gW1 = gW1 + T(ra(xk)) @ rg(dZ1)
     gb1 = gb1 + sT(dZ1)
     return (dXQ, dXK, dXV, d_eta), State(gW1, gb1, gW2, gb2), (d_gamma, d_beta)
 
@@ -294,7 +313,8 @@ def ttt_backward(XQ, XK, XV, last_eta, ttt_norm_weight, ttt_norm_bias, ckpt: Sta
     Returns a dict with the operator's ten output gradients (norm grads per batch element,
     [B,NH,1,F]) in ``dtype``.
     """
-    rnd = _rb if emulate_bf16_operands else _ident
+    rnd = emulate_bf16_operands if isinstance(emulate_bf16_operands, OperandRounding) else \
+        (_rb if emulate_bf16_operands else _ident)
     XQ, XK, XV, gO = XQ.to(dtype), XK.to(dtype), XV.to(dtype), grad_out.to(dtype)
     eta = _eta5(last_eta).to(dtype)
     gamma, beta = _norm_params(ttt_norm_weight, ttt_norm_bias, dtype)
