@@ -91,6 +91,8 @@ def main():
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c4")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-mb", type=int, default=1536, help="mini-batches in the CPU baseline sample")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 1 GiB device copy, so that a counter run has a kernel of known traffic")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (every (batch, head) recurrence is independent and no "
@@ -129,6 +131,12 @@ def main():
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     host.set_synchronize(True)
+    if a.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)     # 1 GiB read + 1 GiB written
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     assert bool(torch.isfinite(t["grad_L_W1_init"]).all()) and bool(torch.isfinite(t["Out"].float()).all())
 
     fwd_ms = sum(e[0].elapsed_time(e[1]) for e in events) / a.steps
