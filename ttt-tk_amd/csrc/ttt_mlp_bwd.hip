@@ -12,28 +12,29 @@
 // the contraction index is bounced once through a wave-private LDS tile (row store + transposing read).
 //
 // State in registers:
-//   replay : W1s [F x hid], W2s [hid x F], W2t [F x hid], b1 (accumulator-row form), b2
-//   reverse: gW1s [F x hid], gW2s [hid x F] (running gradients), W1t [hid x F], W2t [F x hid]
-//            (the weights themselves, stepped back one mini-batch at a time by undoing the update,
-//            so no per-mini-batch weight snapshot is ever written), gb1, gb2.
+//   replay : W1s [F x hid], W2s [hid x F], W2t [F x hid] (fp32 accumulator tiles); b1, b2 in LDS
+//   reverse: gW1s [F x hid], gW2s [hid x F] (running gradients) only; gb1, gb2 in LDS.  The weights
+//            enter the reverse walk as ready-made bf16 MFMA operands: after every mini-batch the replay
+//            stores the operand images of W1^T[shard] and W2[shard]^T, and the walk reads the image of
+//            the state after and before the step (before the first step of a group: converted straight
+//            from the fp32 checkpoint).  Half the accumulator file therefore stays free for products.
 // While a group is replayed the running gradients are parked in the caller's W*_init_group scratch.
-// Saved per mini-batch (caller's *_group scratch): Z1 and Z1_bar as bf16 register images
-// (Z1_group, Z1_bar_group); the two bf16 operands of the weight step, X2 (X2_group) and
-// G1 = -eta*dl/dZ1 (grad_l_wrt_Z1_group), as register images and G2 = -eta*dl/dZ2
-// (grad_x_hat_fused_group) as a tile, so that undoing the step reproduces the update bit for bit;
-// x_hat / grad_output of the fused LayerNorm loss, dl/dZ2 and the output LayerNorm's x_hat as bf16
-// [tok][F] tiles; the two std vectors in fp32.
+// Saved per mini-batch (caller's *_group scratch): Z1 and Z1_bar as bf16 register images (Z1_group,
+// Z1_bar_group); the two weight operand images (X2_group: W1^T[shard], grad_l_wrt_Z1_group:
+// W2[shard]^T); x_hat / grad_output of the fused LayerNorm loss, dl/dZ2 and the output LayerNorm's
+// x_hat as bf16 [tok][F] tiles; the two std vectors in fp32.
 #include "ttt_mlp_common.hpp"
 #include "ttt_mlp_kernels.hpp"
 
 namespace ttt {
 
 constexpr int SB_TILE = 64 * LDB * 2;
-constexpr int SB_XQ = 0;
-constexpr int SB_XK = SB_XQ + SB_TILE;
+constexpr int SB_XQ = 0;                  // reverse: XQ until the post-update stage is done, then (with SB_E2)
+constexpr int SB_E2 = SB_XQ + SB_TILE;    //          the fp32 park of g_y ; replay: XQ and XV
+constexpr int SB_XK = SB_E2 + SB_TILE;
 constexpr int SB_GZ2 = SB_XK + SB_TILE;   // replay: G2 = -eta*dl/dZ2 ; reverse: raw dl/dZ2
-constexpr int SB_E2 = SB_GZ2 + SB_TILE;   // reverse: G2 ; replay: XV
-constexpr int SB_A = SB_E2 + SB_TILE;     // reverse: gZ2_bar, later dZ2
+constexpr int SB_A = SB_GZ2 + SB_TILE;    // reverse: gZ2_bar, later dZ2
+static_assert(2 * SB_TILE >= CS * FD * 4, "g_y park does not fit");
 constexpr int SB_P = SB_A + SB_TILE;      // 4 fp32 partial tiles
 constexpr int SB_PTILE = 64 * LDP * 4;
 constexpr int SB_BNC = SB_P + 4 * SB_PTILE;   // 4 wave-private bounce tiles
@@ -181,6 +182,29 @@ TTT_DEV void acc_scale(Acc& a, float s) {
       for (int i = 0; i < 16; i++) a.b[rb][cb][i] *= s;
 }
 
+// Sum over the 16 lanes of a wave that share lane % 4 (the 16 tokens of a LayerNorm stage), result in
+// all of them: two row rotations inside each row of 16 lanes, then across the four rows.
+TTT_DEV float token_sum16(float x) {
+  x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x124, 0xF, 0xF, false));  // row_ror:4
+  x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x128, 0xF, 0xF, false));  // row_ror:8
+  x += __shfl_xor(x, 16, 64);
+  x += __shfl_xor(x, 32, 64);
+  return x;
+}
+// acc[16r + 4fq + e] += sum over this wave's tokens of x[r][e]   (wave-private LDS vector)
+TTT_DEV void ln_token_sum_add(float* s_acc, const float (&x)[4][4], int q, int fq) {
+#pragma unroll
+  for (int r = 0; r < 4; r++) {
+    f32x4 v;
+#pragma unroll
+    for (int e = 0; e < 4; e++) v[e] = token_sum16(x[r][e]);
+    if (q == 0) {
+      f32x4* d = reinterpret_cast<f32x4*>(s_acc + 16 * r + 4 * fq);
+      *d = *d + v;
+    }
+  }
+}
+
 // ------------------------------------------------------------------ LayerNorm-lane helpers
 // A lane of the LayerNorm stage owns token `tok` and features 16r + 4fq + e (r, e in 0..3).
 TTT_DEV void ln_load(float (&x)[4][4], const bf16* row, int fq) {
@@ -322,6 +346,103 @@ TTT_DEV void ln_gather0(float (&z)[4][4], const float* s_P, int tok, int fq) {
   }
 }
 
+// ---------------------------------------------------------------- just-in-time operand pieces
+// One MFMA operand piece = 8 bf16 per lane = (free block blk, k-step s).  Loading pieces right
+// before the MFMA that consumes them keeps whole 64x64 operands out of the register file.
+constexpr int LDT = 68;   // row stride of the two operand tiles that share a wave's partial tile
+template <int LD>
+TTT_DEV bf16x8 piece_rows(const bf16* tile, int blk, int s, int c, int h) {
+  const bf16* q = tile + (32 * blk + c) * LD + 16 * s + 4 * h;
+  return cat(*reinterpret_cast<const bf16x4*>(q), *reinterpret_cast<const bf16x4*>(q + 8));
+}
+template <int LD>
+TTT_DEV bf16x8 piece_tr(const bf16* tile, int blk, int s, int lane) {
+  const int h = lane >> 5, c = lane & 31, i = lane & 15;
+  const bf16* q = tile + (16 * s + 4 * h + (i >> 2)) * LD + 32 * blk + 16 * (c >> 4) + 4 * (i & 3);
+  return cat(lds_tr4(q), lds_tr4(q + 8 * LD));
+}
+template <int LD>
+TTT_DEV void store_piece_rows(bf16* tile, int blk, int s, int c, int h, bf16x8 v) {
+  bf16* q = tile + (32 * blk + c) * LD + 16 * s + 4 * h;
+  *reinterpret_cast<bf16x4*>(q) = __builtin_shufflevector(v, v, 0, 1, 2, 3);
+  *reinterpret_cast<bf16x4*>(q + 8) = __builtin_shufflevector(v, v, 4, 5, 6, 7);
+}
+template <int LD>
+TTT_DEV void store_opd_rows(bf16* tile, const Opd& o, int c, int h) {
+#pragma unroll
+  for (int fb = 0; fb < 2; fb++)
+#pragma unroll
+    for (int s = 0; s < 4; s++) store_piece_rows<LD>(tile, fb, s, c, h, o.v[fb][s]);
+}
+// Piece (free block fb, k-step s) of the chained operand of an accumulator tile.
+TTT_DEV bf16x8 piece_state(const Acc& x, int fb, int s) { return pack8(x.b[s >> 1][fb], s & 1); }
+template <int LD>
+TTT_DEV void store_state_rows(bf16* tile, const Acc& x, int c, int h) {
+#pragma unroll
+  for (int fb = 0; fb < 2; fb++)
+#pragma unroll
+    for (int s = 0; s < 4; s++) store_piece_rows<LD>(tile, fb, s, c, h, piece_state(x, fb, s));
+}
+#define MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16((a), (b), (c), 0, 0, 0)
+// d += A * B, pieces produced by the callables fa(blk, s) and fb(blk, s).
+template <class FA, class FB>
+TTT_DEV void mma_jit(Acc& d, FA fa, FB fb) {
+#pragma unroll
+  for (int s = 0; s < 4; s++) {
+    const bf16x8 a0 = fa(0, s), a1 = fa(1, s), b0 = fb(0, s), b1 = fb(1, s);
+    d.b[0][0] = MFMA(a0, b0, d.b[0][0]);
+    d.b[0][1] = MFMA(a0, b1, d.b[0][1]);
+    d.b[1][0] = MFMA(a1, b0, d.b[1][0]);
+    d.b[1][1] = MFMA(a1, b1, d.b[1][1]);
+  }
+}
+// s_vec[row] += sum over the contraction of the operand whose pieces fa(rb, s) yields.
+template <class FA>
+TTT_DEV void lds_rowsum_add_jit(float* s_vec, FA fa, bf16x8 ones, int c, int h) {
+  f32x16 t[2];
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) t[rb][i] = 0.f;
+#pragma unroll
+  for (int s = 0; s < 4; s++)
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++) t[rb] = MFMA(fa(rb, s), ones, t[rb]);
+  if (c == 0) {
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        f32x4* q = reinterpret_cast<f32x4*>(s_vec + 32 * rb + 8 * g + 4 * h);
+        f32x4 v = *q;
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] += t[rb][4 * g + e];
+        *q = v;
+      }
+  }
+  WAVE_SYNC();
+}
+
+TTT_DEV bf16x8 cvt8(const f32x4 lo, const f32x4 hi) {
+  bf16x8 o;
+#pragma unroll
+  for (int e = 0; e < 4; e++) { o[e] = (bf16)lo[e]; o[4 + e] = (bf16)hi[e]; }
+  return o;
+}
+// MFMA operand (kappa order) straight from a row-major fp32 matrix: lane = row r0 + 32*fb + c,
+// contraction = columns c0 .. c0+63.
+TTT_DEV Opd opd_from_f32_rows(const float* g, int ld, int r0, int c0, int c, int h) {
+  Opd o;
+#pragma unroll
+  for (int fb = 0; fb < 2; fb++)
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      const float* q = g + (size_t)(r0 + 32 * fb + c) * ld + c0 + 16 * s + 4 * h;
+      o.v[fb][s] = cvt8(*reinterpret_cast<const f32x4*>(q), *reinterpret_cast<const f32x4*>(q + 8));
+    }
+  return o;
+}
+
 __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   bf16* s_xq = reinterpret_cast<bf16*>(smem + SB_XQ);
@@ -355,11 +476,12 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
     s_gb2[tid] = p.grad_L_b2_last[(size_t)bh * FD + tid];
   }
   s_gb1[tid] = p.grad_L_b1_last[(size_t)bh * HID + tid];
-  float dgam[4][4], dbet[4][4];
-#pragma unroll
-  for (int r = 0; r < 4; r++)
-#pragma unroll
-    for (int e = 0; e < 4; e++) dgam[r][e] = dbet[r][e] = 0.f;
+  // Norm-weight / norm-bias gradients accumulate per wave in LDS (summed over the wave's 16 tokens
+  // with cross-lane adds in a fixed order); summed over the waves at the end.
+  float* s_dgw = s_red + (w * 2 + 0) * FD;
+  float* s_dbw = s_red + (w * 2 + 1) * FD;
+  if (lane < FD) { s_dgw[lane] = 0.f; s_dbw[lane] = 0.f; }
+  float* s_gy = reinterpret_cast<float*>(smem + SB_XQ) + tok * FD;   // this lane's row of the g_y park
   bf16x8 ones;
 #pragma unroll
   for (int j = 0; j < 8; j++) ones[j] = (bf16)1.0f;
@@ -372,6 +494,10 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
   const size_t g_T = (size_t)bh * cgs * CS;             // [cgs][64] vectors
   float* park_W1 = p.W1_init_group + (size_t)bh * cgs * FD * HID;
   float* park_W2 = p.W2_init_group + (size_t)bh * cgs * HID * FD;
+  // During the reverse walk the same two 64 KiB slots park what must survive the LayerNorm stage.
+  bf16* park_d1 = reinterpret_cast<bf16*>(park_W1);                  // 32 KiB register image
+  bf16* park_t2 = park_d1 + CS * HID;                                // 32 KiB register image
+  float* park_dk = park_W2 + (size_t)w * (CS * FD) ;                 // 16 KiB per wave
 
   // running gradients wrt the state after the last mini-batch
   Acc gW1s, gW2s;
@@ -380,14 +506,12 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
 
   for (int k = p.K - 1; k >= 0; k--) {
     const int n_mb = min(cgs, p.NC - k * cgs);
-    Acc W2t;  // survives from the replay into the reverse walk
-    Acc W1t;
     // ================================================================= replay
     {
       // park the running gradients while the forward state needs the registers
       acc_store_rows(gW1s, park_W1, HID, 0, 64 * w, c, h);
       acc_store_rows(gW2s, park_W2, FD, 64 * w, 0, c, h);
-      Acc W1s, W2s;
+      Acc W1s, W2s, W2t;
       const size_t slot = (size_t)bh * p.K + k;
       acc_load_rows(W1s, p.W1_ck + slot * FD * HID, HID, 0, 64 * w, c, h);
       acc_load_rows(W2s, p.W2_ck + slot * HID * FD, FD, 64 * w, 0, c, h);
@@ -431,7 +555,6 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
               }
           x2Q = cvt_chain(x2);
         }
-        opd_store(p.X2_group + g_TH + (size_t)j * (CS * HID), x2Q, tid);
         {
           const Opd w2A = cvt_chain(W2s);
           Acc z2;
@@ -476,7 +599,6 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
 #pragma unroll
             for (int e = 0; e < 4; e++) gx[r][e] *= neg_eta;                                   // G2
           ln_store(s_gz2 + tok * LDB, gx, fq);
-          ln_store(p.grad_x_hat_fused_group + so, gx, fq);   // the exact bf16 operand of the weight step
           if (fq == 0) p.std_fused_group[g_T + (size_t)j * CS + tok] = sd;
         }
         __syncthreads();
@@ -499,7 +621,6 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
                 for (int i = 0; i < 16; i++) g1.b[rb][cb][i] *= d1.b[rb][cb][i];
             g1Q = cvt_chain(g1);
           }
-          opd_store(p.grad_l_wrt_Z1_group + g_TH + (size_t)j * (CS * HID), g1Q, tid);
           {
             const Opd g2T = lds_tr_kappa(s_gz2, lane);       // lane = F, contraction = tok
             const Opd x2P = bounce(s_bnc, x2Q, lane);        // lane = hid, contraction = tok
@@ -514,12 +635,15 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
             lds_rowsum_add(s_b1w, g1P, ones, c, h);
           }
         }
+        // operand images of the state after this step, for the reverse walk
+        opd_store(p.grad_l_wrt_Z1_group + g_TH + (size_t)j * (CS * HID), cvt_chain(W2t), tid);   // lane = hid, contraction = F
         // post-update forward on XQ
         {
           Acc z1b;
           acc_init_rows_lds(z1b, s_b1w, h);
           {
             const Opd w1A = cvt_chain(W1s);
+            opd_store(p.X2_group + g_TH + (size_t)j * (CS * HID), bounce(s_bnc, w1A, lane), tid);   // lane = F, contraction = hid
             const Opd xqB = lds_rows_kappa(s_xq, c, h);
             mma(z1b, w1A, xqB);
           }
@@ -547,23 +671,18 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
           if (fq == 0) p.std_ln_group[g_T + (size_t)j * CS + tok] = sd;
         }
       }
-      // W1t = transpose of W1s through this wave's fp32 partial tile
-      __syncthreads();
-      lds_store_partial(s_Pw, W1s, c, h);  // stored [hid][F]
-      __syncthreads();
-#pragma unroll
-      for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-        for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-          for (int i = 0; i < 16; i++)
-            W1t.b[rb][cb][i] = s_Pw[(32 * rb + 8 * (i >> 2) + 4 * h + (i & 3)) * LDP + 32 * cb + c];
       // running gradients back into registers
       acc_load_rows(gW1s, park_W1, HID, 0, 64 * w, c, h);
       acc_load_rows(gW2s, park_W2, FD, 64 * w, 0, c, h);
     }
 
     // ================================================================= reverse walk
+    // Wave-private LDS tiles of the walk: T0 = the bounce tile (row stride LDB); T1, T2 = the two
+    // halves of this wave's fp32 partial tile (row stride LDT), free whenever no partial sum is in it.
+    const size_t slot = (size_t)bh * p.K + k;
+    bf16* const T0 = s_bnc;
+    bf16* const T1 = reinterpret_cast<bf16*>(s_Pw);
+    bf16* const T2 = T1 + 64 * LDT;
     for (int j = n_mb - 1; j >= 0; j--) {
       const int mb = k * cgs + j;
       const size_t xo = x_base + (size_t)mb * (CS * FD);
@@ -576,8 +695,10 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
       stage_tile(s_xq, p.XQ + xo, tid);
       stage_tile(s_xk, p.XK + xo, tid);
       stage_tile(s_gz2, p.grad_l_wrt_Z2_group + so, tid);
-      stage_tile(s_e2, p.grad_x_hat_fused_group + so, tid);   // G2 = -eta * dl/dZ2 as used by the weight step
       if (tid < CS) s_eta[tid] = bf2f(p.last_eta[eta_base + (size_t)mb * CS + tid]);
+      // operand tiles of the state after this step: T1 = W2 rows [hid][F], T2 = W1^T rows [F][hid]
+      store_opd_rows<LDT>(T1, opd_load(p.grad_l_wrt_Z1_group + ho, tid), c, h);
+      store_opd_rows<LDT>(T2, opd_load(p.X2_group + ho, tid), c, h);
 
       // ---- output LayerNorm backward (LayerNorm lanes)
       {
@@ -589,11 +710,13 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
 #pragma unroll
         for (int r = 0; r < 4; r++)
 #pragma unroll
-          for (int e = 0; e < 4; e++) {
-            dbet[r][e] += gO[r][e];
-            dgam[r][e] = __builtin_fmaf(gO[r][e], xh[r][e], dgam[r][e]);
-            gx[r][e] = gO[r][e] * gam[r][e];
-          }
+          for (int e = 0; e < 4; e++) gx[r][e] = gO[r][e] * xh[r][e];
+        ln_token_sum_add(s_dbw, gO, q, fq);
+        ln_token_sum_add(s_dgw, gx, q, fq);
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) gx[r][e] = gO[r][e] * gam[r][e];
         const float s1 = quad_sum(sum16(gx)), s2 = quad_sum(dot16(gx, xh));
         const float sc = 1.f / (FD * sd);
 #pragma unroll
@@ -606,50 +729,42 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
 
       // ---- post-update forward, backwards (uses the state AFTER this mini-batch)
       {
-        Opd x2bQ, gz1bQ;  // lane = tok, contraction = hid
+        Acc dq;
         {
-          Acc gz1b;
+          Acc gz1b;   // (gZ2_bar W2^T) * gelu'(Z1_bar): rows hid, lane = tok
           acc_zero(gz1b);
-          {
-            const Opd gz2bB = lds_rows_kappa(s_a, c, h);   // lane = tok, contraction = F
-            const Opd w2tA = cvt_chain(W2t);               // lane = hid, contraction = F   (W2 after the step)
-            mma(gz1b, w2tA, gz2bB);                        // rows hid, lane = tok
-          }
+          mma_jit(gz1b, [&](int blk, int s) { return piece_rows<LDT>(T1, blk, s, c, h); },
+                  [&](int blk, int s) { return piece_rows<LDB>(s_a, blk, s, c, h); });
+          WAVE_SYNC();   // T1 is overwritten below
           const Opd zimg = opd_load(p.Z1_bar_group + ho, tid);
 #pragma unroll
           for (int cb = 0; cb < 2; cb++)
 #pragma unroll
-            for (int s = 0; s < 4; s++)
+            for (int s = 0; s < 4; s++) {
+              bf16x8 x2b, gzb;
 #pragma unroll
               for (int jj = 0; jj < 8; jj++) {
                 float g, d;
                 gelu_fd((float)zimg.v[cb][s][jj], g, d);
-                gz1b.b[s >> 1][cb][8 * (s & 1) + jj] *= d;
-                x2bQ.v[cb][s][jj] = (bf16)g;
+                x2b[jj] = (bf16)g;
+                gzb[jj] = (bf16)(gz1b.b[s >> 1][cb][8 * (s & 1) + jj] * d);
               }
-          gz1bQ = cvt_chain(gz1b);
+              store_piece_rows<LDB>(T0, cb, s, c, h, x2b);    // X2_bar  rows [tok][hid]
+              store_piece_rows<LDT>(T1, cb, s, c, h, gzb);    // gZ1_bar rows [tok][hid]
+            }
         }
-        {
-          const Opd w1tA = cvt_chain(W1t);                 // lane = F, contraction = hid   (W1 after the step)
-          Acc dq;
-          acc_zero(dq);
-          mma(dq, w1tA, gz1bQ);                            // rows F, lane = tok
-          lds_store_partial(s_Pw, dq, c, h);
-        }
-        {
-          const Opd gz2bT = lds_tr_kappa(s_a, lane);       // lane = F, contraction = tok
-          {
-            const Opd x2bP = bounce(s_bnc, x2bQ, lane);    // lane = hid, contraction = tok
-            mma(gW2s, x2bP, gz2bT);
-          }
-          if (w == 0) lds_rowsum_add(s_gb2, gz2bT, ones, c, h);
-        }
-        {
-          const Opd gz1bP = bounce(s_bnc, gz1bQ, lane);
-          const Opd xqT = lds_tr_kappa(s_xq, lane);
-          mma(gW1s, xqT, gz1bP);
-          lds_rowsum_add(s_gb1w, gz1bP, ones, c, h);
-        }
+        WAVE_SYNC();
+        acc_zero(dq);
+        mma_jit(dq, [&](int blk, int s) { return piece_rows<LDT>(T2, blk, s, c, h); },      // W1 after: lane = F
+                [&](int blk, int s) { return piece_rows<LDT>(T1, blk, s, c, h); });         // gZ1_bar: lane = tok
+        mma_jit(gW2s, [&](int blk, int s) { return piece_tr<LDB>(T0, blk, s, lane); },      // X2_bar^T: lane = hid
+                [&](int blk, int s) { return piece_tr<LDB>(s_a, blk, s, lane); });          // gZ2_bar: lane = F
+        if (w == 0) lds_rowsum_add_jit(s_gb2, [&](int blk, int s) { return piece_tr<LDB>(s_a, blk, s, lane); }, ones, c, h);
+        mma_jit(gW1s, [&](int blk, int s) { return piece_tr<LDB>(s_xq, blk, s, lane); },    // XQ^T: lane = F
+                [&](int blk, int s) { return piece_tr<LDT>(T1, blk, s, lane); });           // gZ1_bar: lane = hid
+        lds_rowsum_add_jit(s_gb1w, [&](int blk, int s) { return piece_tr<LDT>(T1, blk, s, lane); }, ones, c, h);
+        WAVE_SYNC();   // every reader of T1 / T2 is done before the partial tile takes their place
+        lds_store_partial(s_Pw, dq, c, h);
       }
       __syncthreads();  // partial dXQ tiles complete; gb2 holds its value after the first update
       {
@@ -662,112 +777,100 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
           for (int e = 0; e < 4; e++) z[r][e] += gO[r][e];
         ln_accumulate(p.grad_L_XQ + xo + tok * FD, z, fq);
       }
+      __syncthreads();  // dXQ readers of the partial tiles are done: T1 / T2 are free again
 
-      // ---- the weight step, backwards.  Two packed tiles survive the LayerNorm stage:
-      //      d1p = gelu'(Z1) and t2p = -eta * (gZ2 W2^T) * (XK gW1 + gb1) * gelu''(Z1).
-      Opd d1p, t2p;
+      // ---- the weight step, backwards (uses the state BEFORE this mini-batch).
+      //      Survive the LayerNorm stage: X2 in T0; packed d1p = gelu'(Z1) and
+      //      t2p = -eta * (gZ2 W2^T) * (XK gW1 + gb1) * gelu''(Z1); the accumulator dk.
       {
-        const Opd x2Q = opd_load(p.X2_group + ho, tid);      // X2 exactly as the replay fed it to the weight step
-        {
-          // undo the W2 step with the very operands that made it: W2 before = W2 after - X2^T G2
-          const Opd x2P = bounce(s_bnc, x2Q, lane);          // lane = hid, contraction = tok
-          const Opd g2Tn = opd_neg(lds_tr_kappa(s_e2, lane));   // lane = F, contraction = tok
-          mma(W2t, g2Tn, x2P);
-        }
-        Opd uQ;   // (XK gW1 + gb1) * gelu'(Z1), lane = tok
-        float de3[2] = {0.f, 0.f};
-        {
-          const Opd w2tA = cvt_chain(W2t);                   // W2 before the step: lane = hid, contraction = F
-          const Opd gz2B = lds_rows_kappa(s_gz2, c, h);      // lane = tok, contraction = F
-          const Opd gw1A = cvt_chain(gW1s);                  // lane = hid, contraction = F
-          const Opd xkB = lds_rows_kappa(s_xk, c, h);
-          const Opd zimg = opd_load(p.Z1_group + ho, tid);
+        Opd d1p, t2p;
+        Acc dk;
+        // T1 = W2 before the step, rows [hid][F]; T2 = gW1, rows [hid][F]
+        store_opd_rows<LDT>(T1, (j > 0) ? opd_load(p.grad_l_wrt_Z1_group + ho - CS * HID, tid)
+                                        : opd_from_f32_rows(p.W2_ck + slot * HID * FD, FD, 64 * w, 0, c, h), c, h);
+        store_state_rows<LDT>(T2, gW1s, c, h);
+        WAVE_SYNC();
+        Acc R, S;   // R = gZ2 W2^T, S = XK gW1 + gb1   (rows hid, lane = tok)
+        acc_zero(R);
+        acc_init_rows_lds(S, s_gb1w, h);
+        mma_jit(R, [&](int blk, int s) { return piece_rows<LDT>(T1, blk, s, c, h); },
+                [&](int blk, int s) { return piece_rows<LDB>(s_gz2, blk, s, c, h); });
+        mma_jit(S, [&](int blk, int s) { return piece_rows<LDT>(T2, blk, s, c, h); },
+                [&](int blk, int s) { return piece_rows<LDB>(s_xk, blk, s, c, h); });
+        const Opd zimg = opd_load(p.Z1_group + ho, tid);
+        Acc pz;
+        acc_zero(pz);
+        acc_zero(dk);
+        float de1[2] = {0.f, 0.f}, de3[2] = {0.f, 0.f};
 #pragma unroll
-          for (int cb = 0; cb < 2; cb++) {
-            f32x16 R[2], S[2];   // R = gZ2 W2^T, S = XK gW1 + gb1 for tokens 32cb..32cb+31
+        for (int cb = 0; cb < 2; cb++) {
+          bf16x8 x2c[4], uc[4], g1c[4];
 #pragma unroll
-            for (int rb = 0; rb < 2; rb++)
+          for (int s = 0; s < 4; s++)
 #pragma unroll
-              for (int g = 0; g < 4; g++) {
-                const f32x4 v = *reinterpret_cast<const f32x4*>(s_gb1w + 32 * rb + 8 * g + 4 * h);
-#pragma unroll
-                for (int e = 0; e < 4; e++) { S[rb][4 * g + e] = v[e]; R[rb][4 * g + e] = 0.f; }
-              }
-#pragma unroll
-            for (int s = 0; s < 4; s++)
-#pragma unroll
-              for (int rb = 0; rb < 2; rb++) {
-                R[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w2tA.v[rb][s], gz2B.v[cb][s], R[rb], 0, 0, 0);
-                S[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gw1A.v[rb][s], xkB.v[cb][s], S[rb], 0, 0, 0);
-              }
-#pragma unroll
-            for (int s = 0; s < 4; s++)
-#pragma unroll
-              for (int jj = 0; jj < 8; jj++) {
-                float g, a, b;
-                gelu_fdd((float)zimg.v[cb][s][jj], g, a, b);
-                const float r0 = R[s >> 1][8 * (s & 1) + jj], sv = S[s >> 1][8 * (s & 1) + jj];
-                de3[cb] = __builtin_fmaf(r0 * a, sv, de3[cb]);          // dl/dZ1 * S
-                uQ.v[cb][s][jj] = (bf16)(sv * a);
-                d1p.v[cb][s][jj] = (bf16)a;
-                t2p.v[cb][s][jj] = (bf16)(-eta_cb[cb] * r0 * sv * b);
-              }
-          }
-        }
-        // partial ggZ2 / (-eta): gW2^T X2^T + W2^T uQ^T, and the first dEta partial sum
-        {
-          Acc pz;
-          acc_zero(pz);
-          {
-            const Opd gw2A = cvt_chain(gW2s);                // lane = F, contraction = hid
-            mma(pz, gw2A, x2Q);                              // rows F, lane = tok
-          }
-          float de1[2] = {0.f, 0.f};
-          {
-            const Opd gz2B = lds_rows_kappa(s_gz2, c, h);
-#pragma unroll
-            for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-              for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-                for (int t = 0; t < 2; t++)
-#pragma unroll
-                  for (int jj = 0; jj < 8; jj++)
-                    de1[cb] = __builtin_fmaf((float)gz2B.v[cb][2 * rb + t][jj], pz.b[rb][cb][8 * t + jj], de1[cb]);
-          }
-          {
-            const Opd w2sA = bounce(s_bnc, cvt_chain(W2t), lane);   // W2 before the step: lane = F, contraction = hid
-            mma(pz, w2sA, uQ);
-          }
-          __syncthreads();  // dXQ readers of the partial tiles are done
-          lds_store_partial(s_Pw, pz, c, h);
-#pragma unroll
-          for (int cb = 0; cb < 2; cb++) {
-            const float a = half_sum(de1[cb]), b = half_sum(de3[cb]);
-            if (h == 0) {
-              s_deta[(0 * 4 + w) * CS + 32 * cb + c] = a;
-              s_deta[(1 * 4 + w) * CS + 32 * cb + c] = b;
+            for (int jj = 0; jj < 8; jj++) {
+              float g, a, b;
+              gelu_fdd((float)zimg.v[cb][s][jj], g, a, b);
+              const float r0 = R.b[s >> 1][cb][8 * (s & 1) + jj], sv = S.b[s >> 1][cb][8 * (s & 1) + jj];
+              const float gz1 = r0 * a;                                   // dl/dZ1
+              de3[cb] = __builtin_fmaf(gz1, sv, de3[cb]);
+              x2c[s][jj] = (bf16)g;
+              uc[s][jj] = (bf16)(sv * a);
+              g1c[s][jj] = (bf16)(-eta_cb[cb] * gz1);
+              d1p.v[cb][s][jj] = (bf16)a;
+              t2p.v[cb][s][jj] = (bf16)(-eta_cb[cb] * r0 * sv * b);
             }
+#pragma unroll
+          for (int s = 0; s < 4; s++) store_piece_rows<LDB>(T0, cb, s, c, h, x2c[s]);   // X2 rows [tok][hid]
+          // pz[:, cb] = gW2^T X2^T ; dEta partial ; + W2^T u^T.   dk[:, cb] = gW1 G1^T
+#pragma unroll
+          for (int s = 0; s < 4; s++)
+#pragma unroll
+            for (int rb = 0; rb < 2; rb++) pz.b[rb][cb] = MFMA(piece_state(gW2s, rb, s), x2c[s], pz.b[rb][cb]);
+#pragma unroll
+          for (int s = 0; s < 4; s++) {
+            const bf16x8 gzv = piece_rows<LDB>(s_gz2, cb, s, c, h);
+#pragma unroll
+            for (int jj = 0; jj < 8; jj++)
+              de1[cb] = __builtin_fmaf((float)gzv[jj], pz.b[s >> 1][cb][8 * (s & 1) + jj], de1[cb]);
           }
+#pragma unroll
+          for (int s = 0; s < 4; s++)
+#pragma unroll
+            for (int rb = 0; rb < 2; rb++) {
+              pz.b[rb][cb] = MFMA(piece_tr<LDT>(T1, rb, s, lane), uc[s], pz.b[rb][cb]);
+              dk.b[rb][cb] = MFMA(piece_tr<LDT>(T2, rb, s, lane), g1c[s], dk.b[rb][cb]);
+            }
         }
-        // park -eta * uQ in the bounce tile; it is read back transposed after the LayerNorm stage
-        {
-          Opd uh;
+        WAVE_SYNC();   // readers of T1 / T2 done
+        lds_store_partial(s_Pw, pz, c, h);
+        // nothing stays in registers across the LayerNorm stage: park d1p, t2p and dk (L2-resident,
+        // rewritten every mini-batch; 1 KiB per wave instruction)
+        opd_store(park_d1, d1p, tid);
+        opd_store(park_t2, t2p, tid);
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
 #pragma unroll
           for (int cb = 0; cb < 2; cb++)
 #pragma unroll
-            for (int s = 0; s < 4; s++)
+            for (int g = 0; g < 4; g++) {
+              f32x4 v = {dk.b[rb][cb][4 * g], dk.b[rb][cb][4 * g + 1], dk.b[rb][cb][4 * g + 2], dk.b[rb][cb][4 * g + 3]};
+              reinterpret_cast<f32x4*>(park_dk)[((rb * 2 + cb) * 4 + g) * 64 + lane] = v;
+            }
 #pragma unroll
-              for (int jj = 0; jj < 8; jj++) uh.v[cb][s][jj] = (bf16)(-eta_cb[cb] * (float)uQ.v[cb][s][jj]);
-          WAVE_SYNC();
-          lds_store_rows_kappa(s_bnc, uh, c, h);
+        for (int cb = 0; cb < 2; cb++) {
+          const float a = half_sum(de1[cb]), b = half_sum(de3[cb]);
+          if (h == 0) {
+            s_deta[(0 * 4 + w) * CS + 32 * cb + c] = a;
+            s_deta[(1 * 4 + w) * CS + 32 * cb + c] = b;
+          }
         }
       }
       __syncthreads();  // all partial ggZ2 tiles and dEta partial sums are in LDS
 
       // ---- second-order pass through the fused LayerNorm loss (LayerNorm lanes)
-      float gy[4][4];
       {
+        float gy[4][4];
         float gg[4][4], xh[4][4], go[4][4], gz[4][4], gam[4][4];
         ln_gather(gg, s_P, s_gb2, tok, fq);
         const float neg_eta = -s_eta[tok];
@@ -800,7 +903,7 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
 #pragma unroll
           for (int e = 0; e < 4; e++) bb = __builtin_fmaf(go[r][e] * gam[r][e], xh[r][e], bb);
         bb = quad_sum(bb);
-        float gx[4][4];
+        float gx[4][4], dg[4][4];
         const float inv = rsd * (1.f / FD);
         float sg = 0.f, sx = 0.f;
 #pragma unroll
@@ -809,14 +912,15 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
           for (int e = 0; e < 4; e++) {
             const float ggx = (gg[r][e] - (s0 + xh[r][e] * a) * (1.f / FD)) * rsd;
             gy[r][e] = gam[r][e] * ggx;
-            dgam[r][e] += go[r][e] * ggx + gy[r][e] * xh[r][e];
-            dbet[r][e] += gy[r][e];
+            dg[r][e] = go[r][e] * ggx + gy[r][e] * xh[r][e];
             gx[r][e] = gy[r][e] * gam[r][e] - (go[r][e] * gam[r][e] * a + gg[r][e] * bb) * inv;
             sg += (-gx[r][e] * xh[r][e] - gg[r][e] * gz[r][e]) * rsd;
             sx += gx[r][e];
           }
         sg = quad_sum(sg);
         sx = quad_sum(sx);
+        ln_token_sum_add(s_dgw, dg, q, fq);
+        ln_token_sum_add(s_dbw, gy, q, fq);
 #pragma unroll
         for (int r = 0; r < 4; r++)
 #pragma unroll
@@ -824,93 +928,100 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
             gx[r][e] = gx[r][e] * rsd + (sg * xh[r][e] - sx * rsd) * (1.f / FD);   // dZ2
             xh[r][e] = -gy[r][e];                                                   // dXV
           }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {   // g_y is needed again for dXK: park it (XQ / E2 tiles are dead by now)
+          f32x4 v = {gy[r][0], gy[r][1], gy[r][2], gy[r][3]};
+          *reinterpret_cast<f32x4*>(s_gy + 16 * r + 4 * fq) = v;
+        }
         ln_store(s_a + tok * LDB, gx, fq);
         ln_accumulate(p.grad_L_XV + xo + tok * FD, xh, fq);
       }
-      __syncthreads();  // dZ2 tile complete; partial tiles free again
+      __syncthreads();  // dZ2 tile complete; partial tiles (T1 / T2) free again
 
       // ---- inner MLP, backwards (uses the state BEFORE this mini-batch)
       {
+        // T2 = gW1 rows [hid][F] (for S again), T1 = gW2 rows [F][hid] (transposed read gives lane = hid)
+        store_state_rows<LDT>(T2, gW1s, c, h);
+        store_state_rows<LDT>(T1, gW2s, c, h);
         WAVE_SYNC();
-        const Opd uP = lds_tr_kappa(s_bnc, lane);          // -eta*u: lane = hid, contraction = tok
-        Opd dz1Q;                                          // lane = tok, contraction = hid
-        {
-          Acc dx2;
-          acc_zero(dx2);
-          {
-            const Opd gw2T = bounce(s_bnc, cvt_chain(gW2s), lane);   // lane = hid, contraction = F
-            const Opd gz2B = lds_rows_kappa(s_gz2, c, h);            // lane = tok, contraction = F
-            mma(dx2, gw2T, gz2B);                                    // P2 = gZ2 gW2^T  (rows hid, lane = tok)
-          }
+        Acc S, dx2;
+        acc_init_rows_lds(S, s_gb1w, h);
+        acc_zero(dx2);
+        mma_jit(S, [&](int blk, int s) { return piece_rows<LDT>(T2, blk, s, c, h); },
+                [&](int blk, int s) { return piece_rows<LDB>(s_xk, blk, s, c, h); });
+        mma_jit(dx2, [&](int blk, int s) { return piece_tr<LDT>(T1, blk, s, lane); },       // gW2: lane = hid, contraction = F
+                [&](int blk, int s) { return piece_rows<LDB>(s_gz2, blk, s, c, h); });      // P2 = gZ2 gW2^T
 #pragma unroll
-          for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-            for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-              for (int i = 0; i < 16; i++) dx2.b[rb][cb][i] *= -eta_cb[cb];
-          {
-            const Opd dz2B = lds_rows_kappa(s_a, c, h);    // lane = tok, contraction = F
-            const Opd w2tA = cvt_chain(W2t);               // W2 before the step
-            mma(dx2, w2tA, dz2B);                          // + dZ2 W2^T
-          }
-          // dZ1 = dX2*gelu' - eta * R * S * gelu''
+        for (int rb = 0; rb < 2; rb++)
 #pragma unroll
           for (int cb = 0; cb < 2; cb++)
 #pragma unroll
-            for (int s = 0; s < 4; s++)
+            for (int i = 0; i < 16; i++) dx2.b[rb][cb][i] *= -eta_cb[cb];
+        {
+          // W2 before the step: lane = hid, contraction = F
+          const Opd w2tA = (j > 0) ? opd_load(p.grad_l_wrt_Z1_group + ho - CS * HID, tid)
+                                   : opd_from_f32_rows(p.W2_ck + slot * HID * FD, FD, 64 * w, 0, c, h);
+          mma_jit(dx2, [&](int blk, int s) { return w2tA.v[blk][s]; },
+                  [&](int blk, int s) { return piece_rows<LDB>(s_a, blk, s, c, h); });      // + dZ2 W2^T
+        }
+        WAVE_SYNC();   // S and P2 have consumed T2 / T1
+        const Opd d1p = opd_load(park_d1, tid);
+        const Opd t2p = opd_load(park_t2, tid);
+        // dZ1 = dX2*gelu' + t2  -> T1 rows [tok][hid];   -eta * S * gelu' -> T2 rows [tok][hid]
 #pragma unroll
-              for (int jj = 0; jj < 8; jj++)
-                dz1Q.v[cb][s][jj] = (bf16)__builtin_fmaf(dx2.b[s >> 1][cb][8 * (s & 1) + jj], (float)d1p.v[cb][s][jj],
-                                                         (float)t2p.v[cb][s][jj]);
-        }
-        {
-          // G1 = -eta * dl/dZ1 exactly as the replay fed it to the weight step (lane = tok)
-          const Opd g1Q = opd_load(p.grad_l_wrt_Z1_group + ho, tid);
-          Acc dk;
-          acc_zero(dk);
-          {
-            const Opd gw1T = bounce(s_bnc, cvt_chain(gW1s), lane);   // lane = F, contraction = hid
-            mma(dk, gw1T, g1Q);                                      // -eta * gZ1 gW1^T   (rows F, lane = tok)
+        for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+          for (int s = 0; s < 4; s++) {
+            bf16x8 dz, uh;
+#pragma unroll
+            for (int jj = 0; jj < 8; jj++) {
+              const float d1v = (float)d1p.v[cb][s][jj];
+              dz[jj] = (bf16)__builtin_fmaf(dx2.b[s >> 1][cb][8 * (s & 1) + jj], d1v, (float)t2p.v[cb][s][jj]);
+              uh[jj] = (bf16)(-eta_cb[cb] * S.b[s >> 1][cb][8 * (s & 1) + jj] * d1v);
+            }
+            store_piece_rows<LDT>(T1, cb, s, c, h, dz);
+            store_piece_rows<LDT>(T2, cb, s, c, h, uh);
           }
-          {
-            // undo the W1 step: W1 before = W1 after - XK^T G1
-            const Opd g1Pn = opd_neg(bounce(s_bnc, g1Q, lane));      // lane = hid, contraction = tok
-            const Opd xkT = lds_tr_kappa(s_xk, lane);                // lane = F,   contraction = tok
-            mma(W1t, g1Pn, xkT);
-          }
-          {
-            const Opd w1tA = cvt_chain(W1t);                         // W1 before the step
-            mma(dk, w1tA, dz1Q);                                     // + dZ1 W1^T
-          }
-          lds_store_partial(s_Pw, dk, c, h);
-        }
+        WAVE_SYNC();
+        Acc dk;
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+          for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+              const f32x4 v = reinterpret_cast<const f32x4*>(park_dk)[((rb * 2 + cb) * 4 + g) * 64 + lane];
+#pragma unroll
+              for (int e = 0; e < 4; e++) dk.b[rb][cb][4 * g + e] = v[e];
+            }
         {
-          const Opd gz2T = lds_tr_kappa(s_gz2, lane);                // lane = F, contraction = tok
-          mma(gW2s, uP, gz2T);
+          // W1 before the step: lane = F, contraction = hid
+          const Opd w1tA = (j > 0) ? opd_load(p.X2_group + ho - CS * HID, tid)
+                                   : opd_from_f32_rows(p.W1_ck + slot * FD * HID, HID, 0, 64 * w, c, h);
+          mma_jit(dk, [&](int blk, int s) { return w1tA.v[blk][s]; },
+                  [&](int blk, int s) { return piece_rows<LDT>(T1, blk, s, c, h); });       // + dZ1 W1^T
         }
-        {
-          const Opd dz2T = lds_tr_kappa(s_a, lane);                  // lane = F, contraction = tok
-          {
-            const Opd x2P = bounce(s_bnc, opd_load(p.X2_group + ho, tid), lane);
-            mma(gW2s, x2P, dz2T);
-          }
-          if (w == 0) lds_rowsum_add(s_gb2, dz2T, ones, c, h);
-        }
-        {
-          const Opd dz1P = bounce(s_bnc, dz1Q, lane);                // lane = hid, contraction = tok
-          const Opd xkT = lds_tr_kappa(s_xk, lane);
-          mma(gW1s, xkT, dz1P);
-          lds_rowsum_add(s_gb1w, dz1P, ones, c, h);
-        }
+        mma_jit(gW2s, [&](int blk, int s) { return piece_tr<LDT>(T2, blk, s, lane); },      // (-eta u)^T: lane = hid
+                [&](int blk, int s) { return piece_tr<LDB>(s_gz2, blk, s, lane); });        // gZ2: lane = F
+        mma_jit(gW2s, [&](int blk, int s) { return piece_tr<LDB>(T0, blk, s, lane); },      // X2^T: lane = hid
+                [&](int blk, int s) { return piece_tr<LDB>(s_a, blk, s, lane); });          // dZ2: lane = F
+        if (w == 0) lds_rowsum_add_jit(s_gb2, [&](int blk, int s) { return piece_tr<LDB>(s_a, blk, s, lane); }, ones, c, h);
+        mma_jit(gW1s, [&](int blk, int s) { return piece_tr<LDB>(s_xk, blk, s, lane); },    // XK^T: lane = F
+                [&](int blk, int s) { return piece_tr<LDT>(T1, blk, s, lane); });           // dZ1: lane = hid
+        lds_rowsum_add_jit(s_gb1w, [&](int blk, int s) { return piece_tr<LDT>(T1, blk, s, lane); }, ones, c, h);
+        WAVE_SYNC();   // readers of T1 / T2 done
+        lds_store_partial(s_Pw, dk, c, h);
       }
       __syncthreads();  // partial dXK tiles complete
       {
         float z[4][4];
         ln_gather0(z, s_P, tok, fq);
 #pragma unroll
-        for (int r = 0; r < 4; r++)
+        for (int r = 0; r < 4; r++) {
+          const f32x4 v = *reinterpret_cast<const f32x4*>(s_gy + 16 * r + 4 * fq);
 #pragma unroll
-          for (int e = 0; e < 4; e++) z[r][e] += gy[r][e];
+          for (int e = 0; e < 4; e++) z[r][e] += v[e];
+        }
         ln_accumulate(p.grad_L_XK + xo + tok * FD, z, fq);
       }
     }
@@ -922,22 +1033,7 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
   __syncthreads();
   p.grad_L_b1_init[(size_t)bh * HID + tid] = s_gb1[tid];
   if (tid < FD) p.grad_L_b2_init[(size_t)bh * FD + tid] = s_gb2[tid];
-  // norm-weight / norm-bias gradients: sum over the 16 tokens of the wave, then over the 4 waves
-#pragma unroll
-  for (int r = 0; r < 4; r++)
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-      float a = dgam[r][e], b = dbet[r][e];
-#pragma unroll
-      for (int m = 4; m < 64; m <<= 1) {
-        a += __shfl_xor(a, m, 64);
-        b += __shfl_xor(b, m, 64);
-      }
-      if (q == 0) {
-        s_red[(w * 2 + 0) * FD + 16 * r + 4 * fq + e] = a;
-        s_red[(w * 2 + 1) * FD + 16 * r + 4 * fq + e] = b;
-      }
-    }
+  // norm-weight / norm-bias gradients: sum the per-wave LDS accumulators
   __syncthreads();
   if (tid < 2 * FD) {
     const int which = tid / FD, f = tid % FD;
