@@ -443,6 +443,34 @@ TTT_DEV Opd opd_from_f32_rows(const float* g, int ld, int r0, int c0, int c, int
   return o;
 }
 
+// Three [64][64] bf16 tiles + the eta vector of one mini-batch in flight from HBM (per thread).
+struct Staged3 {
+  u32x4 a[2], b[2], c[2];
+  float eta;
+};
+TTT_DEV void stage3_load(Staged3& s, const bf16* ga, const bf16* gb, const bf16* gc, const bf16* geta, size_t tile_off,
+                         size_t eta_off, int tid) {
+#pragma unroll
+  for (int r = 0; r < 2; r++) {
+    const int id = tid + 256 * r;
+    s.a[r] = reinterpret_cast<const u32x4*>(ga + tile_off)[id];
+    s.b[r] = reinterpret_cast<const u32x4*>(gb + tile_off)[id];
+    s.c[r] = reinterpret_cast<const u32x4*>(gc + tile_off)[id];
+  }
+  s.eta = (tid < CS) ? bf2f(geta[eta_off + tid]) : 0.f;
+}
+TTT_DEV void stage3_store(const Staged3& s, bf16* sa, bf16* sb, bf16* sc, float* s_eta, int tid) {
+#pragma unroll
+  for (int r = 0; r < 2; r++) {
+    const int id = tid + 256 * r;
+    const int off = (id >> 3) * LDB + (id & 7) * 8;
+    *reinterpret_cast<u32x4*>(sa + off) = s.a[r];
+    *reinterpret_cast<u32x4*>(sb + off) = s.b[r];
+    *reinterpret_cast<u32x4*>(sc + off) = s.c[r];
+  }
+  if (tid < CS) s_eta[tid] = s.eta;
+}
+
 __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   bf16* s_xq = reinterpret_cast<bf16*>(smem + SB_XQ);
@@ -520,46 +548,48 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
       s_b1[tid] = p.b1_ck[slot * HID + tid];
       if (tid < FD) s_b2[tid] = p.b2_ck[slot * FD + tid];
 
+      bf16* const T0 = s_bnc;                                   // wave-private tiles, as in the reverse walk
+      bf16* const T1 = reinterpret_cast<bf16*>(s_Pw);
+      bf16* const T2 = T1 + 64 * LDT;
+      Staged3 st;
+      stage3_load(st, p.XQ, p.XK, p.XV, p.last_eta, x_base + (size_t)(k * cgs) * (CS * FD), eta_base + (size_t)(k * cgs) * CS, tid);
       for (int j = 0; j < n_mb; j++) {
         const int mb = k * cgs + j;
-        const size_t xo = x_base + (size_t)mb * (CS * FD);
         __syncthreads();
-        stage_tile(s_xq, p.XQ + xo, tid);
-        stage_tile(s_xk, p.XK + xo, tid);
-        stage_tile(s_e2, p.XV + xo, tid);
-        if (tid < CS) s_eta[tid] = bf2f(p.last_eta[eta_base + (size_t)mb * CS + tid]);
+        stage3_store(st, s_xq, s_xk, s_e2, s_eta, tid);
         __syncthreads();
 
-        // Z1^T = W1s^T XK^T + b1  (rows hid, lane = tok)
-        Acc d1;
-        Opd x2Q;  // lane = tok, contraction = hid
+        // Z1^T = W1s^T XK^T + b1  (rows hid, lane = tok); X2 rows [tok][hid] -> T0, gelu'(Z1) packed
+        Opd d1p;
         {
           Acc x2;
           acc_init_rows_lds(x2, s_b1w, h);
-          {
-            const Opd w1A = cvt_chain(W1s);
-            const Opd xkB = lds_rows_kappa(s_xk, c, h);
-            mma(x2, w1A, xkB);
-          }
-          img_store(p.Z1_group + g_TH + (size_t)j * (CS * HID), x2, tid);
+          mma_jit(x2, [&](int blk, int s) { return piece_state(W1s, blk, s); },
+                  [&](int blk, int s) { return piece_rows<LDB>(s_xk, blk, s, c, h); });
+          bf16* img = p.Z1_group + g_TH + (size_t)j * (CS * HID);
 #pragma unroll
-          for (int rb = 0; rb < 2; rb++)
+          for (int cb = 0; cb < 2; cb++)
 #pragma unroll
-            for (int cb = 0; cb < 2; cb++)
+            for (int s = 0; s < 4; s++) {
+              const bf16x8 z = pack8(x2.b[s >> 1][cb], s & 1);
+              reinterpret_cast<bf16x8*>(img)[(cb * 4 + s) * NTHREADS + tid] = z;
+              bf16x8 xv;
 #pragma unroll
-              for (int i = 0; i < 16; i++) {
+              for (int jj = 0; jj < 8; jj++) {
                 float g, d;
-                gelu_fd(x2.b[rb][cb][i], g, d);
-                x2.b[rb][cb][i] = g;
-                d1.b[rb][cb][i] = d;
+                gelu_fd(x2.b[s >> 1][cb][8 * (s & 1) + jj], g, d);
+                xv[jj] = (bf16)g;
+                d1p.v[cb][s][jj] = (bf16)d;
               }
-          x2Q = cvt_chain(x2);
+              store_piece_rows<LDB>(T0, cb, s, c, h, xv);
+            }
         }
+        WAVE_SYNC();
         {
-          const Opd w2A = cvt_chain(W2s);
           Acc z2;
           acc_zero(z2);
-          mma(z2, w2A, x2Q);
+          mma_jit(z2, [&](int blk, int s) { return piece_state(W2s, blk, s); },                  // lane = F, contraction = hid
+                  [&](int blk, int s) { return piece_rows<LDB>(T0, blk, s, c, h); });            // X2: lane = tok
           lds_store_partial(s_Pw, z2, c, h);
         }
         __syncthreads();
@@ -602,65 +632,72 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
           if (fq == 0) p.std_fused_group[g_T + (size_t)j * CS + tok] = sd;
         }
         __syncthreads();
-        // G1 = (W2 G2^T) * gelu'(Z1)  (rows hid, lane = tok); weight step
+        // G1 = (W2 G2^T) * gelu'(Z1)  (rows hid, lane = tok) -> T1 rows [tok][hid]; weight step
         {
-          Opd g1Q;
-          {
-            Acc g1;
-            acc_zero(g1);
-            {
-              const Opd g2B = lds_rows_kappa(s_gz2, c, h);   // lane = tok, contraction = F
-              const Opd w2tA = cvt_chain(W2t);               // lane = hid, contraction = F
-              mma(g1, w2tA, g2B);
+          Acc g1;
+          acc_zero(g1);
+          mma_jit(g1, [&](int blk, int s) { return piece_state(W2t, blk, s); },                  // lane = hid, contraction = F
+                  [&](int blk, int s) { return piece_rows<LDB>(s_gz2, blk, s, c, h); });         // G2: lane = tok
+#pragma unroll
+          for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+              bf16x8 gv;
+#pragma unroll
+              for (int jj = 0; jj < 8; jj++) gv[jj] = (bf16)(g1.b[s >> 1][cb][8 * (s & 1) + jj] * (float)d1p.v[cb][s][jj]);
+              store_piece_rows<LDT>(T1, cb, s, c, h, gv);
             }
-#pragma unroll
-            for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-              for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) g1.b[rb][cb][i] *= d1.b[rb][cb][i];
-            g1Q = cvt_chain(g1);
-          }
-          {
-            const Opd g2T = lds_tr_kappa(s_gz2, lane);       // lane = F, contraction = tok
-            const Opd x2P = bounce(s_bnc, x2Q, lane);        // lane = hid, contraction = tok
-            mma(W2s, x2P, g2T);
-            mma(W2t, g2T, x2P);
-            if (w == 0) lds_rowsum_add(s_b2, g2T, ones, c, h);
-          }
-          {
-            const Opd g1P = bounce(s_bnc, g1Q, lane);
-            const Opd xkT = lds_tr_kappa(s_xk, lane);        // lane = F, contraction = tok
-            mma(W1s, xkT, g1P);
-            lds_rowsum_add(s_b1w, g1P, ones, c, h);
-          }
         }
+        WAVE_SYNC();
+        mma_jit(W2s, [&](int blk, int s) { return piece_tr<LDB>(T0, blk, s, lane); },            // X2^T: lane = hid
+                [&](int blk, int s) { return piece_tr<LDB>(s_gz2, blk, s, lane); });             // G2: lane = F
+        mma_jit(W2t, [&](int blk, int s) { return piece_tr<LDB>(s_gz2, blk, s, lane); },
+                [&](int blk, int s) { return piece_tr<LDB>(T0, blk, s, lane); });
+        if (w == 0) lds_rowsum_add_jit(s_b2, [&](int blk, int s) { return piece_tr<LDB>(s_gz2, blk, s, lane); }, ones, c, h);
+        mma_jit(W1s, [&](int blk, int s) { return piece_tr<LDB>(s_xk, blk, s, lane); },          // XK^T: lane = F
+                [&](int blk, int s) { return piece_tr<LDT>(T1, blk, s, lane); });                // G1: lane = hid
+        lds_rowsum_add_jit(s_b1w, [&](int blk, int s) { return piece_tr<LDT>(T1, blk, s, lane); }, ones, c, h);
         // operand images of the state after this step, for the reverse walk
-        opd_store(p.grad_l_wrt_Z1_group + g_TH + (size_t)j * (CS * HID), cvt_chain(W2t), tid);   // lane = hid, contraction = F
+        {
+          bf16* img2 = p.grad_l_wrt_Z1_group + g_TH + (size_t)j * (CS * HID);   // W2: lane = hid, contraction = F
+          bf16* img1 = p.X2_group + g_TH + (size_t)j * (CS * HID);              // W1^T: lane = F, contraction = hid
+          store_state_rows<LDT>(T2, W1s, c, h);                                 // rows [hid][F]
+#pragma unroll
+          for (int fb = 0; fb < 2; fb++)
+#pragma unroll
+            for (int s = 0; s < 4; s++) reinterpret_cast<bf16x8*>(img2)[(fb * 4 + s) * NTHREADS + tid] = piece_state(W2t, fb, s);
+          WAVE_SYNC();
+#pragma unroll
+          for (int fb = 0; fb < 2; fb++)
+#pragma unroll
+            for (int s = 0; s < 4; s++) reinterpret_cast<bf16x8*>(img1)[(fb * 4 + s) * NTHREADS + tid] = piece_tr<LDT>(T2, fb, s, lane);
+        }
         // post-update forward on XQ
         {
           Acc z1b;
           acc_init_rows_lds(z1b, s_b1w, h);
-          {
-            const Opd w1A = cvt_chain(W1s);
-            opd_store(p.X2_group + g_TH + (size_t)j * (CS * HID), bounce(s_bnc, w1A, lane), tid);   // lane = F, contraction = hid
-            const Opd xqB = lds_rows_kappa(s_xq, c, h);
-            mma(z1b, w1A, xqB);
-          }
-          img_store(p.Z1_bar_group + g_TH + (size_t)j * (CS * HID), z1b, tid);
+          mma_jit(z1b, [&](int blk, int s) { return piece_state(W1s, blk, s); },
+                  [&](int blk, int s) { return piece_rows<LDB>(s_xq, blk, s, c, h); });
+          bf16* img = p.Z1_bar_group + g_TH + (size_t)j * (CS * HID);
+          Opd x2bQ;
 #pragma unroll
-          for (int rb = 0; rb < 2; rb++)
+          for (int cb = 0; cb < 2; cb++)
 #pragma unroll
-            for (int cb = 0; cb < 2; cb++)
+            for (int s = 0; s < 4; s++) {
+              reinterpret_cast<bf16x8*>(img)[(cb * 4 + s) * NTHREADS + tid] = pack8(z1b.b[s >> 1][cb], s & 1);
 #pragma unroll
-              for (int i = 0; i < 16; i++) z1b.b[rb][cb][i] = gelu_f(z1b.b[rb][cb][i]);
-          const Opd x2bQ = cvt_chain(z1b);
-          const Opd w2A = cvt_chain(W2s);
+              for (int jj = 0; jj < 8; jj++) x2bQ.v[cb][s][jj] = (bf16)gelu_f(z1b.b[s >> 1][cb][8 * (s & 1) + jj]);
+            }
           Acc z2;
           acc_zero(z2);
-          mma(z2, w2A, x2bQ);
+          mma_jit(z2, [&](int blk, int s) { return piece_state(W2s, blk, s); },
+                  [&](int blk, int s) { return x2bQ.v[blk][s]; });
+          WAVE_SYNC();   // readers of T1 / T2 are done
           lds_store_partial(s_Pw, z2, c, h);
         }
+        // inputs of the next mini-batch travel while the last LayerNorm stage runs
+        if (j + 1 < n_mb)
+          stage3_load(st, p.XQ, p.XK, p.XV, p.last_eta, x_base + (size_t)(mb + 1) * (CS * FD), eta_base + (size_t)(mb + 1) * CS, tid);
         __syncthreads();
         {
           float z[4][4];
@@ -783,7 +820,6 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
       //      Survive the LayerNorm stage: X2 in T0; packed d1p = gelu'(Z1) and
       //      t2p = -eta * (gZ2 W2^T) * (XK gW1 + gb1) * gelu''(Z1); the accumulator dk.
       {
-        Opd d1p, t2p;
         Acc dk;
         // T1 = W2 before the step, rows [hid][F]; T2 = gW1, rows [hid][F]
         store_opd_rows<LDT>(T1, (j > 0) ? opd_load(p.grad_l_wrt_Z1_group + ho - CS * HID, tid)
@@ -806,7 +842,8 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
         for (int cb = 0; cb < 2; cb++) {
           bf16x8 x2c[4], uc[4], g1c[4];
 #pragma unroll
-          for (int s = 0; s < 4; s++)
+          for (int s = 0; s < 4; s++) {
+            bf16x8 d1c, t2c;
 #pragma unroll
             for (int jj = 0; jj < 8; jj++) {
               float g, a, b;
@@ -817,9 +854,14 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
               x2c[s][jj] = (bf16)g;
               uc[s][jj] = (bf16)(sv * a);
               g1c[s][jj] = (bf16)(-eta_cb[cb] * gz1);
-              d1p.v[cb][s][jj] = (bf16)a;
-              t2p.v[cb][s][jj] = (bf16)(-eta_cb[cb] * r0 * sv * b);
+              d1c[jj] = (bf16)a;
+              t2c[jj] = (bf16)(-eta_cb[cb] * r0 * sv * b);
             }
+            // nothing stays in registers across the LayerNorm stage: d1 and t2 go to their park at once
+            // (L2-resident, rewritten every mini-batch; 1 KiB per wave instruction)
+            reinterpret_cast<bf16x8*>(park_d1)[(cb * 4 + s) * NTHREADS + tid] = d1c;
+            reinterpret_cast<bf16x8*>(park_t2)[(cb * 4 + s) * NTHREADS + tid] = t2c;
+          }
 #pragma unroll
           for (int s = 0; s < 4; s++) store_piece_rows<LDB>(T0, cb, s, c, h, x2c[s]);   // X2 rows [tok][hid]
           // pz[:, cb] = gW2^T X2^T ; dEta partial ; + W2^T u^T.   dk[:, cb] = gW1 G1^T
@@ -844,10 +886,7 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
         }
         WAVE_SYNC();   // readers of T1 / T2 done
         lds_store_partial(s_Pw, pz, c, h);
-        // nothing stays in registers across the LayerNorm stage: park d1p, t2p and dk (L2-resident,
-        // rewritten every mini-batch; 1 KiB per wave instruction)
-        opd_store(park_d1, d1p, tid);
-        opd_store(park_t2, t2p, tid);
+        // the accumulator dk is parked too
 #pragma unroll
         for (int rb = 0; rb < 2; rb++)
 #pragma unroll
