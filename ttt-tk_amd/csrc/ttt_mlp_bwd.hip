@@ -1085,6 +1085,7 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
 
 }  // namespace ttt
 
+extern "C" int ttt_mlp_bwd_threads() { return ttt::NTHREADS; }
 extern "C" int ttt_mlp_bwd_lds_bytes() { return ttt::SM_BWD_BYTES; }
 
 hipError_t ttt_mlp_bwd_enqueue(const ttt::BwdParams& p, hipStream_t stream) {

@@ -104,8 +104,7 @@ extern "C" int ttt_mlp_bwd_launch(const ttt_mlp_bwd_args* a, void* stream) {
 
 extern "C" int ttt_mlp_kernel_info(int which, int* lds_bytes, int* threads_per_workgroup) {
   if (lds_bytes == nullptr || threads_per_workgroup == nullptr) return TTT_MLP_ERR_BAD_ARG;
-  *threads_per_workgroup = 256;
-  if (which == 0) { *lds_bytes = ttt_mlp_fwd_lds_bytes(); return TTT_MLP_OK; }
-  if (which == 1) { *lds_bytes = ttt_mlp_bwd_lds_bytes(); return TTT_MLP_OK; }
+  if (which == 0) { *lds_bytes = ttt_mlp_fwd_lds_bytes(); *threads_per_workgroup = ttt_mlp_fwd_threads(); return TTT_MLP_OK; }
+  if (which == 1) { *lds_bytes = ttt_mlp_bwd_lds_bytes(); *threads_per_workgroup = ttt_mlp_bwd_threads(); return TTT_MLP_OK; }
   return TTT_MLP_ERR_BAD_ARG;
 }

@@ -162,6 +162,102 @@ TTT_DEV float quad_sum(float x) {
 // Sum of lane l and lane l^32, result in both.
 TTT_DEV float half_sum(float x) { return x + __shfl_xor(x, 32, 64); }
 
+// ---------------------------------------------------------------------------- shape-generic tiles
+// Tiles whose extent along the hidden dimension is one 32-wide block (a wave that owns 32 hidden
+// columns) mix with 64-wide token / feature extents, so blocks and k-steps are template parameters.
+template <int RB, int CB> struct AccT { f32x16 b[RB][CB]; };   // (32 RB) x (32 CB) fp32 tile
+template <int FB, int KS> struct OpdT { bf16x8 v[FB][KS]; };   // free index 32 FB, contraction 16 KS
+
+template <int RB, int CB>
+TTT_DEV void acc_zero(AccT<RB, CB>& a) {
+#pragma unroll
+  for (int r = 0; r < RB; r++)
+#pragma unroll
+    for (int c = 0; c < CB; c++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) a.b[r][c][i] = 0.f;
+}
+
+template <int RB, int CB, int KS>
+TTT_DEV void mma(AccT<RB, CB>& d, const OpdT<RB, KS>& a, const OpdT<CB, KS>& b) {
+#pragma unroll
+  for (int s = 0; s < KS; s++)
+#pragma unroll
+    for (int r = 0; r < RB; r++)
+#pragma unroll
+      for (int c = 0; c < CB; c++)
+        d.b[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v[r][s], b.v[c][s], d.b[r][c], 0, 0, 0);
+}
+
+// Accumulator tile (rows = contraction index) -> chained operand, contraction in kappa order.
+template <int RB, int CB>
+TTT_DEV OpdT<CB, 2 * RB> cvt_chain(const AccT<RB, CB>& x) {
+  OpdT<CB, 2 * RB> o;
+#pragma unroll
+  for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+      for (int t = 0; t < 2; t++) o.v[cb][2 * rb + t] = pack8(x.b[rb][cb], t);
+  return o;
+}
+
+// Operand from an LDS tile stored [free index][contraction index], row stride ld elements.
+template <int FB, int KS>
+TTT_DEV OpdT<FB, KS> lds_rows_kappa(const bf16* base, int ld, int c, int h) {
+  OpdT<FB, KS> o;
+#pragma unroll
+  for (int fb = 0; fb < FB; fb++)
+#pragma unroll
+    for (int s = 0; s < KS; s++) {
+      const bf16* p = base + (32 * fb + c) * ld + 16 * s + 4 * h;
+      o.v[fb][s] = cat(*reinterpret_cast<const bf16x4*>(p), *reinterpret_cast<const bf16x4*>(p + 8));
+    }
+  return o;
+}
+
+// Operand from an LDS tile stored [contraction index][free index] through the transposing read.
+template <int FB, int KS>
+TTT_DEV OpdT<FB, KS> lds_tr_kappa(const bf16* base, int ld, int lane) {
+  OpdT<FB, KS> o;
+  const int h = lane >> 5, c = lane & 31, i = lane & 15;
+#pragma unroll
+  for (int fb = 0; fb < FB; fb++)
+#pragma unroll
+    for (int s = 0; s < KS; s++) {
+      const bf16* p = base + (16 * s + 4 * h + (i >> 2)) * ld + 32 * fb + 16 * (c >> 4) + 4 * (i & 3);
+      o.v[fb][s] = cat(lds_tr4(p), lds_tr4(p + 8 * ld));
+    }
+  return o;
+}
+
+// Inverse of lds_rows_kappa: writes an operand as an LDS tile stored [free index][contraction index].
+template <int FB, int KS>
+TTT_DEV void lds_store_rows_kappa(bf16* base, int ld, const OpdT<FB, KS>& o, int c, int h) {
+#pragma unroll
+  for (int fb = 0; fb < FB; fb++)
+#pragma unroll
+    for (int s = 0; s < KS; s++) {
+      bf16* p = base + (32 * fb + c) * ld + 16 * s + 4 * h;
+      *reinterpret_cast<bf16x4*>(p) = __builtin_shufflevector(o.v[fb][s], o.v[fb][s], 0, 1, 2, 3);
+      *reinterpret_cast<bf16x4*>(p + 8) = __builtin_shufflevector(o.v[fb][s], o.v[fb][s], 4, 5, 6, 7);
+    }
+}
+
+// Sum over an aligned group of 8 lanes, result in all 8.
+TTT_DEV float oct_sum(float x) {
+  x = quad_sum(x);
+  return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x141, 0xF, 0xF, false));
+}
+
+// Orders this wave's LDS traffic: everything issued before is complete and nothing after is hoisted.
+#define TTT_WAVE_SYNC()                                     \
+  do {                                                      \
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); \
+    __builtin_amdgcn_wave_barrier();                        \
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront"); \
+  } while (0)
+
 // ---------------------------------------------------------------------------- bf16 helpers
 TTT_DEV float bf_lo(uint32_t u) { return __builtin_bit_cast(float, u << 16); }
 TTT_DEV float bf_hi(uint32_t u) { return __builtin_bit_cast(float, u & 0xffff0000u); }

@@ -5,112 +5,141 @@
 // (W1,b1,W2,b2) is carried through NC mini-batches of 64 tokens; before mini-batch i with
 // i % checkpoint_group_size == 0 the state is stored at checkpoint slot i / checkpoint_group_size.
 //
-// Mapping: one workgroup of 4 wavefronts per (batch, head); wave w owns hidden columns
-// [64w, 64w+64).  The state lives in registers for the whole scan as MFMA accumulator tiles:
+// Mapping: one workgroup of 8 wavefronts (two per SIMD, at most 256 registers each) per (batch,
+// head); wave v owns hidden columns [32v, 32v+32).  The state lives in registers for the whole scan
+// as MFMA accumulator tiles:
 //   W1s = W1[:, shard]      (rows F,   columns hid)  -> chained operand of XK*W1 and of (XQ*W1)^T
 //   W2s = W2[shard, :]      (rows hid, columns F)    -> chained operand of (X2*W2)^T
 //   W2t = W2[shard, :]^T    (rows F,   columns hid)  -> chained operand of gZ2*W2^T
 // so no weight ever goes through LDS; the eta-scaled updates are MFMA accumulations into them.
-// Cross-shard sums of Z2 go through fp32 LDS tiles; each wave then LayerNorms 16 of the 64 tokens
-// with 4 lanes per token.
+// Sums over the hidden dimension (Z2) are formed in two steps: waves v and v+4 exchange halves of
+// their partial tiles through LDS and each finishes one half, then every wave LayerNorms 8 of the
+// 64 tokens (8 lanes per token) from the four pair sums.  All sums have a fixed order.
 #include "ttt_mlp_common.hpp"
 #include "ttt_mlp_kernels.hpp"
 
 namespace ttt {
 
+constexpr int FW_NWAVE = 8;
+constexpr int FW_THREADS = 64 * FW_NWAVE;
+constexpr int FW_NS = HID / FW_NWAVE;                  // hidden columns per wave: 32
+
 // LDS carve-up (bytes)
 constexpr int SM_TILE = 64 * LDB * 2;                   // one bf16 tile: 9216
-constexpr int SM_XQ = 0;
-constexpr int SM_XK = SM_XQ + SM_TILE;
+constexpr int SM_XQ = 0;                                // two buffers, alternating per mini-batch
+constexpr int SM_XK = SM_XQ + 2 * SM_TILE;
 constexpr int SM_XV = SM_XK + SM_TILE;
 constexpr int SM_G2 = SM_XV + SM_TILE;
-constexpr int SM_P = SM_G2 + SM_TILE;                    // 4 fp32 partial tiles; wave w's tile doubles
-constexpr int SM_PTILE = 64 * LDP * 4;                   // as its bf16 X2 transposition buffer
-constexpr int SM_B1 = SM_P + 4 * SM_PTILE;
+constexpr int SM_P = SM_G2 + SM_TILE;                    // 4 fp32 pair-sum tiles [tok][F]
+constexpr int SM_PTILE = 64 * LDP * 4;
+constexpr int SM_X2T = SM_P + 4 * SM_PTILE;             // per wave: X2 shard stored [hid][tok], bf16
+constexpr int SM_X2T_TILE = FW_NS * LDB * 2;
+constexpr int SM_B1 = SM_X2T + FW_NWAVE * SM_X2T_TILE;
 constexpr int SM_B2 = SM_B1 + HID * 4;
 constexpr int SM_ETA = SM_B2 + FD * 4;
-constexpr int SM_FWD_BYTES = SM_ETA + CS * 4;
+constexpr int SM_GAM = SM_ETA + CS * 4;
+constexpr int SM_BET = SM_GAM + FD * 4;
+constexpr int SM_FWD_BYTES = SM_BET + FD * 4;
+static_assert(SM_FWD_BYTES <= 160 * 1024, "forward LDS budget");
 
-struct Staged {  // one mini-batch of inputs in flight from HBM (per thread)
-  u32x4 q[2], k[2], v[2];
+struct Staged {  // one mini-batch of inputs in flight from HBM: one 16-byte chunk per tile per thread
+  u32x4 q, k, v;
   float eta;
 };
 
 TTT_DEV void stage_load(Staged& s, const FwdParams& p, size_t tile_off, size_t eta_off, int tid) {
-#pragma unroll
-  for (int r = 0; r < 2; r++) {
-    const int id = tid + 256 * r;  // 16-byte chunk id: row = id / 8, 8 chunks per 128-byte row
-    s.q[r] = reinterpret_cast<const u32x4*>(p.XQ + tile_off)[id];
-    s.k[r] = reinterpret_cast<const u32x4*>(p.XK + tile_off)[id];
-    s.v[r] = reinterpret_cast<const u32x4*>(p.XV + tile_off)[id];
-  }
+  s.q = reinterpret_cast<const u32x4*>(p.XQ + tile_off)[tid];   // chunk id = tid: row tid / 8, 8 chunks per row
+  s.k = reinterpret_cast<const u32x4*>(p.XK + tile_off)[tid];
+  s.v = reinterpret_cast<const u32x4*>(p.XV + tile_off)[tid];
   s.eta = (tid < CS) ? bf2f(p.last_eta[eta_off + tid]) : 0.f;
 }
 
-TTT_DEV void stage_store(const Staged& s, unsigned char* smem, int tid) {
-#pragma unroll
-  for (int r = 0; r < 2; r++) {
-    const int id = tid + 256 * r;
-    const int off = ((id >> 3) * LDB + (id & 7) * 8) * 2;
-    *reinterpret_cast<u32x4*>(smem + SM_XQ + off) = s.q[r];
-    *reinterpret_cast<u32x4*>(smem + SM_XK + off) = s.k[r];
-    *reinterpret_cast<u32x4*>(smem + SM_XV + off) = s.v[r];
-  }
+TTT_DEV void stage_store(const Staged& s, unsigned char* smem, int xq_buf, int tid) {
+  const int off = ((tid >> 3) * LDB + (tid & 7) * 8) * 2;
+  *reinterpret_cast<u32x4*>(smem + SM_XQ + xq_buf * SM_TILE + off) = s.q;
+  *reinterpret_cast<u32x4*>(smem + SM_XK + off) = s.k;
+  *reinterpret_cast<u32x4*>(smem + SM_XV + off) = s.v;
   if (tid < CS) reinterpret_cast<float*>(smem + SM_ETA)[tid] = s.eta;
 }
 
-__global__ __launch_bounds__(NTHREADS) void ttt_mlp_fwd_kernel(const FwdParams p) {
+// Two-step sum over the wave pair (v, v ^ 4) of a partial tile z (rows F, columns tok): the wave
+// with pair index r gives away row block 1-r, then adds the partner's row block r to its own and
+// leaves the pair sum in the pair's LDS tile, stored [tok][F].  Contains two workgroup barriers.
+template <int R>
+TTT_DEV void pair_give(float* tile, const AccT<2, 2>& z, int c, int h) {
+#pragma unroll
+  for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      const f32x16& x = z.b[1 - R][cb];
+      f32x4 v = {x[4 * g], x[4 * g + 1], x[4 * g + 2], x[4 * g + 3]};
+      *reinterpret_cast<f32x4*>(tile + (32 * cb + c) * LDP + 32 * (1 - R) + 8 * g + 4 * h) = v;
+    }
+}
+template <int R>
+TTT_DEV void pair_take(float* tile, const AccT<2, 2>& z, int c, int h) {
+#pragma unroll
+  for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      float* q = tile + (32 * cb + c) * LDP + 32 * R + 8 * g + 4 * h;
+      const f32x16& x = z.b[R][cb];
+      f32x4 v = *reinterpret_cast<const f32x4*>(q);
+      v[0] += x[4 * g]; v[1] += x[4 * g + 1]; v[2] += x[4 * g + 2]; v[3] += x[4 * g + 3];
+      *reinterpret_cast<f32x4*>(q) = v;
+    }
+}
+TTT_DEV void pair_sum_to_lds(float* tile, const AccT<2, 2>& z, int r, int c, int h) {
+  if (r == 0) pair_give<0>(tile, z, c, h); else pair_give<1>(tile, z, c, h);
+  __syncthreads();
+  if (r == 0) pair_take<0>(tile, z, c, h); else pair_take<1>(tile, z, c, h);
+  __syncthreads();
+}
+
+__global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  bf16* s_xq = reinterpret_cast<bf16*>(smem + SM_XQ);
-  bf16* s_xk = reinterpret_cast<bf16*>(smem + SM_XK);
-  bf16* s_xv = reinterpret_cast<bf16*>(smem + SM_XV);
+  const bf16* s_xk = reinterpret_cast<const bf16*>(smem + SM_XK);
+  const bf16* s_xv = reinterpret_cast<const bf16*>(smem + SM_XV);
   bf16* s_g2 = reinterpret_cast<bf16*>(smem + SM_G2);
   float* s_P = reinterpret_cast<float*>(smem + SM_P);
   float* s_b1 = reinterpret_cast<float*>(smem + SM_B1);
   float* s_b2 = reinterpret_cast<float*>(smem + SM_B2);
   const float* s_eta = reinterpret_cast<const float*>(smem + SM_ETA);
+  float* s_gam = reinterpret_cast<float*>(smem + SM_GAM);
+  float* s_bet = reinterpret_cast<float*>(smem + SM_BET);
 
-  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, h = lane >> 5, c = lane & 31;
-  const int q = lane >> 2, fq = lane & 3, tok = 16 * w + q;  // LayerNorm ownership: 4 lanes per token
+  const int tid = threadIdx.x, v = tid >> 6, lane = tid & 63, h = lane >> 5, c = lane & 31;
+  const int pr = v >> 2;                                    // index inside the wave pair (v & 3)
+  const int tok = 8 * v + (lane >> 3), f0 = 8 * (lane & 7); // LayerNorm ownership: 8 lanes per token, 8 features each
   const int bh = blockIdx.x, head = bh % p.NH;
-  float* s_Pw = s_P + w * 64 * LDP;
-  bf16* s_x2t = reinterpret_cast<bf16*>(s_Pw);
+  const int hid0 = FW_NS * v;
+  float* s_Pp = s_P + (v & 3) * 64 * LDP;
+  bf16* s_x2t = reinterpret_cast<bf16*>(smem + SM_X2T + v * SM_X2T_TILE);
 
   // ---- state -> registers
-  Acc W1s, W2s, W2t;
-  float b1L[2];
-  f32x16 b2acc[2];
+  AccT<2, 1> W1s, W2t;
+  AccT<1, 2> W2s;
+  float b1L;      // b1 of hidden column hid0 + c; b2 lives in LDS (fp32) and is updated there by waves 0 and 1
   {
     const float* W1 = p.W1 + (size_t)bh * FD * HID;
     const float* W2 = p.W2 + (size_t)bh * HID * FD;
 #pragma unroll
-    for (int rb = 0; rb < 2; rb++)
+    for (int b = 0; b < 2; b++)
 #pragma unroll
-      for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-          const int row = 32 * rb + 8 * (i >> 2) + 4 * h + (i & 3), col = 32 * cb + c;
-          W1s.b[rb][cb][i] = W1[row * HID + 64 * w + col];
-          W2s.b[rb][cb][i] = W2[(64 * w + row) * FD + col];
-          W2t.b[rb][cb][i] = W2[(64 * w + col) * FD + row];
-        }
-#pragma unroll
-    for (int cb = 0; cb < 2; cb++) b1L[cb] = p.b1[(size_t)bh * HID + 64 * w + 32 * cb + c];
-#pragma unroll
-    for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-      for (int i = 0; i < 16; i++) b2acc[rb][i] = p.b2[(size_t)bh * FD + 32 * rb + 8 * (i >> 2) + 4 * h + (i & 3)];
-    s_b1[tid] = p.b1[(size_t)bh * HID + tid];
-    if (tid < FD) s_b2[tid] = p.b2[(size_t)bh * FD + tid];
-  }
-  float gam[4][4], bet[4][4];
-#pragma unroll
-  for (int r = 0; r < 4; r++)
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-      gam[r][e] = p.ttt_norm_weight[head * FD + 16 * r + 4 * fq + e];
-      bet[r][e] = p.ttt_norm_bias[head * FD + 16 * r + 4 * fq + e];
+      for (int i = 0; i < 16; i++) {
+        const int row = 8 * (i >> 2) + 4 * h + (i & 3);
+        W1s.b[b][0][i] = W1[(32 * b + row) * HID + hid0 + c];
+        W2t.b[b][0][i] = W2[(hid0 + c) * FD + 32 * b + row];
+        W2s.b[0][b][i] = W2[(hid0 + row) * FD + 32 * b + c];
+      }
+    b1L = p.b1[(size_t)bh * HID + hid0 + c];
+    if (tid < HID) s_b1[tid] = p.b1[(size_t)bh * HID + tid];
+    if (tid < FD) {
+      s_b2[tid] = p.b2[(size_t)bh * FD + tid];
+      s_gam[tid] = p.ttt_norm_weight[head * FD + tid];
+      s_bet[tid] = p.ttt_norm_bias[head * FD + tid];
     }
+  }
   bf16x8 ones;
 #pragma unroll
   for (int j = 0; j < 8; j++) ones[j] = (bf16)1.0f;
@@ -119,11 +148,11 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_fwd_kernel(const FwdParams p
   const size_t eta_base = (size_t)bh * p.NC * CS;
   Staged st;
   stage_load(st, p, x_base, eta_base, tid);
-  stage_store(st, smem, tid);
+  stage_store(st, smem, 0, tid);
   __syncthreads();
 
   for (int mb = 0; mb < p.NC; mb++) {
-    if (mb + 1 < p.NC) stage_load(st, p, x_base + (size_t)(mb + 1) * (CS * FD), eta_base + (size_t)(mb + 1) * CS, tid);
+    const bf16* s_xq = reinterpret_cast<const bf16*>(smem + SM_XQ + (mb & 1) * SM_TILE);
 
     // ---- checkpoint: the state before this mini-batch
     if (mb % p.cgs == 0) {
@@ -131,222 +160,215 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_fwd_kernel(const FwdParams p
       float* cW1 = p.W1_ck + slot * FD * HID;
       float* cW2 = p.W2_ck + slot * HID * FD;
 #pragma unroll
-      for (int rb = 0; rb < 2; rb++)
+      for (int b = 0; b < 2; b++)
 #pragma unroll
-        for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) {
-            const int row = 32 * rb + 8 * (i >> 2) + 4 * h + (i & 3), col = 32 * cb + c;
-            cW1[row * HID + 64 * w + col] = W1s.b[rb][cb][i];
-            cW2[(64 * w + row) * FD + col] = W2s.b[rb][cb][i];
-          }
-      if (h == 0) {
-#pragma unroll
-        for (int cb = 0; cb < 2; cb++) p.b1_ck[slot * HID + 64 * w + 32 * cb + c] = b1L[cb];
-      }
-      if (w == 0 && c == 0) {
-#pragma unroll
-        for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) p.b2_ck[slot * FD + 32 * rb + 8 * (i >> 2) + 4 * h + (i & 3)] = b2acc[rb][i];
-      }
+        for (int i = 0; i < 16; i++) {
+          const int row = 8 * (i >> 2) + 4 * h + (i & 3);
+          cW1[(32 * b + row) * HID + hid0 + c] = W1s.b[b][0][i];
+          cW2[(hid0 + row) * FD + 32 * b + c] = W2s.b[0][b][i];
+        }
+      if (h == 0) p.b1_ck[slot * HID + hid0 + c] = b1L;
+      if (tid < FD) p.b2_ck[slot * FD + tid] = s_b2[tid];
     }
 
     // ---- Z1 = XK W1 + b1 (rows tok, lane = hid);  X2 = gelu(Z1), D1 = gelu'(Z1)
-    Acc x2, d1;
+    AccT<2, 1> x2, d1;
     {
-      const Opd w1op = cvt_chain(W1s);
-      const Opd xkA = lds_rows_kappa(s_xk, c, h);
+      const OpdT<1, 4> w1op = cvt_chain(W1s);
+      const OpdT<2, 4> xkA = lds_rows_kappa<2, 4>(s_xk, LDB, c, h);
 #pragma unroll
       for (int rb = 0; rb < 2; rb++)
 #pragma unroll
-        for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) x2.b[rb][cb][i] = b1L[cb];
+        for (int i = 0; i < 16; i++) x2.b[rb][0][i] = b1L;
       mma(x2, xkA, w1op);
 #pragma unroll
       for (int rb = 0; rb < 2; rb++)
 #pragma unroll
-        for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) {
-            float g, d;
-            gelu_fd(x2.b[rb][cb][i], g, d);
-            x2.b[rb][cb][i] = g;
-            d1.b[rb][cb][i] = d;
-          }
+        for (int i = 0; i < 16; i++) {
+          float g, d;
+          gelu_fd(x2.b[rb][0][i], g, d);
+          x2.b[rb][0][i] = g;
+          d1.b[rb][0][i] = d;
+        }
     }
-    const Opd x2op = cvt_chain(x2);  // lane = hid, contraction = tok
-    lds_store_rows_kappa(s_x2t, x2op, c, h);  // stored [hid][tok]
-    __syncthreads();
+    const OpdT<1, 4> x2op = cvt_chain(x2);                  // lane = hid, contraction = tok
+    lds_store_rows_kappa<1, 4>(s_x2t, LDB, x2op, c, h);     // stored [hid][tok], private to the wave
+    TTT_WAVE_SYNC();
 
-    // ---- Z2^T partial = W2s^T X2^T (rows F, lane = tok) -> fp32 partial tile [tok][F]
+    // ---- Z2^T partial = W2s^T X2^T (rows F, lane = tok), summed over the pair into [tok][F]
     {
-      const Opd w2A = cvt_chain(W2s);
-      const Opd x2B = lds_tr_kappa(s_x2t, lane);
-      Acc z2;
+      const OpdT<2, 2> w2A = cvt_chain(W2s);
+      const OpdT<2, 2> x2B = lds_tr_kappa<2, 2>(s_x2t, LDB, lane);
+      AccT<2, 2> z2;
       acc_zero(z2);
       mma(z2, w2A, x2B);
-      lds_store_partial(s_Pw, z2, c, h);
+      pair_sum_to_lds(s_Pp, z2, pr, c, h);
     }
-    __syncthreads();
 
-    // ---- LayerNorm-fused reconstruction-loss gradient for 16 tokens per wave, 4 lanes per token
+    // ---- LayerNorm-fused reconstruction-loss gradient: 8 tokens per wave, 8 lanes per token
     {
-      float z[4][4];
+      float z[8];
+      {
+        f32x4 a0 = *reinterpret_cast<const f32x4*>(s_b2 + f0);
+        f32x4 a1 = *reinterpret_cast<const f32x4*>(s_b2 + f0 + 4);
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+          a0 += *reinterpret_cast<const f32x4*>(s_P + t * 64 * LDP + tok * LDP + f0);
+          a1 += *reinterpret_cast<const f32x4*>(s_P + t * 64 * LDP + tok * LDP + f0 + 4);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) { z[e] = a0[e]; z[4 + e] = a1[e]; }
+      }
       float sum = 0.f;
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        f32x4 a = *reinterpret_cast<const f32x4*>(s_b2 + 16 * r + 4 * fq);
-#pragma unroll
-        for (int v = 0; v < 4; v++) a += *reinterpret_cast<const f32x4*>(s_P + v * 64 * LDP + tok * LDP + 16 * r + 4 * fq);
-#pragma unroll
-        for (int e = 0; e < 4; e++) { z[r][e] = a[e]; sum += a[e]; }
-      }
-      const float mu = quad_sum(sum) * (1.f / FD);
+      for (int e = 0; e < 8; e++) sum += z[e];
+      const float mu = oct_sum(sum) * (1.f / FD);
       float var = 0.f;
 #pragma unroll
-      for (int r = 0; r < 4; r++)
+      for (int e = 0; e < 8; e++) { z[e] -= mu; var = __builtin_fmaf(z[e], z[e], var); }
+      const float rstd = __builtin_amdgcn_rsqf(oct_sum(var) * (1.f / FD) + LN_EPS);
+      const bf16x8 kv = *reinterpret_cast<const bf16x8*>(s_xk + tok * LDB + f0);
+      const bf16x8 vv = *reinterpret_cast<const bf16x8*>(s_xv + tok * LDB + f0);
+      float gam[8], bet[8];
 #pragma unroll
-        for (int e = 0; e < 4; e++) { z[r][e] -= mu; var = __builtin_fmaf(z[r][e], z[r][e], var); }
-      const float rstd = __builtin_amdgcn_rsqf(quad_sum(var) * (1.f / FD) + LN_EPS);
+      for (int q = 0; q < 2; q++) {
+        const f32x4 gq = *reinterpret_cast<const f32x4*>(s_gam + f0 + 4 * q);
+        const f32x4 bq = *reinterpret_cast<const f32x4*>(s_bet + f0 + 4 * q);
+#pragma unroll
+        for (int e = 0; e < 4; e++) { gam[4 * q + e] = gq[e]; bet[4 * q + e] = bq[e]; }
+      }
       float s1 = 0.f, s2 = 0.f;
-      float gx[4][4];
+      float gx[8];
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        const bf16x4 kv = *reinterpret_cast<const bf16x4*>(s_xk + tok * LDB + 16 * r + 4 * fq);
-        const bf16x4 vv = *reinterpret_cast<const bf16x4*>(s_xv + tok * LDB + 16 * r + 4 * fq);
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          const float xh = z[r][e] * rstd;
-          const float go = __builtin_fmaf(gam[r][e], xh, bet[r][e]) - (bf2f(vv[e]) - bf2f(kv[e]));
-          z[r][e] = xh;
-          gx[r][e] = go * gam[r][e];
-          s1 += gx[r][e];
-          s2 = __builtin_fmaf(gx[r][e], xh, s2);
-        }
+      for (int e = 0; e < 8; e++) {
+        const float xh = z[e] * rstd;
+        const float go = __builtin_fmaf(gam[e], xh, bet[e]) - (bf2f(vv[e]) - bf2f(kv[e]));
+        z[e] = xh;
+        gx[e] = go * gam[e];
+        s1 += gx[e];
+        s2 = __builtin_fmaf(gx[e], xh, s2);
       }
-      s1 = quad_sum(s1);
-      s2 = quad_sum(s2);
+      s1 = oct_sum(s1);
+      s2 = oct_sum(s2);
       const float scale = -s_eta[tok] * rstd * (1.f / FD);  // G2 = -eta * dl/dZ2
+      bf16x8 o;
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        bf16x4 o;
-#pragma unroll
-        for (int e = 0; e < 4; e++) o[e] = (bf16)((FD * gx[r][e] - s1 - z[r][e] * s2) * scale);
-        *reinterpret_cast<bf16x4*>(s_g2 + tok * LDB + 16 * r + 4 * fq) = o;
-      }
+      for (int e = 0; e < 8; e++) o[e] = (bf16)((FD * gx[e] - s1 - z[e] * s2) * scale);
+      *reinterpret_cast<bf16x8*>(s_g2 + tok * LDB + f0) = o;
     }
+    // the next mini-batch's inputs leave HBM now and are written to LDS at the end of this one
+    if (mb + 1 < p.NC) stage_load(st, p, x_base + (size_t)(mb + 1) * (CS * FD), eta_base + (size_t)(mb + 1) * CS, tid);
     __syncthreads();
 
     // ---- G1 = (G2 W2^T) * gelu'(Z1);  state += X^T G
     {
-      const Opd g2A = lds_rows_kappa(s_g2, c, h);   // lane = tok, contraction = F
-      const Opd w2tB = cvt_chain(W2t);              // lane = hid, contraction = F
-      Acc g1;
+      const OpdT<2, 4> g2A = lds_rows_kappa<2, 4>(s_g2, LDB, c, h);   // lane = tok, contraction = F
+      const OpdT<1, 4> w2tB = cvt_chain(W2t);                          // lane = hid, contraction = F
+      AccT<2, 1> g1;
       acc_zero(g1);
-      mma(g1, g2A, w2tB);                           // rows tok, lane = hid
-      float colsum[2] = {0.f, 0.f};
+      mma(g1, g2A, w2tB);                                              // rows tok, lane = hid
+      float colsum = 0.f;
 #pragma unroll
       for (int rb = 0; rb < 2; rb++)
 #pragma unroll
-        for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) {
-            g1.b[rb][cb][i] *= d1.b[rb][cb][i];
-            colsum[cb] += g1.b[rb][cb][i];
-          }
-      const Opd g1op = cvt_chain(g1);               // lane = hid, contraction = tok
-#pragma unroll
-      for (int cb = 0; cb < 2; cb++) b1L[cb] += half_sum(colsum[cb]);
-      const Opd g2T = lds_tr_kappa(s_g2, lane);     // lane = F, contraction = tok
-      mma(W2s, x2op, g2T);                          // W2[shard,:]   += X2^T G2
-      mma(W2t, g2T, x2op);                          // W2[shard,:]^T += G2^T X2
-#pragma unroll
-      for (int s = 0; s < 4; s++)
-#pragma unroll
-        for (int rb = 0; rb < 2; rb++)
-          b2acc[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(g2T.v[rb][s], ones, b2acc[rb], 0, 0, 0);
-      const Opd xkT = lds_tr_kappa(s_xk, lane);     // lane = F, contraction = tok
-      mma(W1s, xkT, g1op);                          // W1[:,shard]   += XK^T G1
-    }
-    if (h == 0) {
-#pragma unroll
-      for (int cb = 0; cb < 2; cb++) s_b1[64 * w + 32 * cb + c] = b1L[cb];
-    }
-    if (w == 0 && c == 0) {
-#pragma unroll
-      for (int rb = 0; rb < 2; rb++)
+        for (int i = 0; i < 16; i++) {
+          g1.b[rb][0][i] *= d1.b[rb][0][i];
+          colsum += g1.b[rb][0][i];
+        }
+      const OpdT<1, 4> g1op = cvt_chain(g1);                           // lane = hid, contraction = tok
+      b1L += half_sum(colsum);
+      const OpdT<2, 4> g2T = lds_tr_kappa<2, 4>(s_g2, LDB, lane);      // lane = F, contraction = tok
+      mma(W2s, x2op, g2T);                                             // W2[shard,:]   += X2^T G2
+      mma(W2t, g2T, x2op);                                             // W2[shard,:]^T += G2^T X2
+      if (v < 2) {                                                     // b2 += column sums of G2 (rows 32v..32v+32)
+        f32x16 b2acc;
 #pragma unroll
         for (int g = 0; g < 4; g++) {
-          f32x4 v = {b2acc[rb][4 * g], b2acc[rb][4 * g + 1], b2acc[rb][4 * g + 2], b2acc[rb][4 * g + 3]};
-          *reinterpret_cast<f32x4*>(s_b2 + 32 * rb + 8 * g + 4 * h) = v;
+          const f32x4 x = *reinterpret_cast<const f32x4*>(s_b2 + 32 * v + 8 * g + 4 * h);
+#pragma unroll
+          for (int e = 0; e < 4; e++) b2acc[4 * g + e] = x[e];
         }
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+          b2acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v == 0 ? g2T.v[0][s] : g2T.v[1][s], ones, b2acc, 0, 0, 0);
+        if (c == 0) {                                                  // read after the next workgroup barrier
+#pragma unroll
+          for (int g = 0; g < 4; g++) {
+            f32x4 x = {b2acc[4 * g], b2acc[4 * g + 1], b2acc[4 * g + 2], b2acc[4 * g + 3]};
+            *reinterpret_cast<f32x4*>(s_b2 + 32 * v + 8 * g + 4 * h) = x;
+          }
+        }
+      }
+      const OpdT<2, 4> xkT = lds_tr_kappa<2, 4>(s_xk, LDB, lane);      // lane = F, contraction = tok
+      mma(W1s, xkT, g1op);                                             // W1[:,shard]   += XK^T G1
     }
-    __syncthreads();
+    if (h == 0) s_b1[hid0 + c] = b1L;        // read back below by this wave only
+    TTT_WAVE_SYNC();
 
     // ---- post-update forward on XQ, transposed: Z1b^T = W1s^T XQ^T (rows hid, lane = tok)
     {
-      const Opd w1A = cvt_chain(W1s);
-      const Opd xqB = lds_rows_kappa(s_xq, c, h);
-      Acc z1b;
+      const OpdT<1, 4> w1A = cvt_chain(W1s);
+      const OpdT<2, 4> xqB = lds_rows_kappa<2, 4>(s_xq, LDB, c, h);
+      AccT<1, 2> z1b;
 #pragma unroll
-      for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-          const f32x4 bv = *reinterpret_cast<const f32x4*>(s_b1 + 64 * w + 32 * rb + 8 * g + 4 * h);
-#pragma unroll
-          for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) z1b.b[rb][cb][4 * g + e] = bv[e];
-        }
-      mma(z1b, w1A, xqB);
-#pragma unroll
-      for (int rb = 0; rb < 2; rb++)
+      for (int g = 0; g < 4; g++) {
+        const f32x4 bv = *reinterpret_cast<const f32x4*>(s_b1 + hid0 + 8 * g + 4 * h);
 #pragma unroll
         for (int cb = 0; cb < 2; cb++)
 #pragma unroll
-          for (int i = 0; i < 16; i++) z1b.b[rb][cb][i] = gelu_f(z1b.b[rb][cb][i]);
-      const Opd x2bB = cvt_chain(z1b);              // lane = tok, contraction = hid
-      const Opd w2A = cvt_chain(W2s);
-      Acc z2;
+          for (int e = 0; e < 4; e++) z1b.b[0][cb][4 * g + e] = bv[e];
+      }
+      mma(z1b, w1A, xqB);
+#pragma unroll
+      for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) z1b.b[0][cb][i] = gelu_f(z1b.b[0][cb][i]);
+      const OpdT<2, 2> x2bB = cvt_chain(z1b);      // lane = tok, contraction = hid
+      const OpdT<2, 2> w2A = cvt_chain(W2s);
+      AccT<2, 2> z2;
       acc_zero(z2);
-      mma(z2, w2A, x2bB);                           // rows F, lane = tok
-      lds_store_partial(s_Pw, z2, c, h);
+      mma(z2, w2A, x2bB);                          // rows F, lane = tok
+      pair_sum_to_lds(s_Pp, z2, pr, c, h);
     }
-    __syncthreads();
 
-    // ---- output LayerNorm + residual, 16 tokens per wave
+    // ---- output LayerNorm + residual, 8 tokens per wave; next mini-batch's inputs into LDS
     {
-      float z[4][4];
+      float z[8];
+      {
+        f32x4 a0 = *reinterpret_cast<const f32x4*>(s_b2 + f0);
+        f32x4 a1 = *reinterpret_cast<const f32x4*>(s_b2 + f0 + 4);
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+          a0 += *reinterpret_cast<const f32x4*>(s_P + t * 64 * LDP + tok * LDP + f0);
+          a1 += *reinterpret_cast<const f32x4*>(s_P + t * 64 * LDP + tok * LDP + f0 + 4);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) { z[e] = a0[e]; z[4 + e] = a1[e]; }
+      }
       float sum = 0.f;
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        f32x4 a = *reinterpret_cast<const f32x4*>(s_b2 + 16 * r + 4 * fq);
-#pragma unroll
-        for (int v = 0; v < 4; v++) a += *reinterpret_cast<const f32x4*>(s_P + v * 64 * LDP + tok * LDP + 16 * r + 4 * fq);
-#pragma unroll
-        for (int e = 0; e < 4; e++) { z[r][e] = a[e]; sum += a[e]; }
-      }
-      const float mu = quad_sum(sum) * (1.f / FD);
+      for (int e = 0; e < 8; e++) sum += z[e];
+      const float mu = oct_sum(sum) * (1.f / FD);
       float var = 0.f;
 #pragma unroll
-      for (int r = 0; r < 4; r++)
+      for (int e = 0; e < 8; e++) { z[e] -= mu; var = __builtin_fmaf(z[e], z[e], var); }
+      const float rstd = __builtin_amdgcn_rsqf(oct_sum(var) * (1.f / FD) + LN_EPS);
+      const bf16x8 qv = *reinterpret_cast<const bf16x8*>(s_xq + tok * LDB + f0);
+      float gam[8], bet[8];
 #pragma unroll
-        for (int e = 0; e < 4; e++) { z[r][e] -= mu; var = __builtin_fmaf(z[r][e], z[r][e], var); }
-      const float rstd = __builtin_amdgcn_rsqf(quad_sum(var) * (1.f / FD) + LN_EPS);
-      bf16* out = p.Out + x_base + (size_t)mb * (CS * FD) + tok * FD;
+      for (int q = 0; q < 2; q++) {
+        const f32x4 gq = *reinterpret_cast<const f32x4*>(s_gam + f0 + 4 * q);
+        const f32x4 bq = *reinterpret_cast<const f32x4*>(s_bet + f0 + 4 * q);
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        const bf16x4 qv = *reinterpret_cast<const bf16x4*>(s_xq + tok * LDB + 16 * r + 4 * fq);
-        bf16x4 o;
-#pragma unroll
-        for (int e = 0; e < 4; e++) o[e] = (bf16)(bf2f(qv[e]) + __builtin_fmaf(gam[r][e], z[r][e] * rstd, bet[r][e]));
-        *reinterpret_cast<bf16x4*>(out + 16 * r + 4 * fq) = o;
+        for (int e = 0; e < 4; e++) { gam[4 * q + e] = gq[e]; bet[4 * q + e] = bq[e]; }
       }
+      bf16x8 o;
+#pragma unroll
+      for (int e = 0; e < 8; e++) o[e] = (bf16)(bf2f(qv[e]) + __builtin_fmaf(gam[e], z[e] * rstd, bet[e]));
+      *reinterpret_cast<bf16x8*>(p.Out + x_base + (size_t)mb * (CS * FD) + tok * FD + f0) = o;
     }
-    __syncthreads();
-    if (mb + 1 < p.NC) stage_store(st, smem, tid);
+    // XK / XV were last read before the pair sum above; the XQ buffer written here is the other one.
+    if (mb + 1 < p.NC) stage_store(st, smem, (mb + 1) & 1, tid);
     __syncthreads();
   }
 }
@@ -354,12 +376,13 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_fwd_kernel(const FwdParams p
 }  // namespace ttt
 
 extern "C" int ttt_mlp_fwd_lds_bytes() { return ttt::SM_FWD_BYTES; }
+extern "C" int ttt_mlp_fwd_threads() { return ttt::FW_THREADS; }
 
 hipError_t ttt_mlp_fwd_enqueue(const ttt::FwdParams& p, hipStream_t stream) {
   // Per-device attribute; cheap enough to set on every launch.
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(ttt::ttt_mlp_fwd_kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, ttt::SM_FWD_BYTES);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(ttt::ttt_mlp_fwd_kernel, dim3(p.B * p.NH), dim3(ttt::NTHREADS), ttt::SM_FWD_BYTES, stream, p);
+  hipLaunchKernelGGL(ttt::ttt_mlp_fwd_kernel, dim3(p.B * p.NH), dim3(ttt::FW_THREADS), ttt::SM_FWD_BYTES, stream, p);
   return hipGetLastError();
 }

@@ -39,3 +39,5 @@ hipError_t ttt_mlp_fwd_enqueue(const ttt::FwdParams& p, hipStream_t stream);
 hipError_t ttt_mlp_bwd_enqueue(const ttt::BwdParams& p, hipStream_t stream);
 extern "C" int ttt_mlp_fwd_lds_bytes();
 extern "C" int ttt_mlp_bwd_lds_bytes();
+extern "C" int ttt_mlp_fwd_threads();
+extern "C" int ttt_mlp_bwd_threads();
