@@ -5,11 +5,16 @@
 // group, last to first, the forward is replayed from the checkpoint while the per-mini-batch
 // activations are saved, then the group is walked backwards producing the ten output gradients.
 //
-// Mapping: one workgroup of 4 wavefronts per (batch, head); wave w owns hidden columns [64w, 64w+64).
-// All [tokens x hidden] activations live in registers in the "Q" orientation (accumulator rows =
-// hidden, lane = token), so per-token scalars (eta, dEta partial sums) are per-lane values and sums
-// over the hidden dimension are in-register sums.  An activation that is also needed with tokens as
-// the contraction index is bounced once through a wave-private LDS tile (row store + transposing read).
+// Mapping: one workgroup of 8 wavefronts (two per SIMD, at most 256 registers each) per (batch,
+// head); wave v owns hidden columns [32v, 32v+32).  All [tokens x hidden] activations live in
+// registers in the "Q" orientation (accumulator rows = hidden, lane = token), so per-token scalars
+// (eta, dEta partial sums) are per-lane values.  An activation that is also needed with tokens as the
+// contraction index is bounced once through a wave-private LDS tile (row store + transposing read).
+//
+// Waves v and v^4 form a pair.  A wave keeps the two token blocks of a Q tile in the order (r, 1-r),
+// r = v / 4: of every product summed over the hidden dimension it keeps token block r and hands token
+// block 1-r to its partner through LDS, which adds its own share; the LayerNorm lanes (8 per token,
+// 8 tokens per wave) then add the four pair sums.  Every sum has a fixed order.
 //
 // State in registers:
 //   replay : W1s [F x hid], W2s [hid x F], W2t [F x hid] (fp32 accumulator tiles); b1, b2 in LDS
@@ -17,7 +22,7 @@
 //            enter the reverse walk as ready-made bf16 MFMA operands: after every mini-batch the replay
 //            stores the operand images of W1^T[shard] and W2[shard]^T, and the walk reads the image of
 //            the state after and before the step (before the first step of a group: converted straight
-//            from the fp32 checkpoint).  Half the accumulator file therefore stays free for products.
+//            from the fp32 checkpoint).
 // While a group is replayed the running gradients are parked in the caller's W*_init_group scratch.
 // Saved per mini-batch (caller's *_group scratch): Z1 and Z1_bar as bf16 register images (Z1_group,
 // Z1_bar_group); the two weight operand images (X2_group: W1^T[shard], grad_l_wrt_Z1_group:
@@ -28,328 +33,176 @@
 
 namespace ttt {
 
-constexpr int SB_TILE = 64 * LDB * 2;
+constexpr int BW_NWAVE = 8;
+constexpr int BW_THREADS = 64 * BW_NWAVE;
+constexpr int BW_NS = HID / BW_NWAVE;     // hidden columns per wave: 32
+constexpr int LDX = 68;                   // row stride (elements) of the shared [64][64] bf16 tiles
+constexpr int LDH = 36;                   // row stride of wave-private [64][32 hid] bf16 tiles
+constexpr int LDF = 68;                   // row stride of wave-private [32 hid][64 F] bf16 tiles
+constexpr int LDR = 72;                   // row stride (floats) of a pair-sum region [32 tok][64 F]
+
+constexpr int SB_TILE = 64 * LDX * 2;     // 8704
 constexpr int SB_XQ = 0;                  // reverse: XQ until the post-update stage is done, then (with SB_E2)
 constexpr int SB_E2 = SB_XQ + SB_TILE;    //          the fp32 park of g_y ; replay: XQ and XV
 constexpr int SB_XK = SB_E2 + SB_TILE;
 constexpr int SB_GZ2 = SB_XK + SB_TILE;   // replay: G2 = -eta*dl/dZ2 ; reverse: raw dl/dZ2
 constexpr int SB_A = SB_GZ2 + SB_TILE;    // reverse: gZ2_bar, later dZ2
 static_assert(2 * SB_TILE >= CS * FD * 4, "g_y park does not fit");
-constexpr int SB_P = SB_A + SB_TILE;      // 4 fp32 partial tiles
-constexpr int SB_PTILE = 64 * LDP * 4;
-constexpr int SB_BNC = SB_P + 4 * SB_PTILE;   // 4 wave-private bounce tiles
-constexpr int SB_B1 = SB_BNC + 4 * SB_TILE;   // b1 during a replay, 256 floats
+constexpr int SB_P = SB_A + SB_TILE;      // 8 pair-sum regions (one per wave), fp32 [32][LDR]
+constexpr int SB_REGION = 32 * LDR * 4;   // 9216: also two wave-private bf16 tiles
+constexpr int SB_WTILE = 64 * LDH * 2;    // 4608
+static_assert(2 * SB_WTILE <= SB_REGION && 32 * LDF * 2 <= SB_WTILE, "private tiles do not fit a region");
+constexpr int SB_BNC = SB_P + BW_NWAVE * SB_REGION;   // 8 wave-private bounce tiles [64][LDH]
+constexpr int SB_B1 = SB_BNC + BW_NWAVE * SB_WTILE;   // b1 during a replay, 256 floats
 constexpr int SB_B2 = SB_B1 + HID * 4;        // b2 during a replay, 64 floats
 constexpr int SB_GB1 = SB_B2 + FD * 4;        // running gradient wrt b1
 constexpr int SB_GB2 = SB_GB1 + HID * 4;      // running gradient wrt b2
 constexpr int SB_GAM = SB_GB2 + FD * 4;       // ttt_norm_weight of this head
 constexpr int SB_BET = SB_GAM + FD * 4;       // ttt_norm_bias of this head
 constexpr int SB_ETA = SB_BET + FD * 4;
-constexpr int SB_DETA = SB_ETA + CS * 4;      // [2][4 waves][64 tokens] partial dEta sums
-constexpr int SB_RED = SB_DETA + 2 * 4 * CS * 4;  // [4 waves][2][64] final norm-grad reduction
-constexpr int SM_BWD_BYTES = SB_RED + 4 * 2 * FD * 4;
+constexpr int SB_DETA = SB_ETA + CS * 4;                  // [8 waves][64 tokens] partial dEta sums
+constexpr int SB_RED = SB_DETA + BW_NWAVE * CS * 4;       // [8 waves][2][64] norm-gradient accumulators
+constexpr int SM_BWD_BYTES = SB_RED + BW_NWAVE * 2 * FD * 4;
 static_assert(SM_BWD_BYTES <= 160 * 1024, "LDS budget of one gfx950 CU exceeded");
 
-// Orders a wave-private LDS store against the transposing read that follows it.  LDS operations of
-// one wave execute in issue order, so only the compiler has to be kept from reordering them.
-#define WAVE_SYNC()                                        \
-  do {                                                     \
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); \
-    __builtin_amdgcn_wave_barrier();                       \
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront"); \
-  } while (0)
+#define WAVE_SYNC() TTT_WAVE_SYNC()
+#define MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16((a), (b), (c), 0, 0, 0)
 
 // ------------------------------------------------------------------ register images in HBM
-// A 64x64 tile as 8 chunks of 8 bf16 per lane; chunk n of thread tid sits at (n*256 + tid)*16 bytes,
-// so every store/load instruction of a wave moves 1 KiB contiguous.
-TTT_DEV void opd_store(bf16* base, const Opd& o, int tid) {
-#pragma unroll
-  for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-    for (int s = 0; s < 4; s++) reinterpret_cast<bf16x8*>(base)[(cb * 4 + s) * NTHREADS + tid] = o.v[cb][s];
-}
-TTT_DEV Opd opd_load(const bf16* base, int tid) {
-  Opd o;
-#pragma unroll
-  for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-    for (int s = 0; s < 4; s++) o.v[cb][s] = reinterpret_cast<const bf16x8*>(base)[(cb * 4 + s) * NTHREADS + tid];
-  return o;
-}
-TTT_DEV void img_store(bf16* base, const Acc& x, int tid) { opd_store(base, cvt_chain(x), tid); }
-// Sign flip of every element (exact).
-TTT_DEV Opd opd_neg(const Opd& o) {
-  Opd r;
-#pragma unroll
-  for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-    for (int s = 0; s < 4; s++) {
-      u32x4 u = __builtin_bit_cast(u32x4, o.v[cb][s]);
-      u ^= 0x80008000u;
-      r.v[cb][s] = __builtin_bit_cast(bf16x8, u);
-    }
-  return r;
-}
-TTT_DEV void img_load(const bf16* base, Acc& x, int tid) {
-#pragma unroll
-  for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-    for (int s = 0; s < 4; s++) {
-      const bf16x8 v = reinterpret_cast<const bf16x8*>(base)[(cb * 4 + s) * NTHREADS + tid];
-#pragma unroll
-      for (int j = 0; j < 8; j++) x.b[s >> 1][cb][8 * (s & 1) + j] = (float)v[j];
-    }
-}
+// A [64 tok x 32 hid] (or [64 F x 32 hid]) bf16 operand as 4 chunks of 8 bf16 per lane; chunk n of
+// thread tid sits at (n*512 + tid)*16 bytes, so every load/store instruction of a wave moves 1 KiB.
+TTT_DEV void chunk_store(bf16* base, int n, int tid, bf16x8 v) { reinterpret_cast<bf16x8*>(base)[n * BW_THREADS + tid] = v; }
+TTT_DEV bf16x8 chunk_load(const bf16* base, int n, int tid) { return reinterpret_cast<const bf16x8*>(base)[n * BW_THREADS + tid]; }
 
 // fp32 accumulator tile <-> HBM in the caller's row-major layout.  `ld` = row length, (r0, c0) =
-// origin of this wave's 64x64 block; accumulator rows are tensor rows.
-TTT_DEV void acc_load_rows(Acc& a, const float* g, int ld, int r0, int c0, int c, int h) {
+// origin of this wave's block; accumulator rows are tensor rows.
+template <int RB, int CB>
+TTT_DEV void acc_load_rows(AccT<RB, CB>& a, const float* g, int ld, int r0, int c0, int c, int h) {
 #pragma unroll
-  for (int rb = 0; rb < 2; rb++)
+  for (int rb = 0; rb < RB; rb++)
 #pragma unroll
-    for (int cb = 0; cb < 2; cb++)
+    for (int cb = 0; cb < CB; cb++)
 #pragma unroll
       for (int i = 0; i < 16; i++)
         a.b[rb][cb][i] = g[(size_t)(r0 + 32 * rb + 8 * (i >> 2) + 4 * h + (i & 3)) * ld + c0 + 32 * cb + c];
 }
-TTT_DEV void acc_store_rows(const Acc& a, float* g, int ld, int r0, int c0, int c, int h) {
+template <int RB, int CB>
+TTT_DEV void acc_store_rows(const AccT<RB, CB>& a, float* g, int ld, int r0, int c0, int c, int h) {
 #pragma unroll
-  for (int rb = 0; rb < 2; rb++)
+  for (int rb = 0; rb < RB; rb++)
 #pragma unroll
-    for (int cb = 0; cb < 2; cb++)
+    for (int cb = 0; cb < CB; cb++)
 #pragma unroll
       for (int i = 0; i < 16; i++)
         g[(size_t)(r0 + 32 * rb + 8 * (i >> 2) + 4 * h + (i & 3)) * ld + c0 + 32 * cb + c] = a.b[rb][cb][i];
 }
 // Same, but accumulator rows are tensor COLUMNS (the tile holds the transpose of the block).
-TTT_DEV void acc_load_cols(Acc& a, const float* g, int ld, int r0, int c0, int c, int h) {
+template <int RB, int CB>
+TTT_DEV void acc_load_cols(AccT<RB, CB>& a, const float* g, int ld, int r0, int c0, int c, int h) {
 #pragma unroll
-  for (int rb = 0; rb < 2; rb++)
+  for (int rb = 0; rb < RB; rb++)
 #pragma unroll
-    for (int cb = 0; cb < 2; cb++)
+    for (int cb = 0; cb < CB; cb++)
 #pragma unroll
       for (int i = 0; i < 16; i++)
         a.b[rb][cb][i] = g[(size_t)(r0 + 32 * cb + c) * ld + c0 + 32 * rb + 8 * (i >> 2) + 4 * h + (i & 3)];
 }
-// Bias vector in accumulator-row form: element of row r, identical in every lane column.
-TTT_DEV void rowvec_load(f32x16 (&v)[2], const float* g, int h) {
-#pragma unroll
-  for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-    for (int i = 0; i < 16; i++) v[rb][i] = g[32 * rb + 8 * (i >> 2) + 4 * h + (i & 3)];
-}
-TTT_DEV void rowvec_store(const f32x16 (&v)[2], float* g, int h) {  // call from lanes with c == 0
-#pragma unroll
-  for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-    for (int i = 0; i < 16; i++) g[32 * rb + 8 * (i >> 2) + 4 * h + (i & 3)] = v[rb][i];
-}
-TTT_DEV void rowvec_store_lds(const f32x16 (&v)[2], float* s, int h) {  // call from lanes with c == 0
-#pragma unroll
-  for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-    for (int g = 0; g < 4; g++) {
-      f32x4 x = {v[rb][4 * g], v[rb][4 * g + 1], v[rb][4 * g + 2], v[rb][4 * g + 3]};
-      *reinterpret_cast<f32x4*>(s + 32 * rb + 8 * g + 4 * h) = x;
-    }
-}
-// v[row block] += sum over the 64-long contraction of operand `a` (lane = row index).
-TTT_DEV void rowsum_mma(f32x16 (&v)[2], const Opd& a, bf16x8 ones) {
-#pragma unroll
-  for (int s = 0; s < 4; s++)
-#pragma unroll
-    for (int rb = 0; rb < 2; rb++) v[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v[rb][s], ones, v[rb], 0, 0, 0);
-}
-TTT_DEV void acc_init_rowvec(Acc& a, const f32x16 (&v)[2]) {
-#pragma unroll
-  for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-    for (int cb = 0; cb < 2; cb++) a.b[rb][cb] = v[rb];
-}
-// Swap the roles of lane index and contraction index of an operand through a wave-private tile.
-TTT_DEV Opd bounce(bf16* tile, const Opd& o, int lane) {
-  WAVE_SYNC();  // earlier readers of the tile are done
-  lds_store_rows_kappa(tile, o, lane & 31, lane >> 5);
-  WAVE_SYNC();
-  return lds_tr_kappa(tile, lane);
-}
-TTT_DEV void acc_scale(Acc& a, float s) {
-#pragma unroll
-  for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-    for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-      for (int i = 0; i < 16; i++) a.b[rb][cb][i] *= s;
-}
 
-// Sum over the 16 lanes of a wave that share lane % 4 (the 16 tokens of a LayerNorm stage), result in
-// all of them: two row rotations inside each row of 16 lanes, then across the four rows.
-TTT_DEV float token_sum16(float x) {
-  x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x124, 0xF, 0xF, false));  // row_ror:4
+// ------------------------------------------------------------------ LayerNorm-lane helpers
+// A lane of a LayerNorm stage owns token `tok` and the 8 features f0 .. f0+7.
+TTT_DEV void ln_load(float (&x)[8], const bf16* p) {      // p 8-byte aligned
+  const bf16x4 a = *reinterpret_cast<const bf16x4*>(p), b = *reinterpret_cast<const bf16x4*>(p + 4);
+#pragma unroll
+  for (int e = 0; e < 4; e++) { x[e] = (float)a[e]; x[4 + e] = (float)b[e]; }
+}
+TTT_DEV void ln_store(bf16* p, const float (&x)[8]) {
+  bf16x4 a, b;
+#pragma unroll
+  for (int e = 0; e < 4; e++) { a[e] = (bf16)x[e]; b[e] = (bf16)x[4 + e]; }
+  *reinterpret_cast<bf16x4*>(p) = a;
+  *reinterpret_cast<bf16x4*>(p + 4) = b;
+}
+// dst = bf16(float(dst) + x): the operator accumulates into these outputs.
+TTT_DEV void ln_accumulate(bf16* p, const float (&x)[8]) {
+  bf16x8 v = *reinterpret_cast<const bf16x8*>(p);
+#pragma unroll
+  for (int e = 0; e < 8; e++) v[e] = (bf16)((float)v[e] + x[e]);
+  *reinterpret_cast<bf16x8*>(p) = v;
+}
+TTT_DEV void ln_load_f32(float (&x)[8], const float* p) {
+  const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
+#pragma unroll
+  for (int e = 0; e < 4; e++) { x[e] = a[e]; x[4 + e] = b[e]; }
+}
+// Sum of the four pair sums of this lane's token / features.  `row` points at this token's row of the
+// first pair's region; the regions of successive pairs are 2 regions apart.
+TTT_DEV void ln_gather(float (&z)[8], const float* row) {
+  f32x4 a = *reinterpret_cast<const f32x4*>(row), b = *reinterpret_cast<const f32x4*>(row + 4);
+#pragma unroll
+  for (int pp = 1; pp < 4; pp++) {
+    a += *reinterpret_cast<const f32x4*>(row + pp * 2 * (32 * LDR));
+    b += *reinterpret_cast<const f32x4*>(row + pp * 2 * (32 * LDR) + 4);
+  }
+#pragma unroll
+  for (int e = 0; e < 4; e++) { z[e] = a[e]; z[4 + e] = b[e]; }
+}
+TTT_DEV float sum8(const float (&x)[8]) {
+  float s = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; e++) s += x[e];
+  return s;
+}
+TTT_DEV float dot8(const float (&x)[8], const float (&y)[8]) {
+  float s = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; e++) s = __builtin_fmaf(x[e], y[e], s);
+  return s;
+}
+// z -> x_hat in place, returns 1/std; *std_out = std.
+TTT_DEV float ln_normalize(float (&z)[8], float* std_out) {
+  const float mu = oct_sum(sum8(z)) * (1.f / FD);
+  float var = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; e++) { z[e] -= mu; var = __builtin_fmaf(z[e], z[e], var); }
+  const float v = oct_sum(var) * (1.f / FD) + LN_EPS;
+  const float rstd = __builtin_amdgcn_rsqf(v);
+#pragma unroll
+  for (int e = 0; e < 8; e++) z[e] *= rstd;
+  *std_out = v * rstd;  // sqrt(v)
+  return rstd;
+}
+// Sum over the 8 lanes of a wave that share lane % 8 (the 8 tokens of a LayerNorm stage), result in
+// all of them: a rotation by 8 inside each row of 16 lanes, then across the four rows.
+TTT_DEV float token_sum8(float x) {
   x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x128, 0xF, 0xF, false));  // row_ror:8
   x += __shfl_xor(x, 16, 64);
   x += __shfl_xor(x, 32, 64);
   return x;
 }
-// acc[16r + 4fq + e] += sum over this wave's tokens of x[r][e]   (wave-private LDS vector)
-TTT_DEV void ln_token_sum_add(float* s_acc, const float (&x)[4][4], int q, int fq) {
+// acc[f0 + e] += sum over this wave's tokens of x[e]   (wave-private LDS vector)
+TTT_DEV void ln_token_sum_add(float* s_acc, const float (&x)[8], int q8, int f0) {
+  f32x4 a, b;
 #pragma unroll
-  for (int r = 0; r < 4; r++) {
-    f32x4 v;
-#pragma unroll
-    for (int e = 0; e < 4; e++) v[e] = token_sum16(x[r][e]);
-    if (q == 0) {
-      f32x4* d = reinterpret_cast<f32x4*>(s_acc + 16 * r + 4 * fq);
-      *d = *d + v;
-    }
+  for (int e = 0; e < 4; e++) { a[e] = token_sum8(x[e]); b[e] = token_sum8(x[4 + e]); }
+  if (q8 == 0) {
+    f32x4* d = reinterpret_cast<f32x4*>(s_acc + f0);
+    d[0] = d[0] + a;
+    d[1] = d[1] + b;
   }
 }
 
-// ------------------------------------------------------------------ LayerNorm-lane helpers
-// A lane of the LayerNorm stage owns token `tok` and features 16r + 4fq + e (r, e in 0..3).
-TTT_DEV void ln_load(float (&x)[4][4], const bf16* row, int fq) {
-#pragma unroll
-  for (int r = 0; r < 4; r++) {
-    const bf16x4 v = *reinterpret_cast<const bf16x4*>(row + 16 * r + 4 * fq);
-#pragma unroll
-    for (int e = 0; e < 4; e++) x[r][e] = (float)v[e];
-  }
+// 16-byte chunk staging of one [64][64] bf16 tile from HBM into an LDS tile with row stride LDX
+// (rows are 8-byte aligned): thread tid moves chunk tid.
+TTT_DEV void lds_put16(bf16* s_tile, int tid, u32x4 v) {
+  uint2* d = reinterpret_cast<uint2*>(s_tile + (tid >> 3) * LDX + (tid & 7) * 8);
+  d[0] = make_uint2(v[0], v[1]);
+  d[1] = make_uint2(v[2], v[3]);
 }
-TTT_DEV void ln_store(bf16* row, const float (&x)[4][4], int fq) {
-#pragma unroll
-  for (int r = 0; r < 4; r++) {
-    bf16x4 v;
-#pragma unroll
-    for (int e = 0; e < 4; e++) v[e] = (bf16)x[r][e];
-    *reinterpret_cast<bf16x4*>(row + 16 * r + 4 * fq) = v;
-  }
-}
-// dst = bf16(float(dst) + x): the operator accumulates into these outputs.
-TTT_DEV void ln_accumulate(bf16* row, const float (&x)[4][4], int fq) {
-#pragma unroll
-  for (int r = 0; r < 4; r++) {
-    bf16x4 v = *reinterpret_cast<const bf16x4*>(row + 16 * r + 4 * fq);
-#pragma unroll
-    for (int e = 0; e < 4; e++) v[e] = (bf16)((float)v[e] + x[r][e]);
-    *reinterpret_cast<bf16x4*>(row + 16 * r + 4 * fq) = v;
-  }
-}
-// Sum of the 4 shard partial tiles (plus a bias vector) for this lane's 16 features.
-TTT_DEV void ln_gather(float (&z)[4][4], const float* s_P, const float* s_bias, int tok, int fq) {
-#pragma unroll
-  for (int r = 0; r < 4; r++) {
-    f32x4 a = *reinterpret_cast<const f32x4*>(s_bias + 16 * r + 4 * fq);
-#pragma unroll
-    for (int v = 0; v < 4; v++) a += *reinterpret_cast<const f32x4*>(s_P + v * 64 * LDP + tok * LDP + 16 * r + 4 * fq);
-#pragma unroll
-    for (int e = 0; e < 4; e++) z[r][e] = a[e];
-  }
-}
-TTT_DEV float sum16(const float (&x)[4][4]) {
-  float s = 0.f;
-#pragma unroll
-  for (int r = 0; r < 4; r++)
-#pragma unroll
-    for (int e = 0; e < 4; e++) s += x[r][e];
-  return s;
-}
-TTT_DEV float dot16(const float (&x)[4][4], const float (&y)[4][4]) {
-  float s = 0.f;
-#pragma unroll
-  for (int r = 0; r < 4; r++)
-#pragma unroll
-    for (int e = 0; e < 4; e++) s = __builtin_fmaf(x[r][e], y[r][e], s);
-  return s;
-}
-// z -> x_hat in place, returns 1/std; *std_out = std.
-TTT_DEV float ln_normalize(float (&z)[4][4], float* std_out) {
-  const float mu = quad_sum(sum16(z)) * (1.f / FD);
-  float var = 0.f;
-#pragma unroll
-  for (int r = 0; r < 4; r++)
-#pragma unroll
-    for (int e = 0; e < 4; e++) { z[r][e] -= mu; var = __builtin_fmaf(z[r][e], z[r][e], var); }
-  const float v = quad_sum(var) * (1.f / FD) + LN_EPS;
-  const float rstd = __builtin_amdgcn_rsqf(v);
-#pragma unroll
-  for (int r = 0; r < 4; r++)
-#pragma unroll
-    for (int e = 0; e < 4; e++) z[r][e] *= rstd;
-  *std_out = v * rstd;  // sqrt(v)
-  return rstd;
-}
-
-// 16-byte chunk staging of one [64][64] bf16 tile from HBM into an LDS tile with row stride LDB.
-TTT_DEV void stage_tile(bf16* s_tile, const bf16* g_tile, int tid) {
-#pragma unroll
-  for (int r = 0; r < 2; r++) {
-    const int id = tid + 256 * r;
-    *reinterpret_cast<u32x4*>(s_tile + (id >> 3) * LDB + (id & 7) * 8) = reinterpret_cast<const u32x4*>(g_tile)[id];
-  }
-}
-
-// C-init of a Q-orientation tile from an LDS vector indexed by accumulator row (64 floats).
-TTT_DEV void acc_init_rows_lds(Acc& a, const float* s_vec, int h) {
-#pragma unroll
-  for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-    for (int g = 0; g < 4; g++) {
-      const f32x4 v = *reinterpret_cast<const f32x4*>(s_vec + 32 * rb + 8 * g + 4 * h);
-#pragma unroll
-      for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-        for (int e = 0; e < 4; e++) a.b[rb][cb][4 * g + e] = v[e];
-    }
-}
-// s_vec[row] += sum over the contraction of operand `a` (lane = row index); the sum is formed on the
-// matrix cores, lanes with c == 0 fold it into the LDS vector.
-TTT_DEV void lds_rowsum_add(float* s_vec, const Opd& a, bf16x8 ones, int c, int h) {
-  f32x16 t[2];
-#pragma unroll
-  for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-    for (int i = 0; i < 16; i++) t[rb][i] = 0.f;
-  rowsum_mma(t, a, ones);
-  if (c == 0) {
-#pragma unroll
-    for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-      for (int g = 0; g < 4; g++) {
-        f32x4* q = reinterpret_cast<f32x4*>(s_vec + 32 * rb + 8 * g + 4 * h);
-        f32x4 v = *q;
-#pragma unroll
-        for (int e = 0; e < 4; e++) v[e] += t[rb][4 * g + e];
-        *q = v;
-      }
-  }
-  // Other lanes of this wave read the vector next; without a fence the compiler may forward the
-  // values each lane saw before the update.
-  WAVE_SYNC();
-}
-TTT_DEV void ln_load_f32(float (&x)[4][4], const float* s_vec, int fq) {
-#pragma unroll
-  for (int r = 0; r < 4; r++) {
-    const f32x4 v = *reinterpret_cast<const f32x4*>(s_vec + 16 * r + 4 * fq);
-#pragma unroll
-    for (int e = 0; e < 4; e++) x[r][e] = v[e];
-  }
-}
-// Sum of the 4 shard partial tiles for this lane's 16 features.
-TTT_DEV void ln_gather0(float (&z)[4][4], const float* s_P, int tok, int fq) {
-#pragma unroll
-  for (int r = 0; r < 4; r++) {
-    f32x4 a = *reinterpret_cast<const f32x4*>(s_P + tok * LDP + 16 * r + 4 * fq);
-#pragma unroll
-    for (int v = 1; v < 4; v++) a += *reinterpret_cast<const f32x4*>(s_P + v * 64 * LDP + tok * LDP + 16 * r + 4 * fq);
-#pragma unroll
-    for (int e = 0; e < 4; e++) z[r][e] = a[e];
-  }
-}
+TTT_DEV void stage_tile(bf16* s_tile, const bf16* g_tile, int tid) { lds_put16(s_tile, tid, reinterpret_cast<const u32x4*>(g_tile)[tid]); }
 
 // ---------------------------------------------------------------- just-in-time operand pieces
 // One MFMA operand piece = 8 bf16 per lane = (free block blk, k-step s).  Loading pieces right
-// before the MFMA that consumes them keeps whole 64x64 operands out of the register file.
-constexpr int LDT = 68;   // row stride of the two operand tiles that share a wave's partial tile
+// before the MFMA that consumes them keeps whole operands out of the register file.
 template <int LD>
 TTT_DEV bf16x8 piece_rows(const bf16* tile, int blk, int s, int c, int h) {
   const bf16* q = tile + (32 * blk + c) * LD + 16 * s + 4 * h;
@@ -367,60 +220,67 @@ TTT_DEV void store_piece_rows(bf16* tile, int blk, int s, int c, int h, bf16x8 v
   *reinterpret_cast<bf16x4*>(q) = __builtin_shufflevector(v, v, 0, 1, 2, 3);
   *reinterpret_cast<bf16x4*>(q + 8) = __builtin_shufflevector(v, v, 4, 5, 6, 7);
 }
-template <int LD>
-TTT_DEV void store_opd_rows(bf16* tile, const Opd& o, int c, int h) {
-#pragma unroll
-  for (int fb = 0; fb < 2; fb++)
-#pragma unroll
-    for (int s = 0; s < 4; s++) store_piece_rows<LD>(tile, fb, s, c, h, o.v[fb][s]);
-}
 // Piece (free block fb, k-step s) of the chained operand of an accumulator tile.
-TTT_DEV bf16x8 piece_state(const Acc& x, int fb, int s) { return pack8(x.b[s >> 1][fb], s & 1); }
-template <int LD>
-TTT_DEV void store_state_rows(bf16* tile, const Acc& x, int c, int h) {
+template <int RB, int CB>
+TTT_DEV bf16x8 piece_state(const AccT<RB, CB>& x, int fb, int s) { return pack8(x.b[s >> 1][fb], s & 1); }
+// Chained operand of an accumulator tile written as an LDS tile stored [free index][contraction index].
+template <int LD, int RB, int CB>
+TTT_DEV void store_state_rows(bf16* tile, const AccT<RB, CB>& x, int c, int h) {
 #pragma unroll
-  for (int fb = 0; fb < 2; fb++)
+  for (int fb = 0; fb < CB; fb++)
 #pragma unroll
-    for (int s = 0; s < 4; s++) store_piece_rows<LD>(tile, fb, s, c, h, piece_state(x, fb, s));
+    for (int s = 0; s < 2 * RB; s++) store_piece_rows<LD>(tile, fb, s, c, h, piece_state(x, fb, s));
 }
-#define MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16((a), (b), (c), 0, 0, 0)
-// d += A * B, pieces produced by the callables fa(blk, s) and fb(blk, s).
-template <class FA, class FB>
-TTT_DEV void mma_jit(Acc& d, FA fa, FB fb) {
+// d += A * B over KS k-steps, pieces produced by the callables fa(row block, s) and fb(column block, s).
+template <int KS, int RB, int CB, class FA, class FB>
+TTT_DEV void mma_jit(AccT<RB, CB>& d, FA fa, FB fb) {
 #pragma unroll
-  for (int s = 0; s < 4; s++) {
-    const bf16x8 a0 = fa(0, s), a1 = fa(1, s), b0 = fb(0, s), b1 = fb(1, s);
-    d.b[0][0] = MFMA(a0, b0, d.b[0][0]);
-    d.b[0][1] = MFMA(a0, b1, d.b[0][1]);
-    d.b[1][0] = MFMA(a1, b0, d.b[1][0]);
-    d.b[1][1] = MFMA(a1, b1, d.b[1][1]);
+  for (int s = 0; s < KS; s++) {
+    bf16x8 a[RB], b[CB];
+#pragma unroll
+    for (int r = 0; r < RB; r++) a[r] = fa(r, s);
+#pragma unroll
+    for (int c = 0; c < CB; c++) b[c] = fb(c, s);
+#pragma unroll
+    for (int r = 0; r < RB; r++)
+#pragma unroll
+      for (int c = 0; c < CB; c++) d.b[r][c] = MFMA(a[r], b[c], d.b[r][c]);
   }
 }
-// s_vec[row] += sum over the contraction of the operand whose pieces fa(rb, s) yields.
+// s_vec[row] += sum over the 64-long contraction of the 32-row operand whose pieces fa(s) yields; the
+// sum is formed on the matrix cores, lanes with c == 0 fold it into the LDS vector.
 template <class FA>
 TTT_DEV void lds_rowsum_add_jit(float* s_vec, FA fa, bf16x8 ones, int c, int h) {
-  f32x16 t[2];
+  f32x16 t;
 #pragma unroll
-  for (int rb = 0; rb < 2; rb++)
+  for (int i = 0; i < 16; i++) t[i] = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; i++) t[rb][i] = 0.f;
-#pragma unroll
-  for (int s = 0; s < 4; s++)
-#pragma unroll
-    for (int rb = 0; rb < 2; rb++) t[rb] = MFMA(fa(rb, s), ones, t[rb]);
+  for (int s = 0; s < 4; s++) t = MFMA(fa(s), ones, t);
   if (c == 0) {
 #pragma unroll
-    for (int rb = 0; rb < 2; rb++)
+    for (int g = 0; g < 4; g++) {
+      f32x4* q = reinterpret_cast<f32x4*>(s_vec + 8 * g + 4 * h);
+      f32x4 v = *q;
 #pragma unroll
-      for (int g = 0; g < 4; g++) {
-        f32x4* q = reinterpret_cast<f32x4*>(s_vec + 32 * rb + 8 * g + 4 * h);
-        f32x4 v = *q;
-#pragma unroll
-        for (int e = 0; e < 4; e++) v[e] += t[rb][4 * g + e];
-        *q = v;
-      }
+      for (int e = 0; e < 4; e++) v[e] += t[4 * g + e];
+      *q = v;
+    }
   }
+  // Other lanes of this wave read the vector next; without a fence the compiler may forward the
+  // values each lane saw before the update.
   WAVE_SYNC();
+}
+// C-init of the rows of a Q-orientation tile from an LDS vector indexed by accumulator row (32 floats).
+template <int CB>
+TTT_DEV void acc_init_rows_lds(AccT<1, CB>& a, const float* s_vec, int h) {
+#pragma unroll
+  for (int g = 0; g < 4; g++) {
+    const f32x4 v = *reinterpret_cast<const f32x4*>(s_vec + 8 * g + 4 * h);
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) a.b[0][cb][4 * g + e] = v[e];
+  }
 }
 
 TTT_DEV bf16x8 cvt8(const f32x4 lo, const f32x4 hi) {
@@ -429,49 +289,60 @@ TTT_DEV bf16x8 cvt8(const f32x4 lo, const f32x4 hi) {
   for (int e = 0; e < 4; e++) { o[e] = (bf16)lo[e]; o[4 + e] = (bf16)hi[e]; }
   return o;
 }
-// MFMA operand (kappa order) straight from a row-major fp32 matrix: lane = row r0 + 32*fb + c,
-// contraction = columns c0 .. c0+63.
-TTT_DEV Opd opd_from_f32_rows(const float* g, int ld, int r0, int c0, int c, int h) {
-  Opd o;
+// Piece (kappa order) straight from a row-major fp32 matrix: lane = row `row`, contraction = columns
+// col0 + 16 s ...
+TTT_DEV bf16x8 piece_from_f32(const float* g, int ld, int row, int col0, int s, int h) {
+  const float* q = g + (size_t)row * ld + col0 + 16 * s + 4 * h;
+  return cvt8(*reinterpret_cast<const f32x4*>(q), *reinterpret_cast<const f32x4*>(q + 8));
+}
+
+// Pair sum of a product z (rows F, column block 0 = the token block this wave keeps, column block 1 =
+// the one it hands over): leaves the pair sum of the kept block in the PARTNER's region, stored
+// [tok in block][F].  Contains two workgroup barriers; the caller makes sure that this wave's own
+// reads of its region (the private tiles T1 / T2) are complete.
+TTT_DEV void pair_sum(float* own, float* partner, const AccT<2, 2>& z, int c, int h) {
 #pragma unroll
-  for (int fb = 0; fb < 2; fb++)
+  for (int rb = 0; rb < 2; rb++)
 #pragma unroll
-    for (int s = 0; s < 4; s++) {
-      const float* q = g + (size_t)(r0 + 32 * fb + c) * ld + c0 + 16 * s + 4 * h;
-      o.v[fb][s] = cvt8(*reinterpret_cast<const f32x4*>(q), *reinterpret_cast<const f32x4*>(q + 8));
+    for (int g = 0; g < 4; g++) {
+      const f32x16& x = z.b[rb][1];
+      f32x4 v = {x[4 * g], x[4 * g + 1], x[4 * g + 2], x[4 * g + 3]};
+      *reinterpret_cast<f32x4*>(own + c * LDR + 32 * rb + 8 * g + 4 * h) = v;
     }
-  return o;
+  __syncthreads();
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      float* q = partner + c * LDR + 32 * rb + 8 * g + 4 * h;
+      const f32x16& x = z.b[rb][0];
+      f32x4 v = *reinterpret_cast<const f32x4*>(q);
+      v[0] += x[4 * g]; v[1] += x[4 * g + 1]; v[2] += x[4 * g + 2]; v[3] += x[4 * g + 3];
+      *reinterpret_cast<f32x4*>(q) = v;
+    }
+  __syncthreads();
 }
 
 // Three [64][64] bf16 tiles + the eta vector of one mini-batch in flight from HBM (per thread).
 struct Staged3 {
-  u32x4 a[2], b[2], c[2];
+  u32x4 a, b, c;
   float eta;
 };
 TTT_DEV void stage3_load(Staged3& s, const bf16* ga, const bf16* gb, const bf16* gc, const bf16* geta, size_t tile_off,
                          size_t eta_off, int tid) {
-#pragma unroll
-  for (int r = 0; r < 2; r++) {
-    const int id = tid + 256 * r;
-    s.a[r] = reinterpret_cast<const u32x4*>(ga + tile_off)[id];
-    s.b[r] = reinterpret_cast<const u32x4*>(gb + tile_off)[id];
-    s.c[r] = reinterpret_cast<const u32x4*>(gc + tile_off)[id];
-  }
+  s.a = reinterpret_cast<const u32x4*>(ga + tile_off)[tid];
+  s.b = reinterpret_cast<const u32x4*>(gb + tile_off)[tid];
+  s.c = reinterpret_cast<const u32x4*>(gc + tile_off)[tid];
   s.eta = (tid < CS) ? bf2f(geta[eta_off + tid]) : 0.f;
 }
 TTT_DEV void stage3_store(const Staged3& s, bf16* sa, bf16* sb, bf16* sc, float* s_eta, int tid) {
-#pragma unroll
-  for (int r = 0; r < 2; r++) {
-    const int id = tid + 256 * r;
-    const int off = (id >> 3) * LDB + (id & 7) * 8;
-    *reinterpret_cast<u32x4*>(sa + off) = s.a[r];
-    *reinterpret_cast<u32x4*>(sb + off) = s.b[r];
-    *reinterpret_cast<u32x4*>(sc + off) = s.c[r];
-  }
+  lds_put16(sa, tid, s.a);
+  lds_put16(sb, tid, s.b);
+  lds_put16(sc, tid, s.c);
   if (tid < CS) s_eta[tid] = s.eta;
 }
 
-__global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p) {
+__global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   bf16* s_xq = reinterpret_cast<bf16*>(smem + SB_XQ);
   bf16* s_xk = reinterpret_cast<bf16*>(smem + SB_XK);
@@ -489,13 +360,21 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
   float* s_deta = reinterpret_cast<float*>(smem + SB_DETA);
   float* s_red = reinterpret_cast<float*>(smem + SB_RED);
 
-  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, h = lane >> 5, c = lane & 31;
-  const int q = lane >> 2, fq = lane & 3, tok = 16 * w + q;
+  const int tid = threadIdx.x, v = tid >> 6, lane = tid & 63, h = lane >> 5, c = lane & 31;
+  const int pp = v & 3, r = v >> 2;                              // pair, index inside the pair
+  const int tb[2] = {r, 1 - r};                                  // token block held in column block 0 / 1 of a Q tile
+  const int q8 = lane >> 3, tok = 8 * v + q8, f0 = 8 * (lane & 7);   // LayerNorm ownership (token block r)
   const int bh = blockIdx.x, head = bh % p.NH;
-  float* s_Pw = s_P + w * 64 * LDP;
-  bf16* s_bnc = reinterpret_cast<bf16*>(smem + SB_BNC) + w * 64 * LDB;
-  float* s_b1w = s_b1 + 64 * w;
-  float* s_gb1w = s_gb1 + 64 * w;
+  const int hid0 = BW_NS * v;
+  float* s_own = s_P + (pp * 2 + r) * (32 * LDR);
+  float* s_partner = s_P + (pp * 2 + (1 - r)) * (32 * LDR);
+  // the pair sums of token block r sit in region 1-r of every pair
+  const float* s_lnrow = s_P + (1 - r) * (32 * LDR) + (tok & 31) * LDR + f0;
+  bf16* const T0 = reinterpret_cast<bf16*>(smem + SB_BNC) + v * (64 * LDH);   // wave-private tiles: T0 = the bounce
+  bf16* const T1 = reinterpret_cast<bf16*>(s_own);                            // tile; T1, T2 = the two halves of
+  bf16* const T2 = T1 + 64 * LDH;                                             // this wave's pair-sum region
+  float* s_b1w = s_b1 + hid0;
+  float* s_gb1w = s_gb1 + hid0;
   const int cgs = p.cgs;
 
   if (tid < FD) {
@@ -503,13 +382,13 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
     s_bet[tid] = p.ttt_norm_bias[head * FD + tid];
     s_gb2[tid] = p.grad_L_b2_last[(size_t)bh * FD + tid];
   }
-  s_gb1[tid] = p.grad_L_b1_last[(size_t)bh * HID + tid];
-  // Norm-weight / norm-bias gradients accumulate per wave in LDS (summed over the wave's 16 tokens
+  if (tid < HID) s_gb1[tid] = p.grad_L_b1_last[(size_t)bh * HID + tid];
+  // Norm-weight / norm-bias gradients accumulate per wave in LDS (summed over the wave's 8 tokens
   // with cross-lane adds in a fixed order); summed over the waves at the end.
-  float* s_dgw = s_red + (w * 2 + 0) * FD;
-  float* s_dbw = s_red + (w * 2 + 1) * FD;
+  float* s_dgw = s_red + (v * 2 + 0) * FD;
+  float* s_dbw = s_red + (v * 2 + 1) * FD;
   if (lane < FD) { s_dgw[lane] = 0.f; s_dbw[lane] = 0.f; }
-  float* s_gy = reinterpret_cast<float*>(smem + SB_XQ) + tok * FD;   // this lane's row of the g_y park
+  float* s_gy = reinterpret_cast<float*>(smem + SB_XQ) + tok * FD + f0;   // this lane's part of the g_y park
   bf16x8 ones;
 #pragma unroll
   for (int j = 0; j < 8; j++) ones[j] = (bf16)1.0f;
@@ -525,32 +404,31 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
   // During the reverse walk the same two 64 KiB slots park what must survive the LayerNorm stage.
   bf16* park_d1 = reinterpret_cast<bf16*>(park_W1);                  // 32 KiB register image
   bf16* park_t2 = park_d1 + CS * HID;                                // 32 KiB register image
-  float* park_dk = park_W2 + (size_t)w * (CS * FD) ;                 // 16 KiB per wave
+  bf16* park_g1 = reinterpret_cast<bf16*>(park_W2);                  // 32 KiB register image
 
   // running gradients wrt the state after the last mini-batch
-  Acc gW1s, gW2s;
-  acc_load_rows(gW1s, p.grad_L_W1_last + (size_t)bh * FD * HID, HID, 0, 64 * w, c, h);
-  acc_load_rows(gW2s, p.grad_L_W2_last + (size_t)bh * HID * FD, FD, 64 * w, 0, c, h);
+  AccT<2, 1> gW1s;
+  AccT<1, 2> gW2s;
+  acc_load_rows(gW1s, p.grad_L_W1_last + (size_t)bh * FD * HID, HID, 0, hid0, c, h);
+  acc_load_rows(gW2s, p.grad_L_W2_last + (size_t)bh * HID * FD, FD, hid0, 0, c, h);
 
   for (int k = p.K - 1; k >= 0; k--) {
     const int n_mb = min(cgs, p.NC - k * cgs);
+    const size_t slot = (size_t)bh * p.K + k;
     // ================================================================= replay
     {
       // park the running gradients while the forward state needs the registers
-      acc_store_rows(gW1s, park_W1, HID, 0, 64 * w, c, h);
-      acc_store_rows(gW2s, park_W2, FD, 64 * w, 0, c, h);
-      Acc W1s, W2s, W2t;
-      const size_t slot = (size_t)bh * p.K + k;
-      acc_load_rows(W1s, p.W1_ck + slot * FD * HID, HID, 0, 64 * w, c, h);
-      acc_load_rows(W2s, p.W2_ck + slot * HID * FD, FD, 64 * w, 0, c, h);
-      acc_load_cols(W2t, p.W2_ck + slot * HID * FD, FD, 64 * w, 0, c, h);
+      acc_store_rows(gW1s, park_W1, HID, 0, hid0, c, h);
+      acc_store_rows(gW2s, park_W2, FD, hid0, 0, c, h);
+      AccT<2, 1> W1s, W2t;
+      AccT<1, 2> W2s;
+      acc_load_rows(W1s, p.W1_ck + slot * FD * HID, HID, 0, hid0, c, h);
+      acc_load_rows(W2s, p.W2_ck + slot * HID * FD, FD, hid0, 0, c, h);
+      acc_load_cols(W2t, p.W2_ck + slot * HID * FD, FD, hid0, 0, c, h);
       __syncthreads();  // previous group's readers of the bias vectors are done
-      s_b1[tid] = p.b1_ck[slot * HID + tid];
+      if (tid < HID) s_b1[tid] = p.b1_ck[slot * HID + tid];
       if (tid < FD) s_b2[tid] = p.b2_ck[slot * FD + tid];
 
-      bf16* const T0 = s_bnc;                                   // wave-private tiles, as in the reverse walk
-      bf16* const T1 = reinterpret_cast<bf16*>(s_Pw);
-      bf16* const T2 = T1 + 64 * LDT;
       Staged3 st;
       stage3_load(st, p.XQ, p.XK, p.XV, p.last_eta, x_base + (size_t)(k * cgs) * (CS * FD), eta_base + (size_t)(k * cgs) * CS, tid);
       for (int j = 0; j < n_mb; j++) {
@@ -560,538 +438,495 @@ __global__ __launch_bounds__(NTHREADS) void ttt_mlp_bwd_kernel(const BwdParams p
         __syncthreads();
 
         // Z1^T = W1s^T XK^T + b1  (rows hid, lane = tok); X2 rows [tok][hid] -> T0, gelu'(Z1) packed
-        Opd d1p;
+        bf16x8 d1p[2][2];
         {
-          Acc x2;
+          AccT<1, 2> x2;
           acc_init_rows_lds(x2, s_b1w, h);
-          mma_jit(x2, [&](int blk, int s) { return piece_state(W1s, blk, s); },
-                  [&](int blk, int s) { return piece_rows<LDB>(s_xk, blk, s, c, h); });
+          mma_jit<4>(x2, [&](int, int s) { return piece_state(W1s, 0, s); },
+                     [&](int i, int s) { return piece_rows<LDX>(s_xk, tb[i], s, c, h); });
           bf16* img = p.Z1_group + g_TH + (size_t)j * (CS * HID);
 #pragma unroll
-          for (int cb = 0; cb < 2; cb++)
+          for (int i = 0; i < 2; i++)
 #pragma unroll
-            for (int s = 0; s < 4; s++) {
-              const bf16x8 z = pack8(x2.b[s >> 1][cb], s & 1);
-              reinterpret_cast<bf16x8*>(img)[(cb * 4 + s) * NTHREADS + tid] = z;
+            for (int t = 0; t < 2; t++) {
+              chunk_store(img, 2 * tb[i] + t, tid, pack8(x2.b[0][i], t));
               bf16x8 xv;
 #pragma unroll
               for (int jj = 0; jj < 8; jj++) {
                 float g, d;
-                gelu_fd(x2.b[s >> 1][cb][8 * (s & 1) + jj], g, d);
+                gelu_fd(x2.b[0][i][8 * t + jj], g, d);
                 xv[jj] = (bf16)g;
-                d1p.v[cb][s][jj] = (bf16)d;
+                d1p[i][t][jj] = (bf16)d;
               }
-              store_piece_rows<LDB>(T0, cb, s, c, h, xv);
+              store_piece_rows<LDH>(T0, tb[i], t, c, h, xv);
             }
         }
         WAVE_SYNC();
         {
-          Acc z2;
+          AccT<2, 2> z2;
           acc_zero(z2);
-          mma_jit(z2, [&](int blk, int s) { return piece_state(W2s, blk, s); },                  // lane = F, contraction = hid
-                  [&](int blk, int s) { return piece_rows<LDB>(T0, blk, s, c, h); });            // X2: lane = tok
-          lds_store_partial(s_Pw, z2, c, h);
+          mma_jit<2>(z2, [&](int rb, int s) { return piece_state(W2s, rb, s); },                 // lane = F, contraction = hid
+                     [&](int i, int s) { return piece_rows<LDH>(T0, tb[i], s, c, h); });         // X2: lane = tok
+          pair_sum(s_own, s_partner, z2, c, h);
         }
-        __syncthreads();
         // fused LayerNorm + reconstruction-loss gradient; saves for the reverse walk
         {
-          float z[4][4], gam[4][4];
-          ln_gather(z, s_P, s_b2, tok, fq);
-          ln_load_f32(gam, s_gam, fq);
+          float z[8], gam[8];
+          {
+            float b2v[8];
+            ln_gather(z, s_lnrow);
+            ln_load_f32(b2v, s_b2 + f0);
+#pragma unroll
+            for (int e = 0; e < 8; e++) z[e] += b2v[e];
+          }
+          ln_load_f32(gam, s_gam + f0);
           float sd;
           const float rstd = ln_normalize(z, &sd);
-          float go[4][4], gx[4][4];
+          float go[8], gx[8];
           {
-            float kv[4][4], vv[4][4], bet[4][4];
-            ln_load(kv, s_xk + tok * LDB, fq);
-            ln_load(vv, s_e2 + tok * LDB, fq);
-            ln_load_f32(bet, s_bet, fq);
+            float kv[8], vv[8], bet[8];
+            ln_load(kv, s_xk + tok * LDX + f0);
+            ln_load(vv, s_e2 + tok * LDX + f0);
+            ln_load_f32(bet, s_bet + f0);
 #pragma unroll
-            for (int r = 0; r < 4; r++)
-#pragma unroll
-              for (int e = 0; e < 4; e++) {
-                go[r][e] = __builtin_fmaf(gam[r][e], z[r][e], bet[r][e]) - (vv[r][e] - kv[r][e]);
-                gx[r][e] = go[r][e] * gam[r][e];
-              }
+            for (int e = 0; e < 8; e++) {
+              go[e] = __builtin_fmaf(gam[e], z[e], bet[e]) - (vv[e] - kv[e]);
+              gx[e] = go[e] * gam[e];
+            }
           }
-          const size_t so = g_TF + (size_t)j * (CS * FD) + tok * FD;
-          ln_store(p.x_hat_fused_group + so, z, fq);
-          ln_store(p.grad_output_fused_group + so, go, fq);
-          const float s1 = quad_sum(sum16(gx)), s2 = quad_sum(dot16(gx, z));
+          const size_t so = g_TF + (size_t)j * (CS * FD) + tok * FD + f0;
+          ln_store(p.x_hat_fused_group + so, z);
+          ln_store(p.grad_output_fused_group + so, go);
+          const float s1 = oct_sum(sum8(gx)), s2 = oct_sum(dot8(gx, z));
           const float sc = rstd * (1.f / FD), neg_eta = -s_eta[tok];
 #pragma unroll
-          for (int r = 0; r < 4; r++)
+          for (int e = 0; e < 8; e++) gx[e] = (FD * gx[e] - s1 - z[e] * s2) * sc;   // dl/dZ2
+          ln_store(p.grad_l_wrt_Z2_group + so, gx);
 #pragma unroll
-            for (int e = 0; e < 4; e++) gx[r][e] = (FD * gx[r][e] - s1 - z[r][e] * s2) * sc;   // dl/dZ2
-          ln_store(p.grad_l_wrt_Z2_group + so, gx, fq);
-#pragma unroll
-          for (int r = 0; r < 4; r++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) gx[r][e] *= neg_eta;                                   // G2
-          ln_store(s_gz2 + tok * LDB, gx, fq);
-          if (fq == 0) p.std_fused_group[g_T + (size_t)j * CS + tok] = sd;
+          for (int e = 0; e < 8; e++) gx[e] *= neg_eta;                             // G2
+          ln_store(s_gz2 + tok * LDX + f0, gx);
+          if ((lane & 7) == 0) p.std_fused_group[g_T + (size_t)j * CS + tok] = sd;
         }
         __syncthreads();
         // G1 = (W2 G2^T) * gelu'(Z1)  (rows hid, lane = tok) -> T1 rows [tok][hid]; weight step
         {
-          Acc g1;
+          AccT<1, 2> g1;
           acc_zero(g1);
-          mma_jit(g1, [&](int blk, int s) { return piece_state(W2t, blk, s); },                  // lane = hid, contraction = F
-                  [&](int blk, int s) { return piece_rows<LDB>(s_gz2, blk, s, c, h); });         // G2: lane = tok
+          mma_jit<4>(g1, [&](int, int s) { return piece_state(W2t, 0, s); },                     // lane = hid, contraction = F
+                     [&](int i, int s) { return piece_rows<LDX>(s_gz2, tb[i], s, c, h); });      // G2: lane = tok
 #pragma unroll
-          for (int cb = 0; cb < 2; cb++)
+          for (int i = 0; i < 2; i++)
 #pragma unroll
-            for (int s = 0; s < 4; s++) {
+            for (int t = 0; t < 2; t++) {
               bf16x8 gv;
 #pragma unroll
-              for (int jj = 0; jj < 8; jj++) gv[jj] = (bf16)(g1.b[s >> 1][cb][8 * (s & 1) + jj] * (float)d1p.v[cb][s][jj]);
-              store_piece_rows<LDT>(T1, cb, s, c, h, gv);
+              for (int jj = 0; jj < 8; jj++) gv[jj] = (bf16)(g1.b[0][i][8 * t + jj] * (float)d1p[i][t][jj]);
+              store_piece_rows<LDH>(T1, tb[i], t, c, h, gv);
             }
         }
         WAVE_SYNC();
-        mma_jit(W2s, [&](int blk, int s) { return piece_tr<LDB>(T0, blk, s, lane); },            // X2^T: lane = hid
-                [&](int blk, int s) { return piece_tr<LDB>(s_gz2, blk, s, lane); });             // G2: lane = F
-        mma_jit(W2t, [&](int blk, int s) { return piece_tr<LDB>(s_gz2, blk, s, lane); },
-                [&](int blk, int s) { return piece_tr<LDB>(T0, blk, s, lane); });
-        if (w == 0) lds_rowsum_add_jit(s_b2, [&](int blk, int s) { return piece_tr<LDB>(s_gz2, blk, s, lane); }, ones, c, h);
-        mma_jit(W1s, [&](int blk, int s) { return piece_tr<LDB>(s_xk, blk, s, lane); },          // XK^T: lane = F
-                [&](int blk, int s) { return piece_tr<LDT>(T1, blk, s, lane); });                // G1: lane = hid
-        lds_rowsum_add_jit(s_b1w, [&](int blk, int s) { return piece_tr<LDT>(T1, blk, s, lane); }, ones, c, h);
+        mma_jit<4>(W2s, [&](int, int s) { return piece_tr<LDH>(T0, 0, s, lane); },               // X2^T: lane = hid
+                   [&](int fb, int s) { return piece_tr<LDX>(s_gz2, fb, s, lane); });            // G2: lane = F
+        mma_jit<4>(W2t, [&](int fb, int s) { return piece_tr<LDX>(s_gz2, fb, s, lane); },
+                   [&](int, int s) { return piece_tr<LDH>(T0, 0, s, lane); });
+        if (v < 2) lds_rowsum_add_jit(s_b2 + 32 * v, [&](int s) { return piece_tr<LDX>(s_gz2, v, s, lane); }, ones, c, h);
+        mma_jit<4>(W1s, [&](int fb, int s) { return piece_tr<LDX>(s_xk, fb, s, lane); },         // XK^T: lane = F
+                   [&](int, int s) { return piece_tr<LDH>(T1, 0, s, lane); });                   // G1: lane = hid
+        lds_rowsum_add_jit(s_b1w, [&](int s) { return piece_tr<LDH>(T1, 0, s, lane); }, ones, c, h);
         // operand images of the state after this step, for the reverse walk
         {
           bf16* img2 = p.grad_l_wrt_Z1_group + g_TH + (size_t)j * (CS * HID);   // W2: lane = hid, contraction = F
           bf16* img1 = p.X2_group + g_TH + (size_t)j * (CS * HID);              // W1^T: lane = F, contraction = hid
-          store_state_rows<LDT>(T2, W1s, c, h);                                 // rows [hid][F]
+          store_state_rows<LDF>(T2, W1s, c, h);                                 // rows [hid][F]
 #pragma unroll
-          for (int fb = 0; fb < 2; fb++)
-#pragma unroll
-            for (int s = 0; s < 4; s++) reinterpret_cast<bf16x8*>(img2)[(fb * 4 + s) * NTHREADS + tid] = piece_state(W2t, fb, s);
+          for (int s = 0; s < 4; s++) chunk_store(img2, s, tid, piece_state(W2t, 0, s));
           WAVE_SYNC();
 #pragma unroll
           for (int fb = 0; fb < 2; fb++)
 #pragma unroll
-            for (int s = 0; s < 4; s++) reinterpret_cast<bf16x8*>(img1)[(fb * 4 + s) * NTHREADS + tid] = piece_tr<LDT>(T2, fb, s, lane);
+            for (int s = 0; s < 2; s++) chunk_store(img1, 2 * fb + s, tid, piece_tr<LDF>(T2, fb, s, lane));
         }
         // post-update forward on XQ
         {
-          Acc z1b;
+          AccT<1, 2> z1b;
           acc_init_rows_lds(z1b, s_b1w, h);
-          mma_jit(z1b, [&](int blk, int s) { return piece_state(W1s, blk, s); },
-                  [&](int blk, int s) { return piece_rows<LDB>(s_xq, blk, s, c, h); });
+          mma_jit<4>(z1b, [&](int, int s) { return piece_state(W1s, 0, s); },
+                     [&](int i, int s) { return piece_rows<LDX>(s_xq, tb[i], s, c, h); });
           bf16* img = p.Z1_bar_group + g_TH + (size_t)j * (CS * HID);
-          Opd x2bQ;
+          bf16x8 x2bQ[2][2];
 #pragma unroll
-          for (int cb = 0; cb < 2; cb++)
+          for (int i = 0; i < 2; i++)
 #pragma unroll
-            for (int s = 0; s < 4; s++) {
-              reinterpret_cast<bf16x8*>(img)[(cb * 4 + s) * NTHREADS + tid] = pack8(z1b.b[s >> 1][cb], s & 1);
+            for (int t = 0; t < 2; t++) {
+              chunk_store(img, 2 * tb[i] + t, tid, pack8(z1b.b[0][i], t));
 #pragma unroll
-              for (int jj = 0; jj < 8; jj++) x2bQ.v[cb][s][jj] = (bf16)gelu_f(z1b.b[s >> 1][cb][8 * (s & 1) + jj]);
+              for (int jj = 0; jj < 8; jj++) x2bQ[i][t][jj] = (bf16)gelu_f(z1b.b[0][i][8 * t + jj]);
             }
-          Acc z2;
+          AccT<2, 2> z2;
           acc_zero(z2);
-          mma_jit(z2, [&](int blk, int s) { return piece_state(W2s, blk, s); },
-                  [&](int blk, int s) { return x2bQ.v[blk][s]; });
-          WAVE_SYNC();   // readers of T1 / T2 are done
-          lds_store_partial(s_Pw, z2, c, h);
+          mma_jit<2>(z2, [&](int rb, int s) { return piece_state(W2s, rb, s); },
+                     [&](int i, int s) { return x2bQ[i][s]; });
+          // inputs of the next mini-batch travel while the pair sum and the last LayerNorm stage run
+          if (j + 1 < n_mb)
+            stage3_load(st, p.XQ, p.XK, p.XV, p.last_eta, x_base + (size_t)(mb + 1) * (CS * FD), eta_base + (size_t)(mb + 1) * CS, tid);
+          WAVE_SYNC();   // this wave's readers of T1 / T2 are done
+          pair_sum(s_own, s_partner, z2, c, h);
         }
-        // inputs of the next mini-batch travel while the last LayerNorm stage runs
-        if (j + 1 < n_mb)
-          stage3_load(st, p.XQ, p.XK, p.XV, p.last_eta, x_base + (size_t)(mb + 1) * (CS * FD), eta_base + (size_t)(mb + 1) * CS, tid);
-        __syncthreads();
         {
-          float z[4][4];
-          ln_gather(z, s_P, s_b2, tok, fq);
+          float z[8], b2v[8];
+          ln_gather(z, s_lnrow);
+          ln_load_f32(b2v, s_b2 + f0);
+#pragma unroll
+          for (int e = 0; e < 8; e++) z[e] += b2v[e];
           float sd;
           ln_normalize(z, &sd);
-          ln_store(p.x_hat_ln_group + g_TF + (size_t)j * (CS * FD) + tok * FD, z, fq);
-          if (fq == 0) p.std_ln_group[g_T + (size_t)j * CS + tok] = sd;
+          ln_store(p.x_hat_ln_group + g_TF + (size_t)j * (CS * FD) + tok * FD + f0, z);
+          if ((lane & 7) == 0) p.std_ln_group[g_T + (size_t)j * CS + tok] = sd;
         }
       }
       // running gradients back into registers
-      acc_load_rows(gW1s, park_W1, HID, 0, 64 * w, c, h);
-      acc_load_rows(gW2s, park_W2, FD, 64 * w, 0, c, h);
+      acc_load_rows(gW1s, park_W1, HID, 0, hid0, c, h);
+      acc_load_rows(gW2s, park_W2, FD, hid0, 0, c, h);
     }
 
     // ================================================================= reverse walk
-    // Wave-private LDS tiles of the walk: T0 = the bounce tile (row stride LDB); T1, T2 = the two
-    // halves of this wave's fp32 partial tile (row stride LDT), free whenever no partial sum is in it.
-    const size_t slot = (size_t)bh * p.K + k;
-    bf16* const T0 = s_bnc;
-    bf16* const T1 = reinterpret_cast<bf16*>(s_Pw);
-    bf16* const T2 = T1 + 64 * LDT;
     for (int j = n_mb - 1; j >= 0; j--) {
       const int mb = k * cgs + j;
       const size_t xo = x_base + (size_t)mb * (CS * FD);
       const size_t so = g_TF + (size_t)j * (CS * FD);
       const size_t ho = g_TH + (size_t)j * (CS * HID);
-      // eta of the token this lane holds in column block cb of a Q-orientation tile
-      const float eta_cb[2] = {bf2f(p.last_eta[eta_base + (size_t)mb * CS + c]),
-                               bf2f(p.last_eta[eta_base + (size_t)mb * CS + 32 + c])};
+      // eta of the token this lane holds in column block i of a Q-orientation tile
+      const float eta_i[2] = {bf2f(p.last_eta[eta_base + (size_t)mb * CS + 32 * tb[0] + c]),
+                              bf2f(p.last_eta[eta_base + (size_t)mb * CS + 32 * tb[1] + c])};
       __syncthreads();
       stage_tile(s_xq, p.XQ + xo, tid);
       stage_tile(s_xk, p.XK + xo, tid);
       stage_tile(s_gz2, p.grad_l_wrt_Z2_group + so, tid);
       if (tid < CS) s_eta[tid] = bf2f(p.last_eta[eta_base + (size_t)mb * CS + tid]);
       // operand tiles of the state after this step: T1 = W2 rows [hid][F], T2 = W1^T rows [F][hid]
-      store_opd_rows<LDT>(T1, opd_load(p.grad_l_wrt_Z1_group + ho, tid), c, h);
-      store_opd_rows<LDT>(T2, opd_load(p.X2_group + ho, tid), c, h);
+#pragma unroll
+      for (int s = 0; s < 4; s++) store_piece_rows<LDF>(T1, 0, s, c, h, chunk_load(p.grad_l_wrt_Z1_group + ho, s, tid));
+#pragma unroll
+      for (int fb = 0; fb < 2; fb++)
+#pragma unroll
+        for (int s = 0; s < 2; s++) store_piece_rows<LDH>(T2, fb, s, c, h, chunk_load(p.X2_group + ho, 2 * fb + s, tid));
 
       // ---- output LayerNorm backward (LayerNorm lanes)
       {
-        float gO[4][4], xh[4][4], gx[4][4], gam[4][4];
-        ln_load(gO, p.grad_L_XQW + xo + tok * FD, fq);
-        ln_load(xh, p.x_hat_ln_group + so + tok * FD, fq);
-        ln_load_f32(gam, s_gam, fq);
+        float gO[8], xh[8], gx[8], gam[8];
+        ln_load(gO, p.grad_L_XQW + xo + tok * FD + f0);
+        ln_load(xh, p.x_hat_ln_group + so + tok * FD + f0);
+        ln_load_f32(gam, s_gam + f0);
         const float sd = p.std_ln_group[g_T + (size_t)j * CS + tok];
 #pragma unroll
-        for (int r = 0; r < 4; r++)
+        for (int e = 0; e < 8; e++) gx[e] = gO[e] * xh[e];
+        ln_token_sum_add(s_dbw, gO, q8, f0);
+        ln_token_sum_add(s_dgw, gx, q8, f0);
 #pragma unroll
-          for (int e = 0; e < 4; e++) gx[r][e] = gO[r][e] * xh[r][e];
-        ln_token_sum_add(s_dbw, gO, q, fq);
-        ln_token_sum_add(s_dgw, gx, q, fq);
-#pragma unroll
-        for (int r = 0; r < 4; r++)
-#pragma unroll
-          for (int e = 0; e < 4; e++) gx[r][e] = gO[r][e] * gam[r][e];
-        const float s1 = quad_sum(sum16(gx)), s2 = quad_sum(dot16(gx, xh));
+        for (int e = 0; e < 8; e++) gx[e] = gO[e] * gam[e];
+        const float s1 = oct_sum(sum8(gx)), s2 = oct_sum(dot8(gx, xh));
         const float sc = 1.f / (FD * sd);
 #pragma unroll
-        for (int r = 0; r < 4; r++)
-#pragma unroll
-          for (int e = 0; e < 4; e++) gx[r][e] = (FD * gx[r][e] - s1 - xh[r][e] * s2) * sc;
-        ln_store(s_a + tok * LDB, gx, fq);  // gZ2_bar
+        for (int e = 0; e < 8; e++) gx[e] = (FD * gx[e] - s1 - xh[e] * s2) * sc;
+        ln_store(s_a + tok * LDX + f0, gx);  // gZ2_bar
       }
       __syncthreads();
 
       // ---- post-update forward, backwards (uses the state AFTER this mini-batch)
       {
-        Acc dq;
+        AccT<2, 2> dq;
         {
-          Acc gz1b;   // (gZ2_bar W2^T) * gelu'(Z1_bar): rows hid, lane = tok
+          AccT<1, 2> gz1b;   // (gZ2_bar W2^T) * gelu'(Z1_bar): rows hid, lane = tok
           acc_zero(gz1b);
-          mma_jit(gz1b, [&](int blk, int s) { return piece_rows<LDT>(T1, blk, s, c, h); },
-                  [&](int blk, int s) { return piece_rows<LDB>(s_a, blk, s, c, h); });
+          mma_jit<4>(gz1b, [&](int, int s) { return piece_rows<LDF>(T1, 0, s, c, h); },
+                     [&](int i, int s) { return piece_rows<LDX>(s_a, tb[i], s, c, h); });
           WAVE_SYNC();   // T1 is overwritten below
-          const Opd zimg = opd_load(p.Z1_bar_group + ho, tid);
 #pragma unroll
-          for (int cb = 0; cb < 2; cb++)
+          for (int i = 0; i < 2; i++)
 #pragma unroll
-            for (int s = 0; s < 4; s++) {
+            for (int t = 0; t < 2; t++) {
+              const bf16x8 zc = chunk_load(p.Z1_bar_group + ho, 2 * tb[i] + t, tid);
               bf16x8 x2b, gzb;
 #pragma unroll
               for (int jj = 0; jj < 8; jj++) {
                 float g, d;
-                gelu_fd((float)zimg.v[cb][s][jj], g, d);
+                gelu_fd((float)zc[jj], g, d);
                 x2b[jj] = (bf16)g;
-                gzb[jj] = (bf16)(gz1b.b[s >> 1][cb][8 * (s & 1) + jj] * d);
+                gzb[jj] = (bf16)(gz1b.b[0][i][8 * t + jj] * d);
               }
-              store_piece_rows<LDB>(T0, cb, s, c, h, x2b);    // X2_bar  rows [tok][hid]
-              store_piece_rows<LDT>(T1, cb, s, c, h, gzb);    // gZ1_bar rows [tok][hid]
+              store_piece_rows<LDH>(T0, tb[i], t, c, h, x2b);    // X2_bar  rows [tok][hid]
+              store_piece_rows<LDH>(T1, tb[i], t, c, h, gzb);    // gZ1_bar rows [tok][hid]
             }
         }
         WAVE_SYNC();
         acc_zero(dq);
-        mma_jit(dq, [&](int blk, int s) { return piece_rows<LDT>(T2, blk, s, c, h); },      // W1 after: lane = F
-                [&](int blk, int s) { return piece_rows<LDT>(T1, blk, s, c, h); });         // gZ1_bar: lane = tok
-        mma_jit(gW2s, [&](int blk, int s) { return piece_tr<LDB>(T0, blk, s, lane); },      // X2_bar^T: lane = hid
-                [&](int blk, int s) { return piece_tr<LDB>(s_a, blk, s, lane); });          // gZ2_bar: lane = F
-        if (w == 0) lds_rowsum_add_jit(s_gb2, [&](int blk, int s) { return piece_tr<LDB>(s_a, blk, s, lane); }, ones, c, h);
-        mma_jit(gW1s, [&](int blk, int s) { return piece_tr<LDB>(s_xq, blk, s, lane); },    // XQ^T: lane = F
-                [&](int blk, int s) { return piece_tr<LDT>(T1, blk, s, lane); });           // gZ1_bar: lane = hid
-        lds_rowsum_add_jit(s_gb1w, [&](int blk, int s) { return piece_tr<LDT>(T1, blk, s, lane); }, ones, c, h);
-        WAVE_SYNC();   // every reader of T1 / T2 is done before the partial tile takes their place
-        lds_store_partial(s_Pw, dq, c, h);
+        mma_jit<2>(dq, [&](int rb, int s) { return piece_rows<LDH>(T2, rb, s, c, h); },        // W1 after: lane = F
+                   [&](int i, int s) { return piece_rows<LDH>(T1, tb[i], s, c, h); });         // gZ1_bar: lane = tok
+        mma_jit<4>(gW2s, [&](int, int s) { return piece_tr<LDH>(T0, 0, s, lane); },            // X2_bar^T: lane = hid
+                   [&](int fb, int s) { return piece_tr<LDX>(s_a, fb, s, lane); });            // gZ2_bar: lane = F
+        if (v < 2) lds_rowsum_add_jit(s_gb2 + 32 * v, [&](int s) { return piece_tr<LDX>(s_a, v, s, lane); }, ones, c, h);
+        mma_jit<4>(gW1s, [&](int fb, int s) { return piece_tr<LDX>(s_xq, fb, s, lane); },      // XQ^T: lane = F
+                   [&](int, int s) { return piece_tr<LDH>(T1, 0, s, lane); });                 // gZ1_bar: lane = hid
+        lds_rowsum_add_jit(s_gb1w, [&](int s) { return piece_tr<LDH>(T1, 0, s, lane); }, ones, c, h);
+        WAVE_SYNC();   // every reader of T1 / T2 is done before the pair sum takes their place
+        pair_sum(s_own, s_partner, dq, c, h);
       }
-      __syncthreads();  // partial dXQ tiles complete; gb2 holds its value after the first update
+      // pair sums of dXQ complete; gb2 holds its value after the first update
       {
-        float z[4][4], gO[4][4];
-        ln_gather0(z, s_P, tok, fq);
-        ln_load(gO, p.grad_L_XQW + xo + tok * FD, fq);
+        float z[8], gO[8];
+        ln_gather(z, s_lnrow);
+        ln_load(gO, p.grad_L_XQW + xo + tok * FD + f0);
 #pragma unroll
-        for (int r = 0; r < 4; r++)
-#pragma unroll
-          for (int e = 0; e < 4; e++) z[r][e] += gO[r][e];
-        ln_accumulate(p.grad_L_XQ + xo + tok * FD, z, fq);
+        for (int e = 0; e < 8; e++) z[e] += gO[e];
+        ln_accumulate(p.grad_L_XQ + xo + tok * FD + f0, z);
       }
-      __syncthreads();  // dXQ readers of the partial tiles are done: T1 / T2 are free again
+      __syncthreads();  // dXQ readers of the regions are done: T1 / T2 are free again
 
       // ---- the weight step, backwards (uses the state BEFORE this mini-batch).
-      //      Survive the LayerNorm stage: X2 in T0; packed d1p = gelu'(Z1) and
-      //      t2p = -eta * (gZ2 W2^T) * (XK gW1 + gb1) * gelu''(Z1); the accumulator dk.
+      //      Parked across the LayerNorm stage: X2 in T0; packed d1 = gelu'(Z1), g1 = -eta * dl/dZ1 and
+      //      t2 = -eta * (gZ2 W2^T) * (XK gW1 + gb1) * gelu''(Z1).
       {
-        Acc dk;
         // T1 = W2 before the step, rows [hid][F]; T2 = gW1, rows [hid][F]
-        store_opd_rows<LDT>(T1, (j > 0) ? opd_load(p.grad_l_wrt_Z1_group + ho - CS * HID, tid)
-                                        : opd_from_f32_rows(p.W2_ck + slot * HID * FD, FD, 64 * w, 0, c, h), c, h);
-        store_state_rows<LDT>(T2, gW1s, c, h);
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+          store_piece_rows<LDF>(T1, 0, s, c, h,
+                                (j > 0) ? chunk_load(p.grad_l_wrt_Z1_group + ho - CS * HID, s, tid)
+                                        : piece_from_f32(p.W2_ck + slot * HID * FD, FD, hid0 + c, 0, s, h));
+        store_state_rows<LDF>(T2, gW1s, c, h);
         WAVE_SYNC();
-        Acc R, S;   // R = gZ2 W2^T, S = XK gW1 + gb1   (rows hid, lane = tok)
-        acc_zero(R);
-        acc_init_rows_lds(S, s_gb1w, h);
-        mma_jit(R, [&](int blk, int s) { return piece_rows<LDT>(T1, blk, s, c, h); },
-                [&](int blk, int s) { return piece_rows<LDB>(s_gz2, blk, s, c, h); });
-        mma_jit(S, [&](int blk, int s) { return piece_rows<LDT>(T2, blk, s, c, h); },
-                [&](int blk, int s) { return piece_rows<LDB>(s_xk, blk, s, c, h); });
-        const Opd zimg = opd_load(p.Z1_group + ho, tid);
-        Acc pz;
+        AccT<2, 2> pz;
         acc_zero(pz);
-        acc_zero(dk);
-        float de1[2] = {0.f, 0.f}, de3[2] = {0.f, 0.f};
+        float de[2] = {0.f, 0.f};
 #pragma unroll
-        for (int cb = 0; cb < 2; cb++) {
-          bf16x8 x2c[4], uc[4], g1c[4];
+        for (int i = 0; i < 2; i++) {
+          AccT<1, 1> R, S;   // R = gZ2 W2^T, S = XK gW1 + gb1   (rows hid, lane = tok)
+          acc_zero(R);
+          acc_init_rows_lds(S, s_gb1w, h);
+          mma_jit<4>(R, [&](int, int s) { return piece_rows<LDF>(T1, 0, s, c, h); },
+                     [&](int, int s) { return piece_rows<LDX>(s_gz2, tb[i], s, c, h); });
+          mma_jit<4>(S, [&](int, int s) { return piece_rows<LDF>(T2, 0, s, c, h); },
+                     [&](int, int s) { return piece_rows<LDX>(s_xk, tb[i], s, c, h); });
+          bf16x8 x2c[2], uc[2];
 #pragma unroll
-          for (int s = 0; s < 4; s++) {
-            bf16x8 d1c, t2c;
+          for (int t = 0; t < 2; t++) {
+            const bf16x8 zc = chunk_load(p.Z1_group + ho, 2 * tb[i] + t, tid);
+            bf16x8 d1c, t2c, g1c;
 #pragma unroll
             for (int jj = 0; jj < 8; jj++) {
               float g, a, b;
-              gelu_fdd((float)zimg.v[cb][s][jj], g, a, b);
-              const float r0 = R.b[s >> 1][cb][8 * (s & 1) + jj], sv = S.b[s >> 1][cb][8 * (s & 1) + jj];
+              gelu_fdd((float)zc[jj], g, a, b);
+              const float r0 = R.b[0][0][8 * t + jj], sv = S.b[0][0][8 * t + jj];
               const float gz1 = r0 * a;                                   // dl/dZ1
-              de3[cb] = __builtin_fmaf(gz1, sv, de3[cb]);
-              x2c[s][jj] = (bf16)g;
-              uc[s][jj] = (bf16)(sv * a);
-              g1c[s][jj] = (bf16)(-eta_cb[cb] * gz1);
+              de[i] = __builtin_fmaf(gz1, sv, de[i]);
+              x2c[t][jj] = (bf16)g;
+              uc[t][jj] = (bf16)(sv * a);
+              g1c[jj] = (bf16)(-eta_i[i] * gz1);
               d1c[jj] = (bf16)a;
-              t2c[jj] = (bf16)(-eta_cb[cb] * r0 * sv * b);
+              t2c[jj] = (bf16)(-eta_i[i] * r0 * sv * b);
             }
-            // nothing stays in registers across the LayerNorm stage: d1 and t2 go to their park at once
-            // (L2-resident, rewritten every mini-batch; 1 KiB per wave instruction)
-            reinterpret_cast<bf16x8*>(park_d1)[(cb * 4 + s) * NTHREADS + tid] = d1c;
-            reinterpret_cast<bf16x8*>(park_t2)[(cb * 4 + s) * NTHREADS + tid] = t2c;
+            // nothing stays in registers across the LayerNorm stage: d1, g1 and t2 go to their parks at
+            // once (L2-resident, rewritten every mini-batch; 1 KiB per wave instruction)
+            chunk_store(park_d1, 2 * tb[i] + t, tid, d1c);
+            chunk_store(park_t2, 2 * tb[i] + t, tid, t2c);
+            chunk_store(park_g1, 2 * tb[i] + t, tid, g1c);
+            store_piece_rows<LDH>(T0, tb[i], t, c, h, x2c[t]);             // X2 rows [tok][hid]
           }
+          // pz[:, i] = gW2^T X2^T ; dEta partial ; + W2^T u^T
 #pragma unroll
-          for (int s = 0; s < 4; s++) store_piece_rows<LDB>(T0, cb, s, c, h, x2c[s]);   // X2 rows [tok][hid]
-          // pz[:, cb] = gW2^T X2^T ; dEta partial ; + W2^T u^T.   dk[:, cb] = gW1 G1^T
+          for (int t = 0; t < 2; t++)
 #pragma unroll
-          for (int s = 0; s < 4; s++)
-#pragma unroll
-            for (int rb = 0; rb < 2; rb++) pz.b[rb][cb] = MFMA(piece_state(gW2s, rb, s), x2c[s], pz.b[rb][cb]);
+            for (int rb = 0; rb < 2; rb++) pz.b[rb][i] = MFMA(piece_state(gW2s, rb, t), x2c[t], pz.b[rb][i]);
 #pragma unroll
           for (int s = 0; s < 4; s++) {
-            const bf16x8 gzv = piece_rows<LDB>(s_gz2, cb, s, c, h);
+            const bf16x8 gzv = piece_rows<LDX>(s_gz2, tb[i], s, c, h);
 #pragma unroll
-            for (int jj = 0; jj < 8; jj++)
-              de1[cb] = __builtin_fmaf((float)gzv[jj], pz.b[s >> 1][cb][8 * (s & 1) + jj], de1[cb]);
+            for (int jj = 0; jj < 8; jj++) de[i] = __builtin_fmaf((float)gzv[jj], pz.b[s >> 1][i][8 * (s & 1) + jj], de[i]);
           }
 #pragma unroll
-          for (int s = 0; s < 4; s++)
+          for (int t = 0; t < 2; t++)
 #pragma unroll
-            for (int rb = 0; rb < 2; rb++) {
-              pz.b[rb][cb] = MFMA(piece_tr<LDT>(T1, rb, s, lane), uc[s], pz.b[rb][cb]);
-              dk.b[rb][cb] = MFMA(piece_tr<LDT>(T2, rb, s, lane), g1c[s], dk.b[rb][cb]);
-            }
+            for (int rb = 0; rb < 2; rb++) pz.b[rb][i] = MFMA(piece_tr<LDF>(T1, rb, t, lane), uc[t], pz.b[rb][i]);
         }
-        WAVE_SYNC();   // readers of T1 / T2 done
-        lds_store_partial(s_Pw, pz, c, h);
-        // the accumulator dk is parked too
 #pragma unroll
-        for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-          for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-              f32x4 v = {dk.b[rb][cb][4 * g], dk.b[rb][cb][4 * g + 1], dk.b[rb][cb][4 * g + 2], dk.b[rb][cb][4 * g + 3]};
-              reinterpret_cast<f32x4*>(park_dk)[((rb * 2 + cb) * 4 + g) * 64 + lane] = v;
-            }
-#pragma unroll
-        for (int cb = 0; cb < 2; cb++) {
-          const float a = half_sum(de1[cb]), b = half_sum(de3[cb]);
-          if (h == 0) {
-            s_deta[(0 * 4 + w) * CS + 32 * cb + c] = a;
-            s_deta[(1 * 4 + w) * CS + 32 * cb + c] = b;
-          }
+        for (int i = 0; i < 2; i++) {
+          const float a = half_sum(de[i]);
+          if (h == 0) s_deta[v * CS + 32 * tb[i] + c] = a;
         }
+        WAVE_SYNC();   // this wave's readers of T1 / T2 are done
+        pair_sum(s_own, s_partner, pz, c, h);
       }
-      __syncthreads();  // all partial ggZ2 tiles and dEta partial sums are in LDS
+      // all pair sums of ggZ2 and the dEta partial sums are in LDS
 
       // ---- second-order pass through the fused LayerNorm loss (LayerNorm lanes)
       {
-        float gy[4][4];
-        float gg[4][4], xh[4][4], go[4][4], gz[4][4], gam[4][4];
-        ln_gather(gg, s_P, s_gb2, tok, fq);
+        float gy[8];
+        float gg[8], xh[8], go[8], gz[8], gam[8], gb[8];
+        ln_gather(gg, s_lnrow);
+        ln_load_f32(gb, s_gb2 + f0);
         const float neg_eta = -s_eta[tok];
 #pragma unroll
-        for (int r = 0; r < 4; r++)
-#pragma unroll
-          for (int e = 0; e < 4; e++) gg[r][e] *= neg_eta;                 // grad wrt dl/dZ2
-        ln_load(xh, p.x_hat_fused_group + so + tok * FD, fq);
-        ln_load(go, p.grad_output_fused_group + so + tok * FD, fq);
-        ln_load(gz, s_gz2 + tok * LDB, fq);
-        ln_load_f32(gam, s_gam, fq);
+        for (int e = 0; e < 8; e++) gg[e] = (gg[e] + gb[e]) * neg_eta;   // grad wrt dl/dZ2
+        ln_load(xh, p.x_hat_fused_group + so + tok * FD + f0);
+        ln_load(go, p.grad_output_fused_group + so + tok * FD + f0);
+        ln_load(gz, s_gz2 + tok * LDX + f0);
+        ln_load_f32(gam, s_gam + f0);
         const float sd = p.std_fused_group[g_T + (size_t)j * CS + tok];
         const float rsd = 1.f / sd;
         // dEta: -(sum_F gZ2*(X2 gW2 + gb2) + sum_H gZ1*(XK gW1 + gb1))
         {
-          float gb[4][4];
-          ln_load_f32(gb, s_gb2, fq);
-          float tot = quad_sum(dot16(gz, gb));
+          float tot = oct_sum(dot8(gz, gb));
 #pragma unroll
-          for (int v = 0; v < 8; v++) tot += s_deta[v * CS + tok];
-          if (fq == 0) {
+          for (int u = 0; u < BW_NWAVE; u++) tot += s_deta[u * CS + tok];
+          if ((lane & 7) == 0) {
             bf16* dst = p.grad_L_last_eta + eta_base + (size_t)mb * CS + tok;
             *dst = (bf16)((float)*dst - tot);
           }
         }
-        const float s0 = quad_sum(sum16(gg)), a = quad_sum(dot16(gg, xh));
+        const float s0 = oct_sum(sum8(gg)), a = oct_sum(dot8(gg, xh));
         float bb = 0.f;
 #pragma unroll
-        for (int r = 0; r < 4; r++)
-#pragma unroll
-          for (int e = 0; e < 4; e++) bb = __builtin_fmaf(go[r][e] * gam[r][e], xh[r][e], bb);
-        bb = quad_sum(bb);
-        float gx[4][4], dg[4][4];
+        for (int e = 0; e < 8; e++) bb = __builtin_fmaf(go[e] * gam[e], xh[e], bb);
+        bb = oct_sum(bb);
+        float gx[8], dg[8];
         const float inv = rsd * (1.f / FD);
         float sg = 0.f, sx = 0.f;
 #pragma unroll
-        for (int r = 0; r < 4; r++)
-#pragma unroll
-          for (int e = 0; e < 4; e++) {
-            const float ggx = (gg[r][e] - (s0 + xh[r][e] * a) * (1.f / FD)) * rsd;
-            gy[r][e] = gam[r][e] * ggx;
-            dg[r][e] = go[r][e] * ggx + gy[r][e] * xh[r][e];
-            gx[r][e] = gy[r][e] * gam[r][e] - (go[r][e] * gam[r][e] * a + gg[r][e] * bb) * inv;
-            sg += (-gx[r][e] * xh[r][e] - gg[r][e] * gz[r][e]) * rsd;
-            sx += gx[r][e];
-          }
-        sg = quad_sum(sg);
-        sx = quad_sum(sx);
-        ln_token_sum_add(s_dgw, dg, q, fq);
-        ln_token_sum_add(s_dbw, gy, q, fq);
-#pragma unroll
-        for (int r = 0; r < 4; r++)
-#pragma unroll
-          for (int e = 0; e < 4; e++) {
-            gx[r][e] = gx[r][e] * rsd + (sg * xh[r][e] - sx * rsd) * (1.f / FD);   // dZ2
-            xh[r][e] = -gy[r][e];                                                   // dXV
-          }
-#pragma unroll
-        for (int r = 0; r < 4; r++) {   // g_y is needed again for dXK: park it (XQ / E2 tiles are dead by now)
-          f32x4 v = {gy[r][0], gy[r][1], gy[r][2], gy[r][3]};
-          *reinterpret_cast<f32x4*>(s_gy + 16 * r + 4 * fq) = v;
+        for (int e = 0; e < 8; e++) {
+          const float ggx = (gg[e] - (s0 + xh[e] * a) * (1.f / FD)) * rsd;
+          gy[e] = gam[e] * ggx;
+          dg[e] = go[e] * ggx + gy[e] * xh[e];
+          gx[e] = gy[e] * gam[e] - (go[e] * gam[e] * a + gg[e] * bb) * inv;
+          sg += (-gx[e] * xh[e] - gg[e] * gz[e]) * rsd;
+          sx += gx[e];
         }
-        ln_store(s_a + tok * LDB, gx, fq);
-        ln_accumulate(p.grad_L_XV + xo + tok * FD, xh, fq);
+        sg = oct_sum(sg);
+        sx = oct_sum(sx);
+        ln_token_sum_add(s_dgw, dg, q8, f0);
+        ln_token_sum_add(s_dbw, gy, q8, f0);
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          gx[e] = gx[e] * rsd + (sg * xh[e] - sx * rsd) * (1.f / FD);   // dZ2
+          xh[e] = -gy[e];                                               // dXV
+        }
+        // g_y is needed again for dXK: park it (the XQ / E2 tiles are dead by now)
+        {
+          f32x4 lo = {gy[0], gy[1], gy[2], gy[3]}, hi = {gy[4], gy[5], gy[6], gy[7]};
+          *reinterpret_cast<f32x4*>(s_gy) = lo;
+          *reinterpret_cast<f32x4*>(s_gy + 4) = hi;
+        }
+        ln_store(s_a + tok * LDX + f0, gx);
+        ln_accumulate(p.grad_L_XV + xo + tok * FD + f0, xh);
       }
-      __syncthreads();  // dZ2 tile complete; partial tiles (T1 / T2) free again
+      __syncthreads();  // dZ2 tile complete; regions (T1 / T2) free again
 
       // ---- inner MLP, backwards (uses the state BEFORE this mini-batch)
       {
-        // T2 = gW1 rows [hid][F] (for S again), T1 = gW2 rows [F][hid] (transposed read gives lane = hid)
-        store_state_rows<LDT>(T2, gW1s, c, h);
-        store_state_rows<LDT>(T1, gW2s, c, h);
+        // T2 = gW1 rows [hid][F] (for S again and for gW1 G1^T), T1 = gW2 rows [F][hid] (transposed
+        // read gives lane = hid)
+        store_state_rows<LDF>(T2, gW1s, c, h);
+        store_state_rows<LDH>(T1, gW2s, c, h);
         WAVE_SYNC();
-        Acc S, dx2;
-        acc_init_rows_lds(S, s_gb1w, h);
-        acc_zero(dx2);
-        mma_jit(S, [&](int blk, int s) { return piece_rows<LDT>(T2, blk, s, c, h); },
-                [&](int blk, int s) { return piece_rows<LDB>(s_xk, blk, s, c, h); });
-        mma_jit(dx2, [&](int blk, int s) { return piece_tr<LDT>(T1, blk, s, lane); },       // gW2: lane = hid, contraction = F
-                [&](int blk, int s) { return piece_rows<LDB>(s_gz2, blk, s, c, h); });      // P2 = gZ2 gW2^T
+        AccT<2, 2> dk;
+        acc_zero(dk);
+        bf16x8 dzp[2][2], uhp[2][2];
 #pragma unroll
-        for (int rb = 0; rb < 2; rb++)
+        for (int i = 0; i < 2; i++) {
+          AccT<1, 1> S, dx2;
+          acc_init_rows_lds(S, s_gb1w, h);
+          acc_zero(dx2);
+          mma_jit<4>(S, [&](int, int s) { return piece_rows<LDF>(T2, 0, s, c, h); },
+                     [&](int, int s) { return piece_rows<LDX>(s_xk, tb[i], s, c, h); });
+          mma_jit<4>(dx2, [&](int, int s) { return piece_tr<LDH>(T1, 0, s, lane); },           // gW2: lane = hid, contraction = F
+                     [&](int, int s) { return piece_rows<LDX>(s_gz2, tb[i], s, c, h); });      // P2 = gZ2 gW2^T
 #pragma unroll
-          for (int cb = 0; cb < 2; cb++)
+          for (int e = 0; e < 16; e++) dx2.b[0][0][e] *= -eta_i[i];
+          // + dZ2 W2^T with W2 before the step: lane = hid, contraction = F
+          mma_jit<4>(dx2, [&](int, int s) {
+                       return (j > 0) ? chunk_load(p.grad_l_wrt_Z1_group + ho - CS * HID, s, tid)
+                                      : piece_from_f32(p.W2_ck + slot * HID * FD, FD, hid0 + c, 0, s, h); },
+                     [&](int, int s) { return piece_rows<LDX>(s_a, tb[i], s, c, h); });
+          // dk[:, i] = gW1 G1^T  (gW1: lane = F, contraction = hid)
 #pragma unroll
-            for (int i = 0; i < 16; i++) dx2.b[rb][cb][i] *= -eta_cb[cb];
-        {
-          // W2 before the step: lane = hid, contraction = F
-          const Opd w2tA = (j > 0) ? opd_load(p.grad_l_wrt_Z1_group + ho - CS * HID, tid)
-                                   : opd_from_f32_rows(p.W2_ck + slot * HID * FD, FD, 64 * w, 0, c, h);
-          mma_jit(dx2, [&](int blk, int s) { return w2tA.v[blk][s]; },
-                  [&](int blk, int s) { return piece_rows<LDB>(s_a, blk, s, c, h); });      // + dZ2 W2^T
-        }
-        WAVE_SYNC();   // S and P2 have consumed T2 / T1
-        const Opd d1p = opd_load(park_d1, tid);
-        const Opd t2p = opd_load(park_t2, tid);
-        // dZ1 = dX2*gelu' + t2  -> T1 rows [tok][hid];   -eta * S * gelu' -> T2 rows [tok][hid]
+          for (int t = 0; t < 2; t++) {
+            const bf16x8 g1c = chunk_load(park_g1, 2 * tb[i] + t, tid);
 #pragma unroll
-        for (int cb = 0; cb < 2; cb++)
+            for (int rb = 0; rb < 2; rb++) dk.b[rb][i] = MFMA(piece_tr<LDF>(T2, rb, t, lane), g1c, dk.b[rb][i]);
+          }
+          // dZ1 = dX2*gelu' + t2 ;  -eta * S * gelu'   (kept as pieces until T1 / T2 may be overwritten)
 #pragma unroll
-          for (int s = 0; s < 4; s++) {
-            bf16x8 dz, uh;
+          for (int t = 0; t < 2; t++) {
+            const bf16x8 d1c = chunk_load(park_d1, 2 * tb[i] + t, tid);
+            const bf16x8 t2c = chunk_load(park_t2, 2 * tb[i] + t, tid);
 #pragma unroll
             for (int jj = 0; jj < 8; jj++) {
-              const float d1v = (float)d1p.v[cb][s][jj];
-              dz[jj] = (bf16)__builtin_fmaf(dx2.b[s >> 1][cb][8 * (s & 1) + jj], d1v, (float)t2p.v[cb][s][jj]);
-              uh[jj] = (bf16)(-eta_cb[cb] * S.b[s >> 1][cb][8 * (s & 1) + jj] * d1v);
+              const float d1v = (float)d1c[jj];
+              dzp[i][t][jj] = (bf16)__builtin_fmaf(dx2.b[0][0][8 * t + jj], d1v, (float)t2c[jj]);
+              uhp[i][t][jj] = (bf16)(-eta_i[i] * S.b[0][0][8 * t + jj] * d1v);
             }
-            store_piece_rows<LDT>(T1, cb, s, c, h, dz);
-            store_piece_rows<LDT>(T2, cb, s, c, h, uh);
+          }
+        }
+        WAVE_SYNC();   // S, P2 and gW1 G1^T have consumed T2 / T1
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+          for (int t = 0; t < 2; t++) {
+            store_piece_rows<LDH>(T1, tb[i], t, c, h, dzp[i][t]);   // dZ1 rows [tok][hid]
+            store_piece_rows<LDH>(T2, tb[i], t, c, h, uhp[i][t]);   // -eta u rows [tok][hid]
           }
         WAVE_SYNC();
-        Acc dk;
-#pragma unroll
-        for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-          for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-              const f32x4 v = reinterpret_cast<const f32x4*>(park_dk)[((rb * 2 + cb) * 4 + g) * 64 + lane];
-#pragma unroll
-              for (int e = 0; e < 4; e++) dk.b[rb][cb][4 * g + e] = v[e];
-            }
-        {
-          // W1 before the step: lane = F, contraction = hid
-          const Opd w1tA = (j > 0) ? opd_load(p.X2_group + ho - CS * HID, tid)
-                                   : opd_from_f32_rows(p.W1_ck + slot * FD * HID, HID, 0, 64 * w, c, h);
-          mma_jit(dk, [&](int blk, int s) { return w1tA.v[blk][s]; },
-                  [&](int blk, int s) { return piece_rows<LDT>(T1, blk, s, c, h); });       // + dZ1 W1^T
-        }
-        mma_jit(gW2s, [&](int blk, int s) { return piece_tr<LDT>(T2, blk, s, lane); },      // (-eta u)^T: lane = hid
-                [&](int blk, int s) { return piece_tr<LDB>(s_gz2, blk, s, lane); });        // gZ2: lane = F
-        mma_jit(gW2s, [&](int blk, int s) { return piece_tr<LDB>(T0, blk, s, lane); },      // X2^T: lane = hid
-                [&](int blk, int s) { return piece_tr<LDB>(s_a, blk, s, lane); });          // dZ2: lane = F
-        if (w == 0) lds_rowsum_add_jit(s_gb2, [&](int blk, int s) { return piece_tr<LDB>(s_a, blk, s, lane); }, ones, c, h);
-        mma_jit(gW1s, [&](int blk, int s) { return piece_tr<LDB>(s_xk, blk, s, lane); },    // XK^T: lane = F
-                [&](int blk, int s) { return piece_tr<LDT>(T1, blk, s, lane); });           // dZ1: lane = hid
-        lds_rowsum_add_jit(s_gb1w, [&](int blk, int s) { return piece_tr<LDT>(T1, blk, s, lane); }, ones, c, h);
-        WAVE_SYNC();   // readers of T1 / T2 done
-        lds_store_partial(s_Pw, dk, c, h);
+        // dk += W1 dZ1^T with W1 before the step: lane = F, contraction = hid
+        mma_jit<2>(dk, [&](int rb, int s) {
+                     return (j > 0) ? chunk_load(p.X2_group + ho - CS * HID, 2 * rb + s, tid)
+                                    : piece_from_f32(p.W1_ck + slot * FD * HID, HID, 32 * rb + c, hid0, s, h); },
+                   [&](int i, int s) { return dzp[i][s]; });
+        mma_jit<4>(gW2s, [&](int, int s) { return piece_tr<LDH>(T2, 0, s, lane); },            // (-eta u)^T: lane = hid
+                   [&](int fb, int s) { return piece_tr<LDX>(s_gz2, fb, s, lane); });          // gZ2: lane = F
+        mma_jit<4>(gW2s, [&](int, int s) { return piece_tr<LDH>(T0, 0, s, lane); },            // X2^T: lane = hid
+                   [&](int fb, int s) { return piece_tr<LDX>(s_a, fb, s, lane); });            // dZ2: lane = F
+        if (v < 2) lds_rowsum_add_jit(s_gb2 + 32 * v, [&](int s) { return piece_tr<LDX>(s_a, v, s, lane); }, ones, c, h);
+        mma_jit<4>(gW1s, [&](int fb, int s) { return piece_tr<LDX>(s_xk, fb, s, lane); },      // XK^T: lane = F
+                   [&](int, int s) { return piece_tr<LDH>(T1, 0, s, lane); });                 // dZ1: lane = hid
+        lds_rowsum_add_jit(s_gb1w, [&](int s) { return piece_tr<LDH>(T1, 0, s, lane); }, ones, c, h);
+        WAVE_SYNC();   // this wave's readers of T1 / T2 are done
+        pair_sum(s_own, s_partner, dk, c, h);
       }
-      __syncthreads();  // partial dXK tiles complete
+      // pair sums of dXK complete
       {
-        float z[4][4];
-        ln_gather0(z, s_P, tok, fq);
+        float z[8], gyv[8];
+        ln_gather(z, s_lnrow);
+        ln_load_f32(gyv, s_gy);
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          const f32x4 v = *reinterpret_cast<const f32x4*>(s_gy + 16 * r + 4 * fq);
-#pragma unroll
-          for (int e = 0; e < 4; e++) z[r][e] += v[e];
-        }
-        ln_accumulate(p.grad_L_XK + xo + tok * FD, z, fq);
+        for (int e = 0; e < 8; e++) z[e] += gyv[e];
+        ln_accumulate(p.grad_L_XK + xo + tok * FD + f0, z);
       }
     }
   }
 
   // ---- outputs that are written once
-  acc_store_rows(gW1s, p.grad_L_W1_init + (size_t)bh * FD * HID, HID, 0, 64 * w, c, h);
-  acc_store_rows(gW2s, p.grad_L_W2_init + (size_t)bh * HID * FD, FD, 64 * w, 0, c, h);
+  acc_store_rows(gW1s, p.grad_L_W1_init + (size_t)bh * FD * HID, HID, 0, hid0, c, h);
+  acc_store_rows(gW2s, p.grad_L_W2_init + (size_t)bh * HID * FD, FD, hid0, 0, c, h);
   __syncthreads();
-  p.grad_L_b1_init[(size_t)bh * HID + tid] = s_gb1[tid];
+  if (tid < HID) p.grad_L_b1_init[(size_t)bh * HID + tid] = s_gb1[tid];
   if (tid < FD) p.grad_L_b2_init[(size_t)bh * FD + tid] = s_gb2[tid];
   // norm-weight / norm-bias gradients: sum the per-wave LDS accumulators
-  __syncthreads();
   if (tid < 2 * FD) {
     const int which = tid / FD, f = tid % FD;
     float s = 0.f;
 #pragma unroll
-    for (int v = 0; v < 4; v++) s += s_red[(v * 2 + which) * FD + f];
+    for (int u = 0; u < BW_NWAVE; u++) s += s_red[(u * 2 + which) * FD + f];
     (which == 0 ? p.grad_L_ttt_norm_weight : p.grad_L_ttt_norm_bias)[(size_t)bh * FD + f] = s;
   }
 }
 
 }  // namespace ttt
 
-extern "C" int ttt_mlp_bwd_threads() { return ttt::NTHREADS; }
+extern "C" int ttt_mlp_bwd_threads() { return ttt::BW_THREADS; }
 extern "C" int ttt_mlp_bwd_lds_bytes() { return ttt::SM_BWD_BYTES; }
 
 hipError_t ttt_mlp_bwd_enqueue(const ttt::BwdParams& p, hipStream_t stream) {
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(ttt::ttt_mlp_bwd_kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, ttt::SM_BWD_BYTES);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(ttt::ttt_mlp_bwd_kernel, dim3(p.B * p.NH), dim3(ttt::NTHREADS), ttt::SM_BWD_BYTES, stream, p);
+  hipLaunchKernelGGL(ttt::ttt_mlp_bwd_kernel, dim3(p.B * p.NH), dim3(ttt::BW_THREADS), ttt::SM_BWD_BYTES, stream, p);
   return hipGetLastError();
 }
