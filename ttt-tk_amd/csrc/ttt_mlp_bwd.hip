@@ -342,6 +342,42 @@ TTT_DEV void stage3_store(const Staged3& s, bf16* sa, bf16* sb, bf16* sc, float*
   if (tid < CS) s_eta[tid] = s.eta;
 }
 
+// What the first stages of one reverse step read from HBM (per thread): all requests are issued
+// together at the top of the step.
+struct RevIn {
+  u32x4 xq, xk, gz;          // chunk tid of the XQ, XK and dl/dZ2 tiles
+  float eta;
+  bf16x4 go[2], xh[2];       // LayerNorm lanes: upstream gradient, x_hat of the output LayerNorm
+  float sd;                  //                  and its std
+};
+TTT_DEV void rev_load(RevIn& in, const BwdParams& p, size_t xo, size_t eo, size_t so, size_t to, int tid, int tok, int f0) {
+  in.xq = reinterpret_cast<const u32x4*>(p.XQ + xo)[tid];
+  in.xk = reinterpret_cast<const u32x4*>(p.XK + xo)[tid];
+  in.gz = reinterpret_cast<const u32x4*>(p.grad_l_wrt_Z2_group + so)[tid];
+  in.eta = (tid < CS) ? bf2f(p.last_eta[eo + tid]) : 0.f;
+  const bf16* q = p.grad_L_XQW + xo + tok * FD + f0;
+  in.go[0] = *reinterpret_cast<const bf16x4*>(q);
+  in.go[1] = *reinterpret_cast<const bf16x4*>(q + 4);
+  q = p.x_hat_ln_group + so + tok * FD + f0;
+  in.xh[0] = *reinterpret_cast<const bf16x4*>(q);
+  in.xh[1] = *reinterpret_cast<const bf16x4*>(q + 4);
+  in.sd = p.std_ln_group[to + tok];
+}
+TTT_DEV void ln_cvt(float (&x)[8], const bf16x4 (&v)[2]) {
+#pragma unroll
+  for (int e = 0; e < 4; e++) { x[e] = (float)v[0][e]; x[4 + e] = (float)v[1][e]; }
+}
+// Piece s of W2[shard] before mini-batch j of the group as an operand (lane = hid row, contraction =
+// F): the image the replay stored after mini-batch j-1, or straight from the fp32 checkpoint.
+TTT_DEV bf16x8 w2_before(const bf16* img_prev, const float* ck, int j, int s, int row, int h, int tid) {
+  return (j > 0) ? chunk_load(img_prev, s, tid) : piece_from_f32(ck, FD, row, 0, s, h);
+}
+// Piece (chunk n = 2*rb + s) of W1[:, shard]^T before mini-batch j (lane = F row, contraction = hid).
+TTT_DEV bf16x8 w1_before(const bf16* img_prev, const float* ck, int j, int n, int row, int col0, int s, int h, int tid) {
+  return (j > 0) ? chunk_load(img_prev, n, tid) : piece_from_f32(ck, HID, row, col0, s, h);
+}
+
+
 __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   bf16* s_xq = reinterpret_cast<bf16*>(smem + SB_XQ);
@@ -566,7 +602,6 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
           acc_zero(z2);
           mma_jit<2>(z2, [&](int rb, int s) { return piece_state(W2s, rb, s); },
                      [&](int i, int s) { return x2bQ[i][s]; });
-          // inputs of the next mini-batch travel while the pair sum and the last LayerNorm stage run
           if (j + 1 < n_mb)
             stage3_load(st, p.XQ, p.XK, p.XV, p.last_eta, x_base + (size_t)(mb + 1) * (CS * FD), eta_base + (size_t)(mb + 1) * CS, tid);
           WAVE_SYNC();   // this wave's readers of T1 / T2 are done
@@ -590,6 +625,12 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
     }
 
     // ================================================================= reverse walk
+    // Operands are fetched from HBM right where they are consumed: with two waves per SIMD the other
+    // wave covers the latency, while holding requests in registers across stages costs more in spills
+    // than it gains (measured).
+    const float* ckW1 = p.W1_ck + slot * FD * HID;
+    const float* ckW2 = p.W2_ck + slot * HID * FD;
+    RevIn in;
     for (int j = n_mb - 1; j >= 0; j--) {
       const int mb = k * cgs + j;
       const size_t xo = x_base + (size_t)mb * (CS * FD);
@@ -599,10 +640,11 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
       const float eta_i[2] = {bf2f(p.last_eta[eta_base + (size_t)mb * CS + 32 * tb[0] + c]),
                               bf2f(p.last_eta[eta_base + (size_t)mb * CS + 32 * tb[1] + c])};
       __syncthreads();
-      stage_tile(s_xq, p.XQ + xo, tid);
-      stage_tile(s_xk, p.XK + xo, tid);
-      stage_tile(s_gz2, p.grad_l_wrt_Z2_group + so, tid);
-      if (tid < CS) s_eta[tid] = bf2f(p.last_eta[eta_base + (size_t)mb * CS + tid]);
+      rev_load(in, p, xo, eta_base + (size_t)mb * CS, so, g_T + (size_t)j * CS, tid, tok, f0);
+      lds_put16(s_xq, tid, in.xq);
+      lds_put16(s_xk, tid, in.xk);
+      lds_put16(s_gz2, tid, in.gz);
+      if (tid < CS) s_eta[tid] = in.eta;
       // operand tiles of the state after this step: T1 = W2 rows [hid][F], T2 = W1^T rows [F][hid]
 #pragma unroll
       for (int s = 0; s < 4; s++) store_piece_rows<LDF>(T1, 0, s, c, h, chunk_load(p.grad_l_wrt_Z1_group + ho, s, tid));
@@ -612,12 +654,13 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
         for (int s = 0; s < 2; s++) store_piece_rows<LDH>(T2, fb, s, c, h, chunk_load(p.X2_group + ho, 2 * fb + s, tid));
 
       // ---- output LayerNorm backward (LayerNorm lanes)
+      float gO[8];
       {
-        float gO[8], xh[8], gx[8], gam[8];
-        ln_load(gO, p.grad_L_XQW + xo + tok * FD + f0);
-        ln_load(xh, p.x_hat_ln_group + so + tok * FD + f0);
+        float xh[8], gx[8], gam[8];
+        ln_cvt(gO, in.go);
+        ln_cvt(xh, in.xh);
         ln_load_f32(gam, s_gam + f0);
-        const float sd = p.std_ln_group[g_T + (size_t)j * CS + tok];
+        const float sd = in.sd;
 #pragma unroll
         for (int e = 0; e < 8; e++) gx[e] = gO[e] * xh[e];
         ln_token_sum_add(s_dbw, gO, q8, f0);
@@ -633,6 +676,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
       __syncthreads();
 
       // ---- post-update forward, backwards (uses the state AFTER this mini-batch)
+      bf16x8 dxq_old;            // the output rows this lane accumulates into
       {
         AccT<2, 2> dq;
         {
@@ -645,12 +689,13 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
           for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int t = 0; t < 2; t++) {
-              const bf16x8 zc = chunk_load(p.Z1_bar_group + ho, 2 * tb[i] + t, tid);
               bf16x8 x2b, gzb;
+              bf16x8 zcb[2][2];
+              zcb[i][t] = chunk_load(p.Z1_bar_group + ho, 2 * tb[i] + t, tid);
 #pragma unroll
               for (int jj = 0; jj < 8; jj++) {
                 float g, d;
-                gelu_fd((float)zc[jj], g, d);
+                gelu_fd((float)zcb[i][t][jj], g, d);
                 x2b[jj] = (bf16)g;
                 gzb[jj] = (bf16)(gz1b.b[0][i][8 * t + jj] * d);
               }
@@ -673,25 +718,27 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
       }
       // pair sums of dXQ complete; gb2 holds its value after the first update
       {
-        float z[8], gO[8];
+        float z[8];
         ln_gather(z, s_lnrow);
-        ln_load(gO, p.grad_L_XQW + xo + tok * FD + f0);
+        dxq_old = *reinterpret_cast<const bf16x8*>(p.grad_L_XQ + xo + tok * FD + f0);
 #pragma unroll
-        for (int e = 0; e < 8; e++) z[e] += gO[e];
-        ln_accumulate(p.grad_L_XQ + xo + tok * FD + f0, z);
+        for (int e = 0; e < 8; e++) dxq_old[e] = (bf16)((float)dxq_old[e] + (z[e] + gO[e]));
+        *reinterpret_cast<bf16x8*>(p.grad_L_XQ + xo + tok * FD + f0) = dxq_old;
       }
       __syncthreads();  // dXQ readers of the regions are done: T1 / T2 are free again
 
       // ---- the weight step, backwards (uses the state BEFORE this mini-batch).
       //      Parked across the LayerNorm stage: X2 in T0; packed d1 = gelu'(Z1), g1 = -eta * dl/dZ1 and
       //      t2 = -eta * (gZ2 W2^T) * (XK gW1 + gb1) * gelu''(Z1).
+      bf16x4 xhf[2], gof[2];     // LayerNorm lanes: x_hat / grad_output of the fused loss, its std,
+      float sdf;                 // and the two outputs the stage accumulates into
+      bf16x8 dxv_old;
+      bf16 deta_old;
       {
         // T1 = W2 before the step, rows [hid][F]; T2 = gW1, rows [hid][F]
 #pragma unroll
         for (int s = 0; s < 4; s++)
-          store_piece_rows<LDF>(T1, 0, s, c, h,
-                                (j > 0) ? chunk_load(p.grad_l_wrt_Z1_group + ho - CS * HID, s, tid)
-                                        : piece_from_f32(p.W2_ck + slot * HID * FD, FD, hid0 + c, 0, s, h));
+          store_piece_rows<LDF>(T1, 0, s, c, h, w2_before(p.grad_l_wrt_Z1_group + ho - CS * HID, ckW2, j, s, hid0 + c, h, tid));
         store_state_rows<LDF>(T2, gW1s, c, h);
         WAVE_SYNC();
         AccT<2, 2> pz;
@@ -707,14 +754,14 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
           mma_jit<4>(S, [&](int, int s) { return piece_rows<LDF>(T2, 0, s, c, h); },
                      [&](int, int s) { return piece_rows<LDX>(s_xk, tb[i], s, c, h); });
           bf16x8 x2c[2], uc[2];
+          const bf16x8 zc[2] = {chunk_load(p.Z1_group + ho, 2 * tb[i], tid), chunk_load(p.Z1_group + ho, 2 * tb[i] + 1, tid)};
 #pragma unroll
           for (int t = 0; t < 2; t++) {
-            const bf16x8 zc = chunk_load(p.Z1_group + ho, 2 * tb[i] + t, tid);
             bf16x8 d1c, t2c, g1c;
 #pragma unroll
             for (int jj = 0; jj < 8; jj++) {
               float g, a, b;
-              gelu_fdd((float)zc[jj], g, a, b);
+              gelu_fdd((float)zc[t][jj], g, a, b);
               const float r0 = R.b[0][0][8 * t + jj], sv = S.b[0][0][8 * t + jj];
               const float gz1 = r0 * a;                                   // dl/dZ1
               de[i] = __builtin_fmaf(gz1, sv, de[i]);
@@ -761,26 +808,33 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
       {
         float gy[8];
         float gg[8], xh[8], go[8], gz[8], gam[8], gb[8];
+        dxv_old = *reinterpret_cast<const bf16x8*>(p.grad_L_XV + xo + tok * FD + f0);
+        deta_old = p.grad_L_last_eta[eta_base + (size_t)mb * CS + tok];
+        {
+          const bf16* q = p.x_hat_fused_group + so + tok * FD + f0;
+          xhf[0] = *reinterpret_cast<const bf16x4*>(q);
+          xhf[1] = *reinterpret_cast<const bf16x4*>(q + 4);
+          q = p.grad_output_fused_group + so + tok * FD + f0;
+          gof[0] = *reinterpret_cast<const bf16x4*>(q);
+          gof[1] = *reinterpret_cast<const bf16x4*>(q + 4);
+          sdf = p.std_fused_group[g_T + (size_t)j * CS + tok];
+        }
         ln_gather(gg, s_lnrow);
         ln_load_f32(gb, s_gb2 + f0);
         const float neg_eta = -s_eta[tok];
 #pragma unroll
         for (int e = 0; e < 8; e++) gg[e] = (gg[e] + gb[e]) * neg_eta;   // grad wrt dl/dZ2
-        ln_load(xh, p.x_hat_fused_group + so + tok * FD + f0);
-        ln_load(go, p.grad_output_fused_group + so + tok * FD + f0);
+        ln_cvt(xh, xhf);
+        ln_cvt(go, gof);
         ln_load(gz, s_gz2 + tok * LDX + f0);
         ln_load_f32(gam, s_gam + f0);
-        const float sd = p.std_fused_group[g_T + (size_t)j * CS + tok];
-        const float rsd = 1.f / sd;
+        const float rsd = 1.f / sdf;
         // dEta: -(sum_F gZ2*(X2 gW2 + gb2) + sum_H gZ1*(XK gW1 + gb1))
         {
           float tot = oct_sum(dot8(gz, gb));
 #pragma unroll
           for (int u = 0; u < BW_NWAVE; u++) tot += s_deta[u * CS + tok];
-          if ((lane & 7) == 0) {
-            bf16* dst = p.grad_L_last_eta + eta_base + (size_t)mb * CS + tok;
-            *dst = (bf16)((float)*dst - tot);
-          }
+          if ((lane & 7) == 0) p.grad_L_last_eta[eta_base + (size_t)mb * CS + tok] = (bf16)((float)deta_old - tot);
         }
         const float s0 = oct_sum(sum8(gg)), a = oct_sum(dot8(gg, xh));
         float bb = 0.f;
@@ -806,7 +860,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
 #pragma unroll
         for (int e = 0; e < 8; e++) {
           gx[e] = gx[e] * rsd + (sg * xh[e] - sx * rsd) * (1.f / FD);   // dZ2
-          xh[e] = -gy[e];                                               // dXV
+          dxv_old[e] = (bf16)((float)dxv_old[e] - gy[e]);                // dXV accumulates -g_y
         }
         // g_y is needed again for dXK: park it (the XQ / E2 tiles are dead by now)
         {
@@ -815,12 +869,16 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
           *reinterpret_cast<f32x4*>(s_gy + 4) = hi;
         }
         ln_store(s_a + tok * LDX + f0, gx);
-        ln_accumulate(p.grad_L_XV + xo + tok * FD + f0, xh);
+        *reinterpret_cast<bf16x8*>(p.grad_L_XV + xo + tok * FD + f0) = dxv_old;
       }
       __syncthreads();  // dZ2 tile complete; regions (T1 / T2) free again
 
       // ---- inner MLP, backwards (uses the state BEFORE this mini-batch)
+      bf16x8 dxk_old;
       {
+        bf16x8 w2b[4];   // W2 before the step: lane = hid, contraction = F
+#pragma unroll
+        for (int s = 0; s < 4; s++) w2b[s] = w2_before(p.grad_l_wrt_Z1_group + ho - CS * HID, ckW2, j, s, hid0 + c, h, tid);
         // T2 = gW1 rows [hid][F] (for S again and for gW1 G1^T), T1 = gW2 rows [F][hid] (transposed
         // read gives lane = hid)
         store_state_rows<LDF>(T2, gW1s, c, h);
@@ -840,30 +898,25 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
                      [&](int, int s) { return piece_rows<LDX>(s_gz2, tb[i], s, c, h); });      // P2 = gZ2 gW2^T
 #pragma unroll
           for (int e = 0; e < 16; e++) dx2.b[0][0][e] *= -eta_i[i];
-          // + dZ2 W2^T with W2 before the step: lane = hid, contraction = F
-          mma_jit<4>(dx2, [&](int, int s) {
-                       return (j > 0) ? chunk_load(p.grad_l_wrt_Z1_group + ho - CS * HID, s, tid)
-                                      : piece_from_f32(p.W2_ck + slot * HID * FD, FD, hid0 + c, 0, s, h); },
+          mma_jit<4>(dx2, [&](int, int s) { return w2b[s]; },                                  // + dZ2 W2^T
                      [&](int, int s) { return piece_rows<LDX>(s_a, tb[i], s, c, h); });
           // dk[:, i] = gW1 G1^T  (gW1: lane = F, contraction = hid)
+          const bf16x8 g1c[2] = {chunk_load(park_g1, 2 * tb[i], tid), chunk_load(park_g1, 2 * tb[i] + 1, tid)};
+          const bf16x8 d1c[2] = {chunk_load(park_d1, 2 * tb[i], tid), chunk_load(park_d1, 2 * tb[i] + 1, tid)};
+          const bf16x8 t2c[2] = {chunk_load(park_t2, 2 * tb[i], tid), chunk_load(park_t2, 2 * tb[i] + 1, tid)};
 #pragma unroll
-          for (int t = 0; t < 2; t++) {
-            const bf16x8 g1c = chunk_load(park_g1, 2 * tb[i] + t, tid);
+          for (int t = 0; t < 2; t++)
 #pragma unroll
-            for (int rb = 0; rb < 2; rb++) dk.b[rb][i] = MFMA(piece_tr<LDF>(T2, rb, t, lane), g1c, dk.b[rb][i]);
-          }
+            for (int rb = 0; rb < 2; rb++) dk.b[rb][i] = MFMA(piece_tr<LDF>(T2, rb, t, lane), g1c[t], dk.b[rb][i]);
           // dZ1 = dX2*gelu' + t2 ;  -eta * S * gelu'   (kept as pieces until T1 / T2 may be overwritten)
 #pragma unroll
-          for (int t = 0; t < 2; t++) {
-            const bf16x8 d1c = chunk_load(park_d1, 2 * tb[i] + t, tid);
-            const bf16x8 t2c = chunk_load(park_t2, 2 * tb[i] + t, tid);
+          for (int t = 0; t < 2; t++)
 #pragma unroll
             for (int jj = 0; jj < 8; jj++) {
-              const float d1v = (float)d1c[jj];
-              dzp[i][t][jj] = (bf16)__builtin_fmaf(dx2.b[0][0][8 * t + jj], d1v, (float)t2c[jj]);
+              const float d1v = (float)d1c[t][jj];
+              dzp[i][t][jj] = (bf16)__builtin_fmaf(dx2.b[0][0][8 * t + jj], d1v, (float)t2c[t][jj]);
               uhp[i][t][jj] = (bf16)(-eta_i[i] * S.b[0][0][8 * t + jj] * d1v);
             }
-          }
         }
         WAVE_SYNC();   // S, P2 and gW1 G1^T have consumed T2 / T1
 #pragma unroll
@@ -874,10 +927,8 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
             store_piece_rows<LDH>(T2, tb[i], t, c, h, uhp[i][t]);   // -eta u rows [tok][hid]
           }
         WAVE_SYNC();
-        // dk += W1 dZ1^T with W1 before the step: lane = F, contraction = hid
-        mma_jit<2>(dk, [&](int rb, int s) {
-                     return (j > 0) ? chunk_load(p.X2_group + ho - CS * HID, 2 * rb + s, tid)
-                                    : piece_from_f32(p.W1_ck + slot * FD * HID, HID, 32 * rb + c, hid0, s, h); },
+        mma_jit<2>(dk, [&](int rb, int s) {                                                    // + W1 dZ1^T, W1 before the step
+                     return w1_before(p.X2_group + ho - CS * HID, ckW1, j, 2 * rb + s, 32 * rb + c, hid0, s, h, tid); },
                    [&](int i, int s) { return dzp[i][s]; });
         mma_jit<4>(gW2s, [&](int, int s) { return piece_tr<LDH>(T2, 0, s, lane); },            // (-eta u)^T: lane = hid
                    [&](int fb, int s) { return piece_tr<LDX>(s_gz2, fb, s, lane); });          // gZ2: lane = F
@@ -895,9 +946,10 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
         float z[8], gyv[8];
         ln_gather(z, s_lnrow);
         ln_load_f32(gyv, s_gy);
+        dxk_old = *reinterpret_cast<const bf16x8*>(p.grad_L_XK + xo + tok * FD + f0);
 #pragma unroll
-        for (int e = 0; e < 8; e++) z[e] += gyv[e];
-        ln_accumulate(p.grad_L_XK + xo + tok * FD + f0, z);
+        for (int e = 0; e < 8; e++) dxk_old[e] = (bf16)((float)dxk_old[e] + (z[e] + gyv[e]));
+        *reinterpret_cast<bf16x8*>(p.grad_L_XK + xo + tok * FD + f0) = dxk_old;
       }
     }
   }
