@@ -40,7 +40,7 @@ extern "C" {
 #define TTT_MLP_ERR_BAD_ARG 1001   /* null pointer or non-positive size           */
 #define TTT_MLP_ERR_BAD_CKPT 1002  /* K != ceil(NC / checkpoint_group_size)       */
 #define TTT_MLP_ERR_ALIGN 1003     /* a pointer is not 16-byte aligned            */
-#define TTT_MLP_ERR_TOO_LARGE 1004 /* B*NH exceeds the grid limit                 */
+#define TTT_MLP_ERR_TOO_LARGE 1004 /* B*NH > 2^31-1, NC > 2^18 or cgs > 2^16         */
 
 /* Forward scan.  Replaces the 16 positional arguments of `ttt_forward`
  * (test_time_training.cpp:25-42).  bf16 tensors are passed as uint16_t bit patterns. */

@@ -71,41 +71,51 @@ static_assert(SM_BWD_BYTES <= 160 * 1024, "LDS budget of one gfx950 CU exceeded"
 // ------------------------------------------------------------------ register images in HBM
 // A [64 tok x 32 hid] (or [64 F x 32 hid]) bf16 operand as 4 chunks of 8 bf16 per lane; chunk n of
 // thread tid sits at (n*512 + tid)*16 bytes, so every load/store instruction of a wave moves 1 KiB.
-TTT_DEV void chunk_store(bf16* base, int n, int tid, bf16x8 v) { reinterpret_cast<bf16x8*>(base)[n * BW_THREADS + tid] = v; }
-TTT_DEV bf16x8 chunk_load(const bf16* base, int n, int tid) { return reinterpret_cast<const bf16x8*>(base)[n * BW_THREADS + tid]; }
+// `img` = byte offset of the image inside the buffer, `t16` = 16 * tid.
+constexpr unsigned IMG_BYTES = CS * HID * 2;          // 32 KiB
+constexpr unsigned CHUNK_BYTES = BW_THREADS * 16;     // 8 KiB
+constexpr unsigned TILE_BYTES = CS * FD * 2;          // one [64][64] bf16 tile in HBM: 8 KiB
+TTT_DEV void chunk_store(gptr_t b, unsigned img, int n, unsigned t16, bf16x8 v) { g_st8h(b, t16, img + n * CHUNK_BYTES, v); }
+TTT_DEV bf16x8 chunk_load(gptr_t b, unsigned img, int n, unsigned t16) { return g_ld8h(b, t16, img + n * CHUNK_BYTES); }
 
 // fp32 accumulator tile <-> HBM in the caller's row-major layout.  `ld` = row length, (r0, c0) =
-// origin of this wave's block; accumulator rows are tensor rows.
+// origin of this wave's block (wave-uniform); accumulator rows are tensor rows.
 template <int RB, int CB>
-TTT_DEV void acc_load_rows(AccT<RB, CB>& a, const float* g, int ld, int r0, int c0, int c, int h) {
+TTT_DEV void acc_load_rows(AccT<RB, CB>& a, gptr_t g, unsigned off, int ld, int r0, int c0, int c, int h) {
+  const unsigned vo = (4 * h * ld + c) * 4;
 #pragma unroll
   for (int rb = 0; rb < RB; rb++)
 #pragma unroll
     for (int cb = 0; cb < CB; cb++)
 #pragma unroll
       for (int i = 0; i < 16; i++)
-        a.b[rb][cb][i] = g[(size_t)(r0 + 32 * rb + 8 * (i >> 2) + 4 * h + (i & 3)) * ld + c0 + 32 * cb + c];
+        a.b[rb][cb][i] = g_ldf(g, vo, off + ((r0 + 32 * rb + 8 * (i >> 2) + (i & 3)) * ld + c0 + 32 * cb) * 4);
 }
 template <int RB, int CB>
-TTT_DEV void acc_store_rows(const AccT<RB, CB>& a, float* g, int ld, int r0, int c0, int c, int h) {
+TTT_DEV void acc_store_rows(const AccT<RB, CB>& a, gptr_t g, unsigned off, int ld, int r0, int c0, int c, int h) {
+  const unsigned vo = (4 * h * ld + c) * 4;
 #pragma unroll
   for (int rb = 0; rb < RB; rb++)
 #pragma unroll
     for (int cb = 0; cb < CB; cb++)
 #pragma unroll
       for (int i = 0; i < 16; i++)
-        g[(size_t)(r0 + 32 * rb + 8 * (i >> 2) + 4 * h + (i & 3)) * ld + c0 + 32 * cb + c] = a.b[rb][cb][i];
+        g_stf(g, vo, off + ((r0 + 32 * rb + 8 * (i >> 2) + (i & 3)) * ld + c0 + 32 * cb) * 4, a.b[rb][cb][i]);
 }
 // Same, but accumulator rows are tensor COLUMNS (the tile holds the transpose of the block).
 template <int RB, int CB>
-TTT_DEV void acc_load_cols(AccT<RB, CB>& a, const float* g, int ld, int r0, int c0, int c, int h) {
+TTT_DEV void acc_load_cols(AccT<RB, CB>& a, gptr_t g, unsigned off, int ld, int r0, int c0, int c, int h) {
+  const unsigned vo = (c * ld + 4 * h) * 4;
 #pragma unroll
   for (int rb = 0; rb < RB; rb++)
 #pragma unroll
     for (int cb = 0; cb < CB; cb++)
 #pragma unroll
-      for (int i = 0; i < 16; i++)
-        a.b[rb][cb][i] = g[(size_t)(r0 + 32 * cb + c) * ld + c0 + 32 * rb + 8 * (i >> 2) + 4 * h + (i & 3)];
+      for (int g4 = 0; g4 < 4; g4++) {
+        const f32x4 x = g_ld4f(g, vo, off + ((r0 + 32 * cb) * ld + c0 + 32 * rb + 8 * g4) * 4);
+#pragma unroll
+        for (int e = 0; e < 4; e++) a.b[rb][cb][4 * g4 + e] = x[e];
+      }
 }
 
 // ------------------------------------------------------------------ LayerNorm-lane helpers
@@ -122,12 +132,16 @@ TTT_DEV void ln_store(bf16* p, const float (&x)[8]) {
   *reinterpret_cast<bf16x4*>(p) = a;
   *reinterpret_cast<bf16x4*>(p + 4) = b;
 }
-// dst = bf16(float(dst) + x): the operator accumulates into these outputs.
-TTT_DEV void ln_accumulate(bf16* p, const float (&x)[8]) {
-  bf16x8 v = *reinterpret_cast<const bf16x8*>(p);
+// 8 features of this lane's token to / from a [tok][F] bf16 tile in HBM (16 bytes per lane).
+TTT_DEV void ln_store_g(gptr_t b, unsigned voff, unsigned soff, const float (&x)[8]) {
+  bf16x8 v;
 #pragma unroll
-  for (int e = 0; e < 8; e++) v[e] = (bf16)((float)v[e] + x[e]);
-  *reinterpret_cast<bf16x8*>(p) = v;
+  for (int e = 0; e < 8; e++) v[e] = (bf16)x[e];
+  g_st8h(b, voff, soff, v);
+}
+TTT_DEV void ln_cvt8(float (&x)[8], bf16x8 v) {
+#pragma unroll
+  for (int e = 0; e < 8; e++) x[e] = (float)v[e];
 }
 TTT_DEV void ln_load_f32(float (&x)[8], const float* p) {
   const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
@@ -198,7 +212,6 @@ TTT_DEV void lds_put16(bf16* s_tile, int tid, u32x4 v) {
   d[0] = make_uint2(v[0], v[1]);
   d[1] = make_uint2(v[2], v[3]);
 }
-TTT_DEV void stage_tile(bf16* s_tile, const bf16* g_tile, int tid) { lds_put16(s_tile, tid, reinterpret_cast<const u32x4*>(g_tile)[tid]); }
 
 // ---------------------------------------------------------------- just-in-time operand pieces
 // One MFMA operand piece = 8 bf16 per lane = (free block blk, k-step s).  Loading pieces right
@@ -289,11 +302,11 @@ TTT_DEV bf16x8 cvt8(const f32x4 lo, const f32x4 hi) {
   for (int e = 0; e < 4; e++) { o[e] = (bf16)lo[e]; o[4 + e] = (bf16)hi[e]; }
   return o;
 }
-// Piece (kappa order) straight from a row-major fp32 matrix: lane = row `row`, contraction = columns
-// col0 + 16 s ...
-TTT_DEV bf16x8 piece_from_f32(const float* g, int ld, int row, int col0, int s, int h) {
-  const float* q = g + (size_t)row * ld + col0 + 16 * s + 4 * h;
-  return cvt8(*reinterpret_cast<const f32x4*>(q), *reinterpret_cast<const f32x4*>(q + 8));
+// Piece (kappa order) straight from a row-major fp32 matrix in HBM: lane = row row0 + c, contraction =
+// columns col0 + 16 s ...; row0, col0, s wave-uniform.
+TTT_DEV bf16x8 piece_from_f32(gptr_t g, unsigned off, int ld, int row0, int col0, int s, int c, int h) {
+  const unsigned vo = (c * ld + 4 * h) * 4, so = off + (row0 * ld + col0 + 16 * s) * 4;
+  return cvt8(g_ld4f(g, vo, so), g_ld4f(g, vo, so + 32));
 }
 
 // Pair sum of a product z (rows F, column block 0 = the token block this wave keeps, column block 1 =
@@ -328,12 +341,12 @@ struct Staged3 {
   u32x4 a, b, c;
   float eta;
 };
-TTT_DEV void stage3_load(Staged3& s, const bf16* ga, const bf16* gb, const bf16* gc, const bf16* geta, size_t tile_off,
-                         size_t eta_off, int tid) {
-  s.a = reinterpret_cast<const u32x4*>(ga + tile_off)[tid];
-  s.b = reinterpret_cast<const u32x4*>(gb + tile_off)[tid];
-  s.c = reinterpret_cast<const u32x4*>(gc + tile_off)[tid];
-  s.eta = (tid < CS) ? bf2f(geta[eta_off + tid]) : 0.f;
+// `mb` = mini-batch index inside this (batch, head); t16 = 16 * tid.
+TTT_DEV void stage3_load(Staged3& s, gptr_t ga, gptr_t gb, gptr_t gc, gptr_t geta, int mb, int tid, unsigned t16) {
+  s.a = g_ld16(ga, t16, mb * TILE_BYTES);
+  s.b = g_ld16(gb, t16, mb * TILE_BYTES);
+  s.c = g_ld16(gc, t16, mb * TILE_BYTES);
+  s.eta = bf2f(g_ldh(geta, 2 * (tid & (CS - 1)), mb * (CS * 2)));   // in bounds for every thread; threads >= CS drop it
 }
 TTT_DEV void stage3_store(const Staged3& s, bf16* sa, bf16* sb, bf16* sc, float* s_eta, int tid) {
   lds_put16(sa, tid, s.a);
@@ -342,41 +355,20 @@ TTT_DEV void stage3_store(const Staged3& s, bf16* sa, bf16* sb, bf16* sc, float*
   if (tid < CS) s_eta[tid] = s.eta;
 }
 
-// What the first stages of one reverse step read from HBM (per thread): all requests are issued
-// together at the top of the step.
-struct RevIn {
-  u32x4 xq, xk, gz;          // chunk tid of the XQ, XK and dl/dZ2 tiles
-  float eta;
-  bf16x4 go[2], xh[2];       // LayerNorm lanes: upstream gradient, x_hat of the output LayerNorm
-  float sd;                  //                  and its std
-};
-TTT_DEV void rev_load(RevIn& in, const BwdParams& p, size_t xo, size_t eo, size_t so, size_t to, int tid, int tok, int f0) {
-  in.xq = reinterpret_cast<const u32x4*>(p.XQ + xo)[tid];
-  in.xk = reinterpret_cast<const u32x4*>(p.XK + xo)[tid];
-  in.gz = reinterpret_cast<const u32x4*>(p.grad_l_wrt_Z2_group + so)[tid];
-  in.eta = (tid < CS) ? bf2f(p.last_eta[eo + tid]) : 0.f;
-  const bf16* q = p.grad_L_XQW + xo + tok * FD + f0;
-  in.go[0] = *reinterpret_cast<const bf16x4*>(q);
-  in.go[1] = *reinterpret_cast<const bf16x4*>(q + 4);
-  q = p.x_hat_ln_group + so + tok * FD + f0;
-  in.xh[0] = *reinterpret_cast<const bf16x4*>(q);
-  in.xh[1] = *reinterpret_cast<const bf16x4*>(q + 4);
-  in.sd = p.std_ln_group[to + tok];
-}
-TTT_DEV void ln_cvt(float (&x)[8], const bf16x4 (&v)[2]) {
-#pragma unroll
-  for (int e = 0; e < 4; e++) { x[e] = (float)v[0][e]; x[4 + e] = (float)v[1][e]; }
-}
 // Piece s of W2[shard] before mini-batch j of the group as an operand (lane = hid row, contraction =
 // F): the image the replay stored after mini-batch j-1, or straight from the fp32 checkpoint.
-TTT_DEV bf16x8 w2_before(const bf16* img_prev, const float* ck, int j, int s, int row, int h, int tid) {
-  return (j > 0) ? chunk_load(img_prev, s, tid) : piece_from_f32(ck, FD, row, 0, s, h);
+TTT_DEV bf16x8 w2_before(gptr_t img, gptr_t ck, unsigned ck_off, int j, int s, int hid0, int c, int h, unsigned t16) {
+  // the image offset is clamped so that the load stays inside the buffer even if it is hoisted above the branch
+  bf16x8 r = chunk_load(img, (j > 0 ? j - 1 : 0) * IMG_BYTES, s, t16);
+  if (j == 0) r = piece_from_f32(ck, ck_off, FD, hid0, 0, s, c, h);
+  return r;
 }
-// Piece (chunk n = 2*rb + s) of W1[:, shard]^T before mini-batch j (lane = F row, contraction = hid).
-TTT_DEV bf16x8 w1_before(const bf16* img_prev, const float* ck, int j, int n, int row, int col0, int s, int h, int tid) {
-  return (j > 0) ? chunk_load(img_prev, n, tid) : piece_from_f32(ck, HID, row, col0, s, h);
+// Piece (row block rb, k-step s) of W1[:, shard]^T before mini-batch j (lane = F row, contraction = hid).
+TTT_DEV bf16x8 w1_before(gptr_t img, gptr_t ck, unsigned ck_off, int j, int rb, int s, int hid0, int c, int h, unsigned t16) {
+  bf16x8 r = chunk_load(img, (j > 0 ? j - 1 : 0) * IMG_BYTES, 2 * rb + s, t16);
+  if (j == 0) r = piece_from_f32(ck, ck_off, HID, 32 * rb, hid0, s, c, h);
+  return r;
 }
-
 
 __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -396,7 +388,8 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
   float* s_deta = reinterpret_cast<float*>(smem + SB_DETA);
   float* s_red = reinterpret_cast<float*>(smem + SB_RED);
 
-  const int tid = threadIdx.x, v = tid >> 6, lane = tid & 63, h = lane >> 5, c = lane & 31;
+  const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5, c = lane & 31;
+  const int v = __builtin_amdgcn_readfirstlane(tid >> 6);        // wave index, in a scalar register
   const int pp = v & 3, r = v >> 2;                              // pair, index inside the pair
   const int tb[2] = {r, 1 - r};                                  // token block held in column block 0 / 1 of a Q tile
   const int q8 = lane >> 3, tok = 8 * v + q8, f0 = 8 * (lane & 7);   // LayerNorm ownership (token block r)
@@ -429,46 +422,83 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
 #pragma unroll
   for (int j = 0; j < 8; j++) ones[j] = (bf16)1.0f;
 
-  const size_t x_base = (size_t)bh * p.NC * (CS * FD);
-  const size_t eta_base = (size_t)bh * p.NC * CS;
-  // per-(b,h) scratch bases
-  const size_t g_TF = (size_t)bh * cgs * (CS * FD);     // [cgs][64][64] tiles
-  const size_t g_TH = (size_t)bh * cgs * (CS * HID);    // [cgs][64][256] tiles (register images)
-  const size_t g_T = (size_t)bh * cgs * CS;             // [cgs][64] vectors
-  float* park_W1 = p.W1_init_group + (size_t)bh * cgs * FD * HID;
-  float* park_W2 = p.W2_init_group + (size_t)bh * cgs * HID * FD;
-  // During the reverse walk the same two 64 KiB slots park what must survive the LayerNorm stage.
-  bf16* park_d1 = reinterpret_cast<bf16*>(park_W1);                  // 32 KiB register image
-  bf16* park_t2 = park_d1 + CS * HID;                                // 32 KiB register image
-  bf16* park_g1 = reinterpret_cast<bf16*>(park_W2);                  // 32 KiB register image
+  // Buffers: base = this (batch, head)'s part of each tensor; offsets inside stay below 2 GiB (checked
+  // by the launcher).  Per-lane offsets: t16 = chunk / tile staging, vln = this LayerNorm lane's 8
+  // features of its token in a [tok][F] bf16 tile, vtok = its token in a [tok] fp32 vector.
+  // Element offsets of this (batch, head) inside each class of tensor.  A buffer descriptor is built
+  // where it is used, from the kernel argument and one of these offsets; the offsets are made opaque
+  // to the optimiser once per mini-batch (REFRESH_OFFSETS) so that the thirty descriptors are not all
+  // hoisted out of the loops and kept in scalar registers at once.
+  size_t ox = uni64((size_t)bh * p.NC * (CS * FD));     // [NC][64][64] inputs / outputs
+  size_t oe = uni64((size_t)bh * p.NC * CS);            // [NC][64] eta, d eta
+  size_t of = uni64((size_t)bh * cgs * (CS * FD));      // [cgs][64][64] scratch tiles
+  size_t oh = uni64((size_t)bh * cgs * (CS * HID));     // [cgs][64][256] scratch tiles (register images)
+  size_t ot = uni64((size_t)bh * cgs * CS);             // [cgs][64] scratch vectors
+  size_t opk = uni64((size_t)bh * cgs * (FD * HID));    // W1_init_group / W2_init_group
+  size_t ock = uni64((size_t)bh * p.K * (FD * HID));    // W1 / W2 checkpoints
+  // The tensor pointers are read from the kernel-argument segment (scalar loads) where they are used,
+  // through a pointer that is refreshed with the offsets, instead of all fifty living in scalar registers.
+  typedef const __attribute__((address_space(4))) BwdParams* KernArgs;
+  KernArgs ka = (KernArgs)__builtin_amdgcn_kernarg_segment_ptr();
+#define REFRESH_OFFSETS() asm volatile("" : "+s"(ka), "+s"(ox), "+s"(oe), "+s"(of), "+s"(oh), "+s"(ot), "+s"(opk), "+s"(ock))
+#define bXQ gbuf(ka->XQ + ox)
+#define bXK gbuf(ka->XK + ox)
+#define bXV gbuf(ka->XV + ox)
+#define bGO gbuf(ka->grad_L_XQW + ox)
+#define bETA gbuf(ka->last_eta + oe)
+#define bZ1 gbuf(ka->Z1_group + oh)
+#define bZ1B gbuf(ka->Z1_bar_group + oh)
+#define bIMG1 gbuf(ka->X2_group + oh)
+#define bIMG2 gbuf(ka->grad_l_wrt_Z1_group + oh)
+#define bXHF gbuf(ka->x_hat_fused_group + of)
+#define bGOF gbuf(ka->grad_output_fused_group + of)
+#define bGZ2 gbuf(ka->grad_l_wrt_Z2_group + of)
+#define bXHL gbuf(ka->x_hat_ln_group + of)
+#define bSDF gbuf(ka->std_fused_group + ot)
+#define bSDL gbuf(ka->std_ln_group + ot)
+  // While a group is replayed the running gradients are parked in W*_init_group; during the reverse
+  // walk the same two 64 KiB slots park what must survive the LayerNorm stage (three 32 KiB images).
+#define bPW1 gbuf(ka->W1_init_group + opk)
+#define bPW2 gbuf(ka->W2_init_group + opk)
+  constexpr unsigned PARK_D1 = 0, PARK_T2 = IMG_BYTES, PARK_G1 = 0;   // d1, t2 in bPW1; g1 in bPW2
+#define bCW1 gbuf(ka->W1_ck + ock)
+#define bCW2 gbuf(ka->W2_ck + ock)
+#define bDXQ gbuf(ka->grad_L_XQ + ox)
+#define bDXK gbuf(ka->grad_L_XK + ox)
+#define bDXV gbuf(ka->grad_L_XV + ox)
+#define bDETA gbuf(ka->grad_L_last_eta + oe)
+  const unsigned t16 = 16 * tid, vln = (tok * FD + f0) * 2, vtok = 4 * tok;
 
   // running gradients wrt the state after the last mini-batch
   AccT<2, 1> gW1s;
   AccT<1, 2> gW2s;
-  acc_load_rows(gW1s, p.grad_L_W1_last + (size_t)bh * FD * HID, HID, 0, hid0, c, h);
-  acc_load_rows(gW2s, p.grad_L_W2_last + (size_t)bh * HID * FD, FD, hid0, 0, c, h);
+  acc_load_rows(gW1s, gbuf(p.grad_L_W1_last + (size_t)bh * FD * HID), 0, HID, 0, hid0, c, h);
+  acc_load_rows(gW2s, gbuf(p.grad_L_W2_last + (size_t)bh * HID * FD), 0, FD, hid0, 0, c, h);
 
   for (int k = p.K - 1; k >= 0; k--) {
     const int n_mb = min(cgs, p.NC - k * cgs);
+    REFRESH_OFFSETS();
     const size_t slot = (size_t)bh * p.K + k;
+    const unsigned ckW = k * (FD * HID * 4);   // byte offset of this group's checkpoint in bCW1 / bCW2
     // ================================================================= replay
     {
       // park the running gradients while the forward state needs the registers
-      acc_store_rows(gW1s, park_W1, HID, 0, hid0, c, h);
-      acc_store_rows(gW2s, park_W2, FD, hid0, 0, c, h);
+      acc_store_rows(gW1s, bPW1, 0, HID, 0, hid0, c, h);
+      acc_store_rows(gW2s, bPW2, 0, FD, hid0, 0, c, h);
       AccT<2, 1> W1s, W2t;
       AccT<1, 2> W2s;
-      acc_load_rows(W1s, p.W1_ck + slot * FD * HID, HID, 0, hid0, c, h);
-      acc_load_rows(W2s, p.W2_ck + slot * HID * FD, FD, hid0, 0, c, h);
-      acc_load_cols(W2t, p.W2_ck + slot * HID * FD, FD, hid0, 0, c, h);
+      acc_load_rows(W1s, bCW1, ckW, HID, 0, hid0, c, h);
+      acc_load_rows(W2s, bCW2, ckW, FD, hid0, 0, c, h);
+      acc_load_cols(W2t, bCW2, ckW, FD, hid0, 0, c, h);
       __syncthreads();  // previous group's readers of the bias vectors are done
       if (tid < HID) s_b1[tid] = p.b1_ck[slot * HID + tid];
       if (tid < FD) s_b2[tid] = p.b2_ck[slot * FD + tid];
 
       Staged3 st;
-      stage3_load(st, p.XQ, p.XK, p.XV, p.last_eta, x_base + (size_t)(k * cgs) * (CS * FD), eta_base + (size_t)(k * cgs) * CS, tid);
+      stage3_load(st, bXQ, bXK, bXV, bETA, k * cgs, tid, t16);
       for (int j = 0; j < n_mb; j++) {
         const int mb = k * cgs + j;
+        REFRESH_OFFSETS();
         __syncthreads();
         stage3_store(st, s_xq, s_xk, s_e2, s_eta, tid);
         __syncthreads();
@@ -480,12 +510,11 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
           acc_init_rows_lds(x2, s_b1w, h);
           mma_jit<4>(x2, [&](int, int s) { return piece_state(W1s, 0, s); },
                      [&](int i, int s) { return piece_rows<LDX>(s_xk, tb[i], s, c, h); });
-          bf16* img = p.Z1_group + g_TH + (size_t)j * (CS * HID);
 #pragma unroll
           for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int t = 0; t < 2; t++) {
-              chunk_store(img, 2 * tb[i] + t, tid, pack8(x2.b[0][i], t));
+              chunk_store(bZ1, j * IMG_BYTES, 2 * tb[i] + t, t16, pack8(x2.b[0][i], t));
               bf16x8 xv;
 #pragma unroll
               for (int jj = 0; jj < 8; jj++) {
@@ -530,18 +559,17 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
               gx[e] = go[e] * gam[e];
             }
           }
-          const size_t so = g_TF + (size_t)j * (CS * FD) + tok * FD + f0;
-          ln_store(p.x_hat_fused_group + so, z);
-          ln_store(p.grad_output_fused_group + so, go);
+          ln_store_g(bXHF, vln, j * TILE_BYTES, z);
+          ln_store_g(bGOF, vln, j * TILE_BYTES, go);
           const float s1 = oct_sum(sum8(gx)), s2 = oct_sum(dot8(gx, z));
           const float sc = rstd * (1.f / FD), neg_eta = -s_eta[tok];
 #pragma unroll
           for (int e = 0; e < 8; e++) gx[e] = (FD * gx[e] - s1 - z[e] * s2) * sc;   // dl/dZ2
-          ln_store(p.grad_l_wrt_Z2_group + so, gx);
+          ln_store_g(bGZ2, vln, j * TILE_BYTES, gx);
 #pragma unroll
           for (int e = 0; e < 8; e++) gx[e] *= neg_eta;                             // G2
           ln_store(s_gz2 + tok * LDX + f0, gx);
-          if ((lane & 7) == 0) p.std_fused_group[g_T + (size_t)j * CS + tok] = sd;
+          if ((lane & 7) == 0) g_stf(bSDF, vtok, j * (CS * 4), sd);
         }
         __syncthreads();
         // G1 = (W2 G2^T) * gelu'(Z1)  (rows hid, lane = tok) -> T1 rows [tok][hid]; weight step
@@ -571,16 +599,15 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
         lds_rowsum_add_jit(s_b1w, [&](int s) { return piece_tr<LDH>(T1, 0, s, lane); }, ones, c, h);
         // operand images of the state after this step, for the reverse walk
         {
-          bf16* img2 = p.grad_l_wrt_Z1_group + g_TH + (size_t)j * (CS * HID);   // W2: lane = hid, contraction = F
-          bf16* img1 = p.X2_group + g_TH + (size_t)j * (CS * HID);              // W1^T: lane = F, contraction = hid
+          // bIMG2: W2, lane = hid, contraction = F;  bIMG1: W1^T, lane = F, contraction = hid
           store_state_rows<LDF>(T2, W1s, c, h);                                 // rows [hid][F]
 #pragma unroll
-          for (int s = 0; s < 4; s++) chunk_store(img2, s, tid, piece_state(W2t, 0, s));
+          for (int s = 0; s < 4; s++) chunk_store(bIMG2, j * IMG_BYTES, s, t16, piece_state(W2t, 0, s));
           WAVE_SYNC();
 #pragma unroll
           for (int fb = 0; fb < 2; fb++)
 #pragma unroll
-            for (int s = 0; s < 2; s++) chunk_store(img1, 2 * fb + s, tid, piece_tr<LDF>(T2, fb, s, lane));
+            for (int s = 0; s < 2; s++) chunk_store(bIMG1, j * IMG_BYTES, 2 * fb + s, t16, piece_tr<LDF>(T2, fb, s, lane));
         }
         // post-update forward on XQ
         {
@@ -588,13 +615,12 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
           acc_init_rows_lds(z1b, s_b1w, h);
           mma_jit<4>(z1b, [&](int, int s) { return piece_state(W1s, 0, s); },
                      [&](int i, int s) { return piece_rows<LDX>(s_xq, tb[i], s, c, h); });
-          bf16* img = p.Z1_bar_group + g_TH + (size_t)j * (CS * HID);
           bf16x8 x2bQ[2][2];
 #pragma unroll
           for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int t = 0; t < 2; t++) {
-              chunk_store(img, 2 * tb[i] + t, tid, pack8(z1b.b[0][i], t));
+              chunk_store(bZ1B, j * IMG_BYTES, 2 * tb[i] + t, t16, pack8(z1b.b[0][i], t));
 #pragma unroll
               for (int jj = 0; jj < 8; jj++) x2bQ[i][t][jj] = (bf16)gelu_f(z1b.b[0][i][8 * t + jj]);
             }
@@ -603,7 +629,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
           mma_jit<2>(z2, [&](int rb, int s) { return piece_state(W2s, rb, s); },
                      [&](int i, int s) { return x2bQ[i][s]; });
           if (j + 1 < n_mb)
-            stage3_load(st, p.XQ, p.XK, p.XV, p.last_eta, x_base + (size_t)(mb + 1) * (CS * FD), eta_base + (size_t)(mb + 1) * CS, tid);
+            stage3_load(st, bXQ, bXK, bXV, bETA, mb + 1, tid, t16);
           WAVE_SYNC();   // this wave's readers of T1 / T2 are done
           pair_sum(s_own, s_partner, z2, c, h);
         }
@@ -615,52 +641,52 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
           for (int e = 0; e < 8; e++) z[e] += b2v[e];
           float sd;
           ln_normalize(z, &sd);
-          ln_store(p.x_hat_ln_group + g_TF + (size_t)j * (CS * FD) + tok * FD + f0, z);
-          if ((lane & 7) == 0) p.std_ln_group[g_T + (size_t)j * CS + tok] = sd;
+          ln_store_g(bXHL, vln, j * TILE_BYTES, z);
+          if ((lane & 7) == 0) g_stf(bSDL, vtok, j * (CS * 4), sd);
         }
       }
       // running gradients back into registers
-      acc_load_rows(gW1s, park_W1, HID, 0, hid0, c, h);
-      acc_load_rows(gW2s, park_W2, FD, hid0, 0, c, h);
+      acc_load_rows(gW1s, bPW1, 0, HID, 0, hid0, c, h);
+      acc_load_rows(gW2s, bPW2, 0, FD, hid0, 0, c, h);
     }
 
     // ================================================================= reverse walk
     // Operands are fetched from HBM right where they are consumed: with two waves per SIMD the other
     // wave covers the latency, while holding requests in registers across stages costs more in spills
     // than it gains (measured).
-    const float* ckW1 = p.W1_ck + slot * FD * HID;
-    const float* ckW2 = p.W2_ck + slot * HID * FD;
-    RevIn in;
     for (int j = n_mb - 1; j >= 0; j--) {
       const int mb = k * cgs + j;
-      const size_t xo = x_base + (size_t)mb * (CS * FD);
-      const size_t so = g_TF + (size_t)j * (CS * FD);
-      const size_t ho = g_TH + (size_t)j * (CS * HID);
+      REFRESH_OFFSETS();
+      const unsigned xo = mb * TILE_BYTES;       // this mini-batch in the input / output tensors
+      const unsigned so = j * TILE_BYTES;        // its slot in the [cgs][64][64] scratch tensors
+      const unsigned ho = j * IMG_BYTES;         // its slot in the [cgs][64][256] scratch tensors
       // eta of the token this lane holds in column block i of a Q-orientation tile
-      const float eta_i[2] = {bf2f(p.last_eta[eta_base + (size_t)mb * CS + 32 * tb[0] + c]),
-                              bf2f(p.last_eta[eta_base + (size_t)mb * CS + 32 * tb[1] + c])};
+      const float eta_i[2] = {bf2f(g_ldh(bETA, 2 * c, mb * (CS * 2) + 64 * tb[0])), bf2f(g_ldh(bETA, 2 * c, mb * (CS * 2) + 64 * tb[1]))};
       __syncthreads();
-      rev_load(in, p, xo, eta_base + (size_t)mb * CS, so, g_T + (size_t)j * CS, tid, tok, f0);
-      lds_put16(s_xq, tid, in.xq);
-      lds_put16(s_xk, tid, in.xk);
-      lds_put16(s_gz2, tid, in.gz);
-      if (tid < CS) s_eta[tid] = in.eta;
+      {
+        const u32x4 xq = g_ld16(bXQ, t16, xo), xk = g_ld16(bXK, t16, xo), gz = g_ld16(bGZ2, t16, so);
+        const float eta = bf2f(g_ldh(bETA, 2 * (tid & (CS - 1)), mb * (CS * 2)));
+        lds_put16(s_xq, tid, xq);
+        lds_put16(s_xk, tid, xk);
+        lds_put16(s_gz2, tid, gz);
+        if (tid < CS) s_eta[tid] = eta;
+      }
       // operand tiles of the state after this step: T1 = W2 rows [hid][F], T2 = W1^T rows [F][hid]
 #pragma unroll
-      for (int s = 0; s < 4; s++) store_piece_rows<LDF>(T1, 0, s, c, h, chunk_load(p.grad_l_wrt_Z1_group + ho, s, tid));
+      for (int s = 0; s < 4; s++) store_piece_rows<LDF>(T1, 0, s, c, h, chunk_load(bIMG2, ho, s, t16));
 #pragma unroll
       for (int fb = 0; fb < 2; fb++)
 #pragma unroll
-        for (int s = 0; s < 2; s++) store_piece_rows<LDH>(T2, fb, s, c, h, chunk_load(p.X2_group + ho, 2 * fb + s, tid));
+        for (int s = 0; s < 2; s++) store_piece_rows<LDH>(T2, fb, s, c, h, chunk_load(bIMG1, ho, 2 * fb + s, t16));
 
       // ---- output LayerNorm backward (LayerNorm lanes)
       float gO[8];
       {
         float xh[8], gx[8], gam[8];
-        ln_cvt(gO, in.go);
-        ln_cvt(xh, in.xh);
+        ln_cvt8(gO, g_ld8h(bGO, vln, xo));
+        ln_cvt8(xh, g_ld8h(bXHL, vln, so));
         ln_load_f32(gam, s_gam + f0);
-        const float sd = in.sd;
+        const float sd = g_ldf(bSDL, vtok, j * (CS * 4));
 #pragma unroll
         for (int e = 0; e < 8; e++) gx[e] = gO[e] * xh[e];
         ln_token_sum_add(s_dbw, gO, q8, f0);
@@ -691,7 +717,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
             for (int t = 0; t < 2; t++) {
               bf16x8 x2b, gzb;
               bf16x8 zcb[2][2];
-              zcb[i][t] = chunk_load(p.Z1_bar_group + ho, 2 * tb[i] + t, tid);
+              zcb[i][t] = chunk_load(bZ1B, ho, 2 * tb[i] + t, t16);
 #pragma unroll
               for (int jj = 0; jj < 8; jj++) {
                 float g, d;
@@ -720,25 +746,23 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
       {
         float z[8];
         ln_gather(z, s_lnrow);
-        dxq_old = *reinterpret_cast<const bf16x8*>(p.grad_L_XQ + xo + tok * FD + f0);
+        dxq_old = g_ld8h(bDXQ, vln, xo);
 #pragma unroll
         for (int e = 0; e < 8; e++) dxq_old[e] = (bf16)((float)dxq_old[e] + (z[e] + gO[e]));
-        *reinterpret_cast<bf16x8*>(p.grad_L_XQ + xo + tok * FD + f0) = dxq_old;
+        g_st8h(bDXQ, vln, xo, dxq_old);
       }
       __syncthreads();  // dXQ readers of the regions are done: T1 / T2 are free again
 
       // ---- the weight step, backwards (uses the state BEFORE this mini-batch).
       //      Parked across the LayerNorm stage: X2 in T0; packed d1 = gelu'(Z1), g1 = -eta * dl/dZ1 and
       //      t2 = -eta * (gZ2 W2^T) * (XK gW1 + gb1) * gelu''(Z1).
-      bf16x4 xhf[2], gof[2];     // LayerNorm lanes: x_hat / grad_output of the fused loss, its std,
-      float sdf;                 // and the two outputs the stage accumulates into
-      bf16x8 dxv_old;
+      bf16x8 dxv_old;            // LayerNorm lanes: the two outputs the stage accumulates into
       bf16 deta_old;
       {
         // T1 = W2 before the step, rows [hid][F]; T2 = gW1, rows [hid][F]
 #pragma unroll
         for (int s = 0; s < 4; s++)
-          store_piece_rows<LDF>(T1, 0, s, c, h, w2_before(p.grad_l_wrt_Z1_group + ho - CS * HID, ckW2, j, s, hid0 + c, h, tid));
+          store_piece_rows<LDF>(T1, 0, s, c, h, w2_before(bIMG2, bCW2, ckW, j, s, hid0, c, h, t16));
         store_state_rows<LDF>(T2, gW1s, c, h);
         WAVE_SYNC();
         AccT<2, 2> pz;
@@ -754,7 +778,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
           mma_jit<4>(S, [&](int, int s) { return piece_rows<LDF>(T2, 0, s, c, h); },
                      [&](int, int s) { return piece_rows<LDX>(s_xk, tb[i], s, c, h); });
           bf16x8 x2c[2], uc[2];
-          const bf16x8 zc[2] = {chunk_load(p.Z1_group + ho, 2 * tb[i], tid), chunk_load(p.Z1_group + ho, 2 * tb[i] + 1, tid)};
+          const bf16x8 zc[2] = {chunk_load(bZ1, ho, 2 * tb[i], t16), chunk_load(bZ1, ho, 2 * tb[i] + 1, t16)};
 #pragma unroll
           for (int t = 0; t < 2; t++) {
             bf16x8 d1c, t2c, g1c;
@@ -773,9 +797,9 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
             }
             // nothing stays in registers across the LayerNorm stage: d1, g1 and t2 go to their parks at
             // once (L2-resident, rewritten every mini-batch; 1 KiB per wave instruction)
-            chunk_store(park_d1, 2 * tb[i] + t, tid, d1c);
-            chunk_store(park_t2, 2 * tb[i] + t, tid, t2c);
-            chunk_store(park_g1, 2 * tb[i] + t, tid, g1c);
+            chunk_store(bPW1, PARK_D1, 2 * tb[i] + t, t16, d1c);
+            chunk_store(bPW1, PARK_T2, 2 * tb[i] + t, t16, t2c);
+            chunk_store(bPW2, PARK_G1, 2 * tb[i] + t, t16, g1c);
             store_piece_rows<LDH>(T0, tb[i], t, c, h, x2c[t]);             // X2 rows [tok][hid]
           }
           // pz[:, i] = gW2^T X2^T ; dEta partial ; + W2^T u^T
@@ -808,24 +832,17 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
       {
         float gy[8];
         float gg[8], xh[8], go[8], gz[8], gam[8], gb[8];
-        dxv_old = *reinterpret_cast<const bf16x8*>(p.grad_L_XV + xo + tok * FD + f0);
-        deta_old = p.grad_L_last_eta[eta_base + (size_t)mb * CS + tok];
-        {
-          const bf16* q = p.x_hat_fused_group + so + tok * FD + f0;
-          xhf[0] = *reinterpret_cast<const bf16x4*>(q);
-          xhf[1] = *reinterpret_cast<const bf16x4*>(q + 4);
-          q = p.grad_output_fused_group + so + tok * FD + f0;
-          gof[0] = *reinterpret_cast<const bf16x4*>(q);
-          gof[1] = *reinterpret_cast<const bf16x4*>(q + 4);
-          sdf = p.std_fused_group[g_T + (size_t)j * CS + tok];
-        }
+        dxv_old = g_ld8h(bDXV, vln, xo);
+        deta_old = g_ldh(bDETA, 2 * tok, mb * (CS * 2));
+        const bf16x8 xhf = g_ld8h(bXHF, vln, so), gof = g_ld8h(bGOF, vln, so);
+        const float sdf = g_ldf(bSDF, vtok, j * (CS * 4));
         ln_gather(gg, s_lnrow);
         ln_load_f32(gb, s_gb2 + f0);
         const float neg_eta = -s_eta[tok];
 #pragma unroll
         for (int e = 0; e < 8; e++) gg[e] = (gg[e] + gb[e]) * neg_eta;   // grad wrt dl/dZ2
-        ln_cvt(xh, xhf);
-        ln_cvt(go, gof);
+        ln_cvt8(xh, xhf);
+        ln_cvt8(go, gof);
         ln_load(gz, s_gz2 + tok * LDX + f0);
         ln_load_f32(gam, s_gam + f0);
         const float rsd = 1.f / sdf;
@@ -834,7 +851,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
           float tot = oct_sum(dot8(gz, gb));
 #pragma unroll
           for (int u = 0; u < BW_NWAVE; u++) tot += s_deta[u * CS + tok];
-          if ((lane & 7) == 0) p.grad_L_last_eta[eta_base + (size_t)mb * CS + tok] = (bf16)((float)deta_old - tot);
+          if ((lane & 7) == 0) g_sth(bDETA, 2 * tok, mb * (CS * 2), (bf16)((float)deta_old - tot));
         }
         const float s0 = oct_sum(sum8(gg)), a = oct_sum(dot8(gg, xh));
         float bb = 0.f;
@@ -869,7 +886,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
           *reinterpret_cast<f32x4*>(s_gy + 4) = hi;
         }
         ln_store(s_a + tok * LDX + f0, gx);
-        *reinterpret_cast<bf16x8*>(p.grad_L_XV + xo + tok * FD + f0) = dxv_old;
+        g_st8h(bDXV, vln, xo, dxv_old);
       }
       __syncthreads();  // dZ2 tile complete; regions (T1 / T2) free again
 
@@ -878,7 +895,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
       {
         bf16x8 w2b[4];   // W2 before the step: lane = hid, contraction = F
 #pragma unroll
-        for (int s = 0; s < 4; s++) w2b[s] = w2_before(p.grad_l_wrt_Z1_group + ho - CS * HID, ckW2, j, s, hid0 + c, h, tid);
+        for (int s = 0; s < 4; s++) w2b[s] = w2_before(bIMG2, bCW2, ckW, j, s, hid0, c, h, t16);
         // T2 = gW1 rows [hid][F] (for S again and for gW1 G1^T), T1 = gW2 rows [F][hid] (transposed
         // read gives lane = hid)
         store_state_rows<LDF>(T2, gW1s, c, h);
@@ -901,9 +918,9 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
           mma_jit<4>(dx2, [&](int, int s) { return w2b[s]; },                                  // + dZ2 W2^T
                      [&](int, int s) { return piece_rows<LDX>(s_a, tb[i], s, c, h); });
           // dk[:, i] = gW1 G1^T  (gW1: lane = F, contraction = hid)
-          const bf16x8 g1c[2] = {chunk_load(park_g1, 2 * tb[i], tid), chunk_load(park_g1, 2 * tb[i] + 1, tid)};
-          const bf16x8 d1c[2] = {chunk_load(park_d1, 2 * tb[i], tid), chunk_load(park_d1, 2 * tb[i] + 1, tid)};
-          const bf16x8 t2c[2] = {chunk_load(park_t2, 2 * tb[i], tid), chunk_load(park_t2, 2 * tb[i] + 1, tid)};
+          const bf16x8 g1c[2] = {chunk_load(bPW2, PARK_G1, 2 * tb[i], t16), chunk_load(bPW2, PARK_G1, 2 * tb[i] + 1, t16)};
+          const bf16x8 d1c[2] = {chunk_load(bPW1, PARK_D1, 2 * tb[i], t16), chunk_load(bPW1, PARK_D1, 2 * tb[i] + 1, t16)};
+          const bf16x8 t2c[2] = {chunk_load(bPW1, PARK_T2, 2 * tb[i], t16), chunk_load(bPW1, PARK_T2, 2 * tb[i] + 1, t16)};
 #pragma unroll
           for (int t = 0; t < 2; t++)
 #pragma unroll
@@ -928,7 +945,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
           }
         WAVE_SYNC();
         mma_jit<2>(dk, [&](int rb, int s) {                                                    // + W1 dZ1^T, W1 before the step
-                     return w1_before(p.X2_group + ho - CS * HID, ckW1, j, 2 * rb + s, 32 * rb + c, hid0, s, h, tid); },
+                     return w1_before(bIMG1, bCW1, ckW, j, rb, s, hid0, c, h, t16); },
                    [&](int i, int s) { return dzp[i][s]; });
         mma_jit<4>(gW2s, [&](int, int s) { return piece_tr<LDH>(T2, 0, s, lane); },            // (-eta u)^T: lane = hid
                    [&](int fb, int s) { return piece_tr<LDX>(s_gz2, fb, s, lane); });          // gZ2: lane = F
@@ -946,17 +963,17 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
         float z[8], gyv[8];
         ln_gather(z, s_lnrow);
         ln_load_f32(gyv, s_gy);
-        dxk_old = *reinterpret_cast<const bf16x8*>(p.grad_L_XK + xo + tok * FD + f0);
+        dxk_old = g_ld8h(bDXK, vln, xo);
 #pragma unroll
         for (int e = 0; e < 8; e++) dxk_old[e] = (bf16)((float)dxk_old[e] + (z[e] + gyv[e]));
-        *reinterpret_cast<bf16x8*>(p.grad_L_XK + xo + tok * FD + f0) = dxk_old;
+        g_st8h(bDXK, vln, xo, dxk_old);
       }
     }
   }
 
   // ---- outputs that are written once
-  acc_store_rows(gW1s, p.grad_L_W1_init + (size_t)bh * FD * HID, HID, 0, hid0, c, h);
-  acc_store_rows(gW2s, p.grad_L_W2_init + (size_t)bh * HID * FD, FD, hid0, 0, c, h);
+  acc_store_rows(gW1s, gbuf(p.grad_L_W1_init + (size_t)bh * FD * HID), 0, HID, 0, hid0, c, h);
+  acc_store_rows(gW2s, gbuf(p.grad_L_W2_init + (size_t)bh * HID * FD), 0, FD, hid0, 0, c, h);
   __syncthreads();
   if (tid < HID) p.grad_L_b1_init[(size_t)bh * HID + tid] = s_gb1[tid];
   if (tid < FD) p.grad_L_b2_init[(size_t)bh * FD + tid] = s_gb2[tid];
@@ -969,6 +986,30 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
     (which == 0 ? p.grad_L_ttt_norm_weight : p.grad_L_ttt_norm_bias)[(size_t)bh * FD + f] = s;
   }
 }
+#undef REFRESH_OFFSETS
+#undef bXQ
+#undef bXK
+#undef bXV
+#undef bGO
+#undef bETA
+#undef bZ1
+#undef bZ1B
+#undef bIMG1
+#undef bIMG2
+#undef bXHF
+#undef bGOF
+#undef bGZ2
+#undef bXHL
+#undef bSDF
+#undef bSDL
+#undef bPW1
+#undef bPW2
+#undef bCW1
+#undef bCW2
+#undef bDXQ
+#undef bDXK
+#undef bDXV
+#undef bDETA
 
 }  // namespace ttt
 

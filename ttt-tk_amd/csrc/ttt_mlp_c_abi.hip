@@ -17,6 +17,8 @@ int check_sizes(int B, int NH, int NC, int K, int cgs) {
   if (B <= 0 || NH <= 0 || NC <= 0 || K <= 0 || cgs <= 0) return TTT_MLP_ERR_BAD_ARG;
   if ((long long)K != ((long long)NC + cgs - 1) / cgs) return TTT_MLP_ERR_BAD_CKPT;
   if ((long long)B * NH > 0x7fffffffLL) return TTT_MLP_ERR_TOO_LARGE;
+  // the kernels address one (batch, head) with 32-bit byte offsets: 8 KiB per mini-batch, 32 KiB per group slot
+  if (NC > (1 << 18) || cgs > (1 << 16)) return TTT_MLP_ERR_TOO_LARGE;
   return TTT_MLP_OK;
 }
 
@@ -33,7 +35,7 @@ extern "C" const char* ttt_mlp_error_string(int code) {
     case TTT_MLP_ERR_BAD_ARG: return "ttt_mlp: null pointer or non-positive size";
     case TTT_MLP_ERR_BAD_CKPT: return "ttt_mlp: number of checkpoints K must equal ceil(NC / checkpoint_group_size)";
     case TTT_MLP_ERR_ALIGN: return "ttt_mlp: every tensor pointer must be 16-byte aligned";
-    case TTT_MLP_ERR_TOO_LARGE: return "ttt_mlp: B*NH exceeds the launch grid limit";
+    case TTT_MLP_ERR_TOO_LARGE: return "ttt_mlp: B*NH exceeds the launch grid limit, or NC > 262144, or checkpoint_group_size > 65536";
     default: return hipGetErrorString(static_cast<hipError_t>(code));
   }
 }

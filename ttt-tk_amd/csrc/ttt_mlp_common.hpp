@@ -258,6 +258,47 @@ TTT_DEV float oct_sum(float x) {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront"); \
   } while (0)
 
+// ---------------------------------------------------------------------------- HBM addressing
+// Every HBM access of the kernels is "wave-uniform 64-bit base + wave-uniform 32-bit offset + 32-bit
+// per-lane offset".  Written this way the uniform parts stay in scalar registers (global_load /
+// global_store with a scalar base and a 32-bit vector offset), so a lane needs one offset register
+// per access pattern instead of one 64-bit address per access.  Buffer (MUBUF) instructions would
+// give the same economy but must not be mixed with scratch traffic: the two kinds of load do not
+// return in issue order on this hardware while the compiler counts them as one in-order stream.
+typedef const __attribute__((address_space(1))) char* gptr_t;   // global address space: global_load / global_store
+TTT_DEV unsigned uni(unsigned x) { return __builtin_amdgcn_readfirstlane(x); }   // pins a wave-uniform value to a scalar register
+TTT_DEV uint64_t uni64(uint64_t a) {
+  return (static_cast<uint64_t>(uni(static_cast<unsigned>(a >> 32))) << 32) | uni(static_cast<unsigned>(a));
+}
+TTT_DEV gptr_t gbuf(const void* base) { return (gptr_t)uni64(reinterpret_cast<uint64_t>(base)); }
+template <class T>
+TTT_DEV T g_ld(gptr_t b, unsigned voff, unsigned soff) {
+  typedef const __attribute__((address_space(1))) T* ptr_t;
+  gptr_t q = b + static_cast<uint64_t>(uni(soff));
+  // The empty statements keep the scalar sum in scalar registers and the zero-extension of the lane
+  // offset next to the access, which is what lets the instruction selector use the
+  // "scalar base + 32-bit vector offset" form.
+  asm("" : "+s"(q), "+v"(voff));
+  return *(ptr_t)(q + static_cast<uint64_t>(voff));
+}
+template <class T>
+TTT_DEV void g_st(gptr_t b, unsigned voff, unsigned soff, T v) {
+  typedef __attribute__((address_space(1))) T* ptr_t;
+  gptr_t q = b + static_cast<uint64_t>(uni(soff));
+  asm("" : "+s"(q), "+v"(voff));
+  *(ptr_t)(q + static_cast<uint64_t>(voff)) = v;
+}
+TTT_DEV u32x4 g_ld16(gptr_t b, unsigned voff, unsigned soff) { return g_ld<u32x4>(b, voff, soff); }
+TTT_DEV void g_st16(gptr_t b, unsigned voff, unsigned soff, u32x4 v) { g_st<u32x4>(b, voff, soff, v); }
+TTT_DEV bf16x8 g_ld8h(gptr_t b, unsigned voff, unsigned soff) { return g_ld<bf16x8>(b, voff, soff); }
+TTT_DEV void g_st8h(gptr_t b, unsigned voff, unsigned soff, bf16x8 v) { g_st<bf16x8>(b, voff, soff, v); }
+TTT_DEV f32x4 g_ld4f(gptr_t b, unsigned voff, unsigned soff) { return g_ld<f32x4>(b, voff, soff); }
+TTT_DEV void g_st4f(gptr_t b, unsigned voff, unsigned soff, f32x4 v) { g_st<f32x4>(b, voff, soff, v); }
+TTT_DEV float g_ldf(gptr_t b, unsigned voff, unsigned soff) { return g_ld<float>(b, voff, soff); }
+TTT_DEV void g_stf(gptr_t b, unsigned voff, unsigned soff, float v) { g_st<float>(b, voff, soff, v); }
+TTT_DEV bf16 g_ldh(gptr_t b, unsigned voff, unsigned soff) { return g_ld<bf16>(b, voff, soff); }
+TTT_DEV void g_sth(gptr_t b, unsigned voff, unsigned soff, bf16 v) { g_st<bf16>(b, voff, soff, v); }
+
 // ---------------------------------------------------------------------------- bf16 helpers
 TTT_DEV float bf_lo(uint32_t u) { return __builtin_bit_cast(float, u << 16); }
 TTT_DEV float bf_hi(uint32_t u) { return __builtin_bit_cast(float, u & 0xffff0000u); }
