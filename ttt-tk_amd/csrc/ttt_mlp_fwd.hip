@@ -47,11 +47,14 @@ struct Staged {  // one mini-batch of inputs in flight from HBM: one 16-byte chu
   float eta;
 };
 
-TTT_DEV void stage_load(Staged& s, const FwdParams& p, size_t tile_off, size_t eta_off, int tid) {
-  s.q = reinterpret_cast<const u32x4*>(p.XQ + tile_off)[tid];   // chunk id = tid: row tid / 8, 8 chunks per row
-  s.k = reinterpret_cast<const u32x4*>(p.XK + tile_off)[tid];
-  s.v = reinterpret_cast<const u32x4*>(p.XV + tile_off)[tid];
-  s.eta = (tid < CS) ? bf2f(p.last_eta[eta_off + tid]) : 0.f;
+// gq / gk / gv / ge = this (batch, head)'s XQ, XK, XV, last_eta; thread tid moves 16-byte chunk tid
+// (row tid / 8, 8 chunks per row) of each tile of mini-batch mb.
+constexpr unsigned TILE_BYTES = CS * FD * 2;
+TTT_DEV void stage_load(Staged& s, gptr_t gq, gptr_t gk, gptr_t gv, gptr_t ge, int mb, int tid) {
+  s.q = g_ld16(gq, 16 * tid, mb * TILE_BYTES);
+  s.k = g_ld16(gk, 16 * tid, mb * TILE_BYTES);
+  s.v = g_ld16(gv, 16 * tid, mb * TILE_BYTES);
+  s.eta = bf2f(g_ldh(ge, 2 * (tid & (CS - 1)), mb * (CS * 2)));   // threads >= CS drop it
 }
 
 TTT_DEV void stage_store(const Staged& s, unsigned char* smem, int xq_buf, int tid) {
@@ -108,7 +111,8 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
   float* s_gam = reinterpret_cast<float*>(smem + SM_GAM);
   float* s_bet = reinterpret_cast<float*>(smem + SM_BET);
 
-  const int tid = threadIdx.x, v = tid >> 6, lane = tid & 63, h = lane >> 5, c = lane & 31;
+  const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5, c = lane & 31;
+  const int v = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave index, in a scalar register
   const int pr = v >> 2;                                    // index inside the wave pair (v & 3)
   const int tok = 8 * v + (lane >> 3), f0 = 8 * (lane & 7); // LayerNorm ownership: 8 lanes per token, 8 features each
   const int bh = blockIdx.x, head = bh % p.NH;
@@ -121,16 +125,15 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
   AccT<1, 2> W2s;
   float b1L;      // b1 of hidden column hid0 + c; b2 lives in LDS (fp32) and is updated there by waves 0 and 1
   {
-    const float* W1 = p.W1 + (size_t)bh * FD * HID;
-    const float* W2 = p.W2 + (size_t)bh * HID * FD;
+    const gptr_t W1 = gbuf(p.W1 + (size_t)bh * FD * HID), W2 = gbuf(p.W2 + (size_t)bh * HID * FD);
 #pragma unroll
     for (int b = 0; b < 2; b++)
 #pragma unroll
       for (int i = 0; i < 16; i++) {
-        const int row = 8 * (i >> 2) + 4 * h + (i & 3);
-        W1s.b[b][0][i] = W1[(32 * b + row) * HID + hid0 + c];
-        W2t.b[b][0][i] = W2[(hid0 + c) * FD + 32 * b + row];
-        W2s.b[0][b][i] = W2[(hid0 + row) * FD + 32 * b + c];
+        const int row = 8 * (i >> 2) + (i & 3);   // + 4h in the lane offset
+        W1s.b[b][0][i] = g_ldf(W1, (4 * h * HID + c) * 4, ((32 * b + row) * HID + hid0) * 4);
+        W2t.b[b][0][i] = g_ldf(W2, (c * FD + 4 * h) * 4, (hid0 * FD + 32 * b + row) * 4);
+        W2s.b[0][b][i] = g_ldf(W2, (4 * h * FD + c) * 4, ((hid0 + row) * FD + 32 * b) * 4);
       }
     b1L = p.b1[(size_t)bh * HID + hid0 + c];
     if (tid < HID) s_b1[tid] = p.b1[(size_t)bh * HID + tid];
@@ -144,10 +147,13 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
 #pragma unroll
   for (int j = 0; j < 8; j++) ones[j] = (bf16)1.0f;
 
-  const size_t x_base = (size_t)bh * p.NC * (CS * FD);
-  const size_t eta_base = (size_t)bh * p.NC * CS;
+  // HBM addressing: scalar base of this (batch, head) + scalar offset of the mini-batch + lane offset
+  const size_t x_base = uni64((size_t)bh * p.NC * (CS * FD));
+  const gptr_t gXQ = gbuf(p.XQ + x_base), gXK = gbuf(p.XK + x_base), gXV = gbuf(p.XV + x_base), gOut = gbuf(p.Out + x_base);
+  const gptr_t gEta = gbuf(p.last_eta + uni64((size_t)bh * p.NC * CS));
+  const gptr_t gW1ck = gbuf(p.W1_ck + uni64((size_t)bh * p.K * FD * HID)), gW2ck = gbuf(p.W2_ck + uni64((size_t)bh * p.K * HID * FD));
   Staged st;
-  stage_load(st, p, x_base, eta_base, tid);
+  stage_load(st, gXQ, gXK, gXV, gEta, 0, tid);
   stage_store(st, smem, 0, tid);
   __syncthreads();
 
@@ -157,15 +163,14 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
     // ---- checkpoint: the state before this mini-batch
     if (mb % p.cgs == 0) {
       const size_t slot = (size_t)bh * p.K + mb / p.cgs;
-      float* cW1 = p.W1_ck + slot * FD * HID;
-      float* cW2 = p.W2_ck + slot * HID * FD;
+      const unsigned ck = (mb / p.cgs) * (FD * HID * 4);   // byte offset of the slot in gW1ck / gW2ck
 #pragma unroll
       for (int b = 0; b < 2; b++)
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-          const int row = 8 * (i >> 2) + 4 * h + (i & 3);
-          cW1[(32 * b + row) * HID + hid0 + c] = W1s.b[b][0][i];
-          cW2[(hid0 + row) * FD + 32 * b + c] = W2s.b[0][b][i];
+          const int row = 8 * (i >> 2) + (i & 3);   // + 4h in the lane offset
+          g_stf(gW1ck, (4 * h * HID + c) * 4, ck + ((32 * b + row) * HID + hid0) * 4, W1s.b[b][0][i]);
+          g_stf(gW2ck, (4 * h * FD + c) * 4, ck + ((hid0 + row) * FD + 32 * b) * 4, W2s.b[0][b][i]);
         }
       if (h == 0) p.b1_ck[slot * HID + hid0 + c] = b1L;
       if (tid < FD) p.b2_ck[slot * FD + tid] = s_b2[tid];
@@ -257,7 +262,7 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
       *reinterpret_cast<bf16x8*>(s_g2 + tok * LDB + f0) = o;
     }
     // the next mini-batch's inputs leave HBM now and are written to LDS at the end of this one
-    if (mb + 1 < p.NC) stage_load(st, p, x_base + (size_t)(mb + 1) * (CS * FD), eta_base + (size_t)(mb + 1) * CS, tid);
+    if (mb + 1 < p.NC) stage_load(st, gXQ, gXK, gXV, gEta, mb + 1, tid);
     __syncthreads();
 
     // ---- G1 = (G2 W2^T) * gelu'(Z1);  state += X^T G
@@ -365,7 +370,7 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
       bf16x8 o;
 #pragma unroll
       for (int e = 0; e < 8; e++) o[e] = (bf16)(bf2f(qv[e]) + __builtin_fmaf(gam[e], z[e] * rstd, bet[e]));
-      *reinterpret_cast<bf16x8*>(p.Out + x_base + (size_t)mb * (CS * FD) + tok * FD + f0) = o;
+      g_st8h(gOut, (tok * FD + f0) * 2, mb * TILE_BYTES, o);
     }
     // XK / XV were last read before the pair sum above; the XQ buffer written here is the other one.
     if (mb + 1 < p.NC) stage_store(st, smem, (mb + 1) & 1, tid);
