@@ -468,6 +468,19 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
 #define bDXV gbuf(ka->grad_L_XV + ox)
 #define bDETA gbuf(ka->grad_L_last_eta + oe)
   const unsigned t16 = 16 * tid, vln = (tok * FD + f0) * 2, vtok = 4 * tok;
+  // Everything derived from the lane index is cheap to recompute and expensive to keep: a value
+  // computed once before the loops is held in a register (or spilled and reloaded) for the whole
+  // kernel.  LANE_VARS re-derives the lot from a lane index the optimiser cannot see through, so
+  // each stage that opens with it gets fresh, short-lived copies.
+  int lane_v = lane;
+#define LANE_VARS                                                                                       \
+  asm volatile("" : "+v"(lane_v));                                                                      \
+  const int lane = lane_v, h = lane >> 5, c = lane & 31, tid = (v << 6) | lane;                         \
+  const int q8 = lane >> 3, tok = 8 * v + q8, f0 = 8 * (lane & 7);                                      \
+  const unsigned t16 = 16 * tid, vln = (tok * FD + f0) * 2, vtok = 4 * tok;                             \
+  const float* s_lnrow = s_P + (1 - r) * (32 * LDR) + (tok & 31) * LDR + f0;                            \
+  float* s_gy = reinterpret_cast<float*>(smem + SB_XQ) + tok * FD + f0;                                 \
+  (void)h; (void)c; (void)tid; (void)q8; (void)t16; (void)vln; (void)vtok; (void)s_lnrow; (void)s_gy
 
   // running gradients wrt the state after the last mini-batch
   AccT<2, 1> gW1s;
@@ -499,6 +512,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
       for (int j = 0; j < n_mb; j++) {
         const int mb = k * cgs + j;
         REFRESH_OFFSETS();
+        LANE_VARS;
         __syncthreads();
         stage3_store(st, s_xq, s_xk, s_e2, s_eta, tid);
         __syncthreads();
@@ -506,6 +520,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
         // Z1^T = W1s^T XK^T + b1  (rows hid, lane = tok); X2 rows [tok][hid] -> T0, gelu'(Z1) packed
         bf16x8 d1p[2][2];
         {
+          LANE_VARS;
           AccT<1, 2> x2;
           acc_init_rows_lds(x2, s_b1w, h);
           mma_jit<4>(x2, [&](int, int s) { return piece_state(W1s, 0, s); },
@@ -528,6 +543,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
         }
         WAVE_SYNC();
         {
+          LANE_VARS;
           AccT<2, 2> z2;
           acc_zero(z2);
           mma_jit<2>(z2, [&](int rb, int s) { return piece_state(W2s, rb, s); },                 // lane = F, contraction = hid
@@ -536,6 +552,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
         }
         // fused LayerNorm + reconstruction-loss gradient; saves for the reverse walk
         {
+          LANE_VARS;
           float z[8], gam[8];
           {
             float b2v[8];
@@ -574,6 +591,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
         __syncthreads();
         // G1 = (W2 G2^T) * gelu'(Z1)  (rows hid, lane = tok) -> T1 rows [tok][hid]; weight step
         {
+          LANE_VARS;
           AccT<1, 2> g1;
           acc_zero(g1);
           mma_jit<4>(g1, [&](int, int s) { return piece_state(W2t, 0, s); },                     // lane = hid, contraction = F
@@ -589,6 +607,8 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
             }
         }
         WAVE_SYNC();
+        {   // weight step
+          LANE_VARS;
         mma_jit<4>(W2s, [&](int, int s) { return piece_tr<LDH>(T0, 0, s, lane); },               // X2^T: lane = hid
                    [&](int fb, int s) { return piece_tr<LDX>(s_gz2, fb, s, lane); });            // G2: lane = F
         mma_jit<4>(W2t, [&](int fb, int s) { return piece_tr<LDX>(s_gz2, fb, s, lane); },
@@ -597,8 +617,10 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
         mma_jit<4>(W1s, [&](int fb, int s) { return piece_tr<LDX>(s_xk, fb, s, lane); },         // XK^T: lane = F
                    [&](int, int s) { return piece_tr<LDH>(T1, 0, s, lane); });                   // G1: lane = hid
         lds_rowsum_add_jit(s_b1w, [&](int s) { return piece_tr<LDH>(T1, 0, s, lane); }, ones, c, h);
+        }
         // operand images of the state after this step, for the reverse walk
         {
+          LANE_VARS;
           // bIMG2: W2, lane = hid, contraction = F;  bIMG1: W1^T, lane = F, contraction = hid
           store_state_rows<LDF>(T2, W1s, c, h);                                 // rows [hid][F]
 #pragma unroll
@@ -611,6 +633,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
         }
         // post-update forward on XQ
         {
+          LANE_VARS;
           AccT<1, 2> z1b;
           acc_init_rows_lds(z1b, s_b1w, h);
           mma_jit<4>(z1b, [&](int, int s) { return piece_state(W1s, 0, s); },
@@ -634,6 +657,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
           pair_sum(s_own, s_partner, z2, c, h);
         }
         {
+          LANE_VARS;
           float z[8], b2v[8];
           ln_gather(z, s_lnrow);
           ln_load_f32(b2v, s_b2 + f0);
@@ -657,6 +681,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
     for (int j = n_mb - 1; j >= 0; j--) {
       const int mb = k * cgs + j;
       REFRESH_OFFSETS();
+      LANE_VARS;
       const unsigned xo = mb * TILE_BYTES;       // this mini-batch in the input / output tensors
       const unsigned so = j * TILE_BYTES;        // its slot in the [cgs][64][64] scratch tensors
       const unsigned ho = j * IMG_BYTES;         // its slot in the [cgs][64][256] scratch tensors
@@ -664,24 +689,26 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
       const float eta_i[2] = {bf2f(g_ldh(bETA, 2 * c, mb * (CS * 2) + 64 * tb[0])), bf2f(g_ldh(bETA, 2 * c, mb * (CS * 2) + 64 * tb[1]))};
       __syncthreads();
       {
+        LANE_VARS;
         const u32x4 xq = g_ld16(bXQ, t16, xo), xk = g_ld16(bXK, t16, xo), gz = g_ld16(bGZ2, t16, so);
         const float eta = bf2f(g_ldh(bETA, 2 * (tid & (CS - 1)), mb * (CS * 2)));
         lds_put16(s_xq, tid, xq);
         lds_put16(s_xk, tid, xk);
         lds_put16(s_gz2, tid, gz);
         if (tid < CS) s_eta[tid] = eta;
+        // operand tiles of the state after this step: T1 = W2 rows [hid][F], T2 = W1^T rows [F][hid]
+#pragma unroll
+        for (int s = 0; s < 4; s++) store_piece_rows<LDF>(T1, 0, s, c, h, chunk_load(bIMG2, ho, s, t16));
+#pragma unroll
+        for (int fb = 0; fb < 2; fb++)
+#pragma unroll
+          for (int s = 0; s < 2; s++) store_piece_rows<LDH>(T2, fb, s, c, h, chunk_load(bIMG1, ho, 2 * fb + s, t16));
       }
-      // operand tiles of the state after this step: T1 = W2 rows [hid][F], T2 = W1^T rows [F][hid]
-#pragma unroll
-      for (int s = 0; s < 4; s++) store_piece_rows<LDF>(T1, 0, s, c, h, chunk_load(bIMG2, ho, s, t16));
-#pragma unroll
-      for (int fb = 0; fb < 2; fb++)
-#pragma unroll
-        for (int s = 0; s < 2; s++) store_piece_rows<LDH>(T2, fb, s, c, h, chunk_load(bIMG1, ho, 2 * fb + s, t16));
 
       // ---- output LayerNorm backward (LayerNorm lanes)
       float gO[8];
       {
+        LANE_VARS;
         float xh[8], gx[8], gam[8];
         ln_cvt8(gO, g_ld8h(bGO, vln, xo));
         ln_cvt8(xh, g_ld8h(bXHL, vln, so));
@@ -704,8 +731,10 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
       // ---- post-update forward, backwards (uses the state AFTER this mini-batch)
       bf16x8 dxq_old;            // the output rows this lane accumulates into
       {
+        LANE_VARS;
         AccT<2, 2> dq;
         {
+          LANE_VARS;
           AccT<1, 2> gz1b;   // (gZ2_bar W2^T) * gelu'(Z1_bar): rows hid, lane = tok
           acc_zero(gz1b);
           mma_jit<4>(gz1b, [&](int, int s) { return piece_rows<LDF>(T1, 0, s, c, h); },
@@ -744,6 +773,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
       }
       // pair sums of dXQ complete; gb2 holds its value after the first update
       {
+        LANE_VARS;
         float z[8];
         ln_gather(z, s_lnrow);
         dxq_old = g_ld8h(bDXQ, vln, xo);
@@ -759,6 +789,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
       bf16x8 dxv_old;            // LayerNorm lanes: the two outputs the stage accumulates into
       bf16 deta_old;
       {
+        LANE_VARS;
         // T1 = W2 before the step, rows [hid][F]; T2 = gW1, rows [hid][F]
 #pragma unroll
         for (int s = 0; s < 4; s++)
@@ -830,6 +861,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
 
       // ---- second-order pass through the fused LayerNorm loss (LayerNorm lanes)
       {
+        LANE_VARS;
         float gy[8];
         float gg[8], xh[8], go[8], gz[8], gam[8], gb[8];
         dxv_old = g_ld8h(bDXV, vln, xo);
@@ -848,6 +880,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
         const float rsd = 1.f / sdf;
         // dEta: -(sum_F gZ2*(X2 gW2 + gb2) + sum_H gZ1*(XK gW1 + gb1))
         {
+          LANE_VARS;
           float tot = oct_sum(dot8(gz, gb));
 #pragma unroll
           for (int u = 0; u < BW_NWAVE; u++) tot += s_deta[u * CS + tok];
@@ -881,6 +914,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
         }
         // g_y is needed again for dXK: park it (the XQ / E2 tiles are dead by now)
         {
+          LANE_VARS;
           f32x4 lo = {gy[0], gy[1], gy[2], gy[3]}, hi = {gy[4], gy[5], gy[6], gy[7]};
           *reinterpret_cast<f32x4*>(s_gy) = lo;
           *reinterpret_cast<f32x4*>(s_gy + 4) = hi;
@@ -893,6 +927,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
       // ---- inner MLP, backwards (uses the state BEFORE this mini-batch)
       bf16x8 dxk_old;
       {
+        LANE_VARS;
         bf16x8 w2b[4];   // W2 before the step: lane = hid, contraction = F
 #pragma unroll
         for (int s = 0; s < 4; s++) w2b[s] = w2_before(bIMG2, bCW2, ckW, j, s, hid0, c, h, t16);
@@ -960,6 +995,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
       }
       // pair sums of dXK complete
       {
+        LANE_VARS;
         float z[8], gyv[8];
         ln_gather(z, s_lnrow);
         ln_load_f32(gyv, s_gy);
@@ -987,6 +1023,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
   }
 }
 #undef REFRESH_OFFSETS
+#undef LANE_VARS
 #undef bXQ
 #undef bXK
 #undef bXV
