@@ -119,6 +119,15 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
   const int hid0 = FW_NS * v;
   float* s_Pp = s_P + (v & 3) * 64 * LDP;
   bf16* s_x2t = reinterpret_cast<bf16*>(smem + SM_X2T + v * SM_X2T_TILE);
+  // Everything derived from the lane index is cheap to recompute and expensive to keep in a register
+  // (or spilled) for the whole scan: LANE_VARS re-derives it from a lane index the optimiser cannot see
+  // through, so each stage that opens with it gets fresh, short-lived copies.
+  int lane_v = lane;
+#define LANE_VARS                                                               \
+  asm volatile("" : "+v"(lane_v));                                              \
+  const int lane = lane_v, h = lane >> 5, c = lane & 31, tid = (v << 6) | lane; \
+  const int tok = 8 * v + (lane >> 3), f0 = 8 * (lane & 7);                     \
+  (void)h; (void)c; (void)tid; (void)tok; (void)f0
 
   // ---- state -> registers
   AccT<2, 1> W1s, W2t;
@@ -158,10 +167,12 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
   __syncthreads();
 
   for (int mb = 0; mb < p.NC; mb++) {
+    LANE_VARS;
     const bf16* s_xq = reinterpret_cast<const bf16*>(smem + SM_XQ + (mb & 1) * SM_TILE);
 
     // ---- checkpoint: the state before this mini-batch
     if (mb % p.cgs == 0) {
+      LANE_VARS;
       const size_t slot = (size_t)bh * p.K + mb / p.cgs;
       const unsigned ck = (mb / p.cgs) * (FD * HID * 4);   // byte offset of the slot in gW1ck / gW2ck
 #pragma unroll
@@ -179,6 +190,7 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
     // ---- Z1 = XK W1 + b1 (rows tok, lane = hid);  X2 = gelu(Z1), D1 = gelu'(Z1)
     AccT<2, 1> x2, d1;
     {
+      LANE_VARS;
       const OpdT<1, 4> w1op = cvt_chain(W1s);
       const OpdT<2, 4> xkA = lds_rows_kappa<2, 4>(s_xk, LDB, c, h);
 #pragma unroll
@@ -197,11 +209,15 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
         }
     }
     const OpdT<1, 4> x2op = cvt_chain(x2);                  // lane = hid, contraction = tok
-    lds_store_rows_kappa<1, 4>(s_x2t, LDB, x2op, c, h);     // stored [hid][tok], private to the wave
+    {
+      LANE_VARS;
+      lds_store_rows_kappa<1, 4>(s_x2t, LDB, x2op, c, h);   // stored [hid][tok], private to the wave
+    }
     TTT_WAVE_SYNC();
 
     // ---- Z2^T partial = W2s^T X2^T (rows F, lane = tok), summed over the pair into [tok][F]
     {
+      LANE_VARS;
       const OpdT<2, 2> w2A = cvt_chain(W2s);
       const OpdT<2, 2> x2B = lds_tr_kappa<2, 2>(s_x2t, LDB, lane);
       AccT<2, 2> z2;
@@ -212,6 +228,7 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
 
     // ---- LayerNorm-fused reconstruction-loss gradient: 8 tokens per wave, 8 lanes per token
     {
+      LANE_VARS;
       float z[8];
       {
         f32x4 a0 = *reinterpret_cast<const f32x4*>(s_b2 + f0);
@@ -262,11 +279,15 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
       *reinterpret_cast<bf16x8*>(s_g2 + tok * LDB + f0) = o;
     }
     // the next mini-batch's inputs leave HBM now and are written to LDS at the end of this one
-    if (mb + 1 < p.NC) stage_load(st, gXQ, gXK, gXV, gEta, mb + 1, tid);
+    {
+      LANE_VARS;
+      if (mb + 1 < p.NC) stage_load(st, gXQ, gXK, gXV, gEta, mb + 1, tid);
+    }
     __syncthreads();
 
     // ---- G1 = (G2 W2^T) * gelu'(Z1);  state += X^T G
     {
+      LANE_VARS;
       const OpdT<2, 4> g2A = lds_rows_kappa<2, 4>(s_g2, LDB, c, h);   // lane = tok, contraction = F
       const OpdT<1, 4> w2tB = cvt_chain(W2t);                          // lane = hid, contraction = F
       AccT<2, 1> g1;
@@ -307,11 +328,15 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
       const OpdT<2, 4> xkT = lds_tr_kappa<2, 4>(s_xk, LDB, lane);      // lane = F, contraction = tok
       mma(W1s, xkT, g1op);                                             // W1[:,shard]   += XK^T G1
     }
-    if (h == 0) s_b1[hid0 + c] = b1L;        // read back below by this wave only
+    {
+      LANE_VARS;
+      if (h == 0) s_b1[hid0 + c] = b1L;      // read back below by this wave only
+    }
     TTT_WAVE_SYNC();
 
     // ---- post-update forward on XQ, transposed: Z1b^T = W1s^T XQ^T (rows hid, lane = tok)
     {
+      LANE_VARS;
       const OpdT<1, 4> w1A = cvt_chain(W1s);
       const OpdT<2, 4> xqB = lds_rows_kappa<2, 4>(s_xq, LDB, c, h);
       AccT<1, 2> z1b;
@@ -338,6 +363,7 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
 
     // ---- output LayerNorm + residual, 8 tokens per wave; next mini-batch's inputs into LDS
     {
+      LANE_VARS;
       float z[8];
       {
         f32x4 a0 = *reinterpret_cast<const f32x4*>(s_b2 + f0);
@@ -373,9 +399,13 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
       g_st8h(gOut, (tok * FD + f0) * 2, mb * TILE_BYTES, o);
     }
     // XK / XV were last read before the pair sum above; the XQ buffer written here is the other one.
-    if (mb + 1 < p.NC) stage_store(st, smem, (mb + 1) & 1, tid);
+    {
+      LANE_VARS;
+      if (mb + 1 < p.NC) stage_store(st, smem, (mb + 1) & 1, tid);
+    }
     __syncthreads();
   }
+#undef LANE_VARS
 }
 
 }  // namespace ttt
