@@ -73,6 +73,10 @@ def test_forward_launch_rejects_bad_arguments_before_touching_the_gpu(lib):
     a.XK = 0x1000
     a.NC = 0
     assert lib.ttt_mlp_fwd_launch(ctypes.byref(a), None) == 1001
+    a.NC, a.checkpoint_group_size, a.K = (1 << 18) + 1, 1, (1 << 18) + 1   # beyond the 32-bit offsets of one (batch, head)
+    assert lib.ttt_mlp_fwd_launch(ctypes.byref(a), None) == 1004
+    a.NC, a.checkpoint_group_size, a.K = 1 << 17, (1 << 16) + 1, 2
+    assert lib.ttt_mlp_fwd_launch(ctypes.byref(a), None) == 1004
     assert lib.ttt_mlp_bwd_launch(None, None) == 1001
 
 

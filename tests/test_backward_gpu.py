@@ -14,8 +14,9 @@ FWD_KEYS = ("XQ", "XK", "XV", "last_eta", "ttt_norm_weight", "ttt_norm_bias", "W
 UP_KEYS = ("grad_L_W1_last", "grad_L_b1_last", "grad_L_W2_last", "grad_L_b2_last", "grad_L_XQW_mini_batch")
 
 
-def run_fwd_bwd(d, cgs, hw_forward=True):
-    """Forward on the GPU (or oracle checkpoints when hw_forward is False), then backward on the GPU."""
+def run_fwd_bwd(d, cgs, hw_forward=True, scratch_fill=None):
+    """Forward on the GPU (or oracle checkpoints when hw_forward is False), then backward on the GPU.
+    scratch_fill: value written into the sixteen *_group workspace tensors before the backward."""
     import ttt_mlp_host as host
     dev = torch.device("cuda:0")
     B, NH, NC = d["XQ"].shape[:3]
@@ -30,6 +31,10 @@ def run_fwd_bwd(d, cgs, hw_forward=True):
         t["Out"].zero_()
     out_before = t["Out"].clone()
     t.update(host.alloc_backward_buffers(B, NH, NC, cgs, dev))
+    if scratch_fill is not None:
+        for name, v in t.items():
+            if name.endswith("_group"):
+                v.fill_(scratch_fill)
     ret = host.backward(t, cgs)
     assert ret.data_ptr() == t["Out"].data_ptr()
     assert torch.equal(t["Out"], out_before), "backward must leave Out untouched"
@@ -109,3 +114,23 @@ def test_matches_committed_golden_samples():
         if not err <= 6e-2:                            # 2e-2 of max|ref| is about 6e-2 of the rms here
             failures.append((name, err))
     assert not failures, failures
+
+
+GRADS = ("grad_L_ttt_norm_weight", "grad_L_ttt_norm_bias", "grad_L_W1_init", "grad_L_b1_init", "grad_L_W2_init",
+         "grad_L_b2_init", "grad_L_last_eta", "grad_L_XQ", "grad_L_XK", "grad_L_XV")
+
+
+@pytest.mark.parametrize("B,NH,NC,cgs", [(1, 1, 1, 1), (2, 3, 9, 4), (1, 4, 32, 8)])
+def test_bit_reproducible_and_independent_of_workspace_contents(B, NH, NC, cgs):
+    """Every sum in the kernels has a fixed order and the workspace is written before it is read: repeated runs,
+    and runs whose *_group workspace starts as NaN, zeros or 1e30, give bit-identical outputs (ragged group and
+    first-step-of-a-group paths included).  A read of unwritten workspace, a reordered sum or a missed wait shows
+    up here as a difference."""
+    d = orc.make_inputs(B, NH, NC, seed=11)
+    randomize_affine(d, 11)
+    base = run_fwd_bwd(d, cgs)
+    for fill in (None, float("nan"), 0.0, 1e30, None):
+        again = run_fwd_bwd(d, cgs, scratch_fill=fill)
+        for name in ("Out",) + GRADS:
+            assert torch.isfinite(again[name]).all(), (name, fill)
+            assert torch.equal(base[name], again[name]), (name, fill)
