@@ -509,13 +509,12 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
 
       Staged3 st;
       stage3_load(st, bXQ, bXK, bXV, bETA, k * cgs, tid, t16);
+      stage3_store(st, s_xq, s_xk, s_e2, s_eta, tid);
       for (int j = 0; j < n_mb; j++) {
         const int mb = k * cgs + j;
         REFRESH_OFFSETS();
         LANE_VARS;
-        __syncthreads();
-        stage3_store(st, s_xq, s_xk, s_e2, s_eta, tid);
-        __syncthreads();
+        __syncthreads();   // the staged inputs (and, for j = 0, the biases) are visible
 
         // Z1^T = W1s^T XK^T + b1  (rows hid, lane = tok); X2 rows [tok][hid] -> T0, gelu'(Z1) packed
         bf16x8 d1p[2][2];
@@ -655,6 +654,8 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
             stage3_load(st, bXQ, bXK, bXV, bETA, mb + 1, tid, t16);
           WAVE_SYNC();   // this wave's readers of T1 / T2 are done
           pair_sum(s_own, s_partner, z2, c, h);
+          // every reader of this mini-batch's XQ / XK / XV tiles is past the barriers above
+          if (j + 1 < n_mb) stage3_store(st, s_xq, s_xk, s_e2, s_eta, tid);
         }
         {
           LANE_VARS;
