@@ -139,3 +139,13 @@ def test_host_allocator_shapes():
     assert b["grad_L_ttt_norm_weight"].shape == (2, 3, 1, 64)      # per batch element
     for k in ("grad_L_last_eta", "grad_L_XQ", "grad_L_XK", "grad_L_XV"):
         assert b[k].abs().max() == 0
+
+
+def test_host_module_offers_the_autograd_wrapper(lib):
+    import inspect
+    import torch
+    import ttt_mlp_host as host
+    assert issubclass(host.TTTMLPFunction, torch.autograd.Function)
+    assert list(inspect.signature(host.ttt_mlp).parameters) == [
+        "XQ", "XK", "XV", "last_eta", "ttt_norm_weight", "ttt_norm_bias", "W1", "b1", "W2", "b2", "checkpoint_group_size"]
+    assert "grad_last" in inspect.signature(host.ttt_mlp_backward).parameters

@@ -90,3 +90,67 @@ def backward(t: Dict[str, torch.Tensor], cgs: int) -> torch.Tensor:
 
 def set_synchronize(on: bool) -> None:
     _ext.set_synchronize(bool(on))
+
+
+class TTTMLPFunction(torch.autograd.Function):
+    """`Out = ttt_mlp(XQ, XK, XV, last_eta, ttt_norm_weight, ttt_norm_bias, W1, b1, W2, b2)` with the
+    remat backward, as the usage block of the upstream README (README.md:22-96) and its test harness
+    (kernels/ttt_backward/matching.py:393-436, 522-523) call the two operators:
+      forward  allocates the checkpoints and Out and calls `ttt_forward`; only the inputs and the
+               checkpoints are kept for the backward (that is the point of the remat scheme);
+      backward allocates the sixteen scratch tensors and the zero-filled accumulating outputs, calls
+               `ttt_backward`, and sums the per-batch-element norm gradients over B.
+    The state after the last mini-batch is not an output of `ttt_forward`, so its upstream gradient is
+    zero here; `ttt_mlp_backward` below takes it explicitly.
+    Shapes / dtypes are the operator's: XQ, XK, XV [B,NH,NC,64,64] bf16, last_eta [B,NH,NC,64,1] bf16,
+    norm weight / bias [1,NH,1,64] fp32, W1 [B,NH,64,256], b1 [B,NH,1,256], W2 [B,NH,256,64],
+    b2 [B,NH,1,64] fp32; everything contiguous and on the GPU."""
+
+    @staticmethod
+    def forward(ctx, XQ, XK, XV, last_eta, ttt_norm_weight, ttt_norm_bias, W1, b1, W2, b2, checkpoint_group_size):
+        cgs = int(checkpoint_group_size)
+        B, NH, NC = XQ.shape[:3]
+        t = dict(XQ=XQ, XK=XK, XV=XV, last_eta=last_eta, ttt_norm_weight=ttt_norm_weight, ttt_norm_bias=ttt_norm_bias,
+                 W1=W1, b1=b1, W2=W2, b2=b2)
+        t = {k: v.detach().contiguous() for k, v in t.items()}
+        t.update(alloc_forward_buffers(B, NH, NC, cgs, XQ.device))
+        forward(t, cgs)
+        ctx.cgs = cgs
+        ctx.save_for_backward(t["XQ"], t["XK"], t["XV"], t["last_eta"], t["ttt_norm_weight"], t["ttt_norm_bias"],
+                              t["W1_checkpoints"], t["b1_checkpoints"], t["W2_checkpoints"], t["b2_checkpoints"])
+        return t["Out"]
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        XQ, XK, XV, last_eta, nw, nb, W1c, b1c, W2c, b2c = ctx.saved_tensors
+        g = ttt_mlp_backward(XQ, XK, XV, last_eta, nw, nb, (W1c, b1c, W2c, b2c), grad_out, ctx.cgs)
+        return (g["grad_L_XQ"], g["grad_L_XK"], g["grad_L_XV"], g["grad_L_last_eta"],
+                g["grad_L_ttt_norm_weight"].sum(dim=0, keepdim=True), g["grad_L_ttt_norm_bias"].sum(dim=0, keepdim=True),
+                g["grad_L_W1_init"], g["grad_L_b1_init"], g["grad_L_W2_init"], g["grad_L_b2_init"], None)
+
+
+def ttt_mlp_backward(XQ, XK, XV, last_eta, ttt_norm_weight, ttt_norm_bias, checkpoints, grad_out, cgs, grad_last=None):
+    """One `ttt_backward` call with freshly allocated workspace.  `checkpoints` = (W1, b1, W2, b2) checkpoints of the
+    forward; `grad_last` = upstream gradients wrt the state after the last mini-batch (W1, b1, W2, b2 shapes), zeros
+    when omitted.  Returns the ten gradients by the operator's names; the norm gradients are per batch element."""
+    B, NH, NC = XQ.shape[:3]
+    dev = XQ.device
+    f32 = dict(dtype=torch.float32, device=dev)
+    t = dict(XQ=XQ, XK=XK, XV=XV, last_eta=last_eta, ttt_norm_weight=ttt_norm_weight, ttt_norm_bias=ttt_norm_bias,
+             grad_L_XQW_mini_batch=grad_out.to(torch.bfloat16).contiguous())
+    for name, c in zip(("W1_checkpoints", "b1_checkpoints", "W2_checkpoints", "b2_checkpoints"), checkpoints):
+        t[name] = c
+    if grad_last is None:
+        grad_last = (torch.zeros(B, NH, F, HID, **f32), torch.zeros(B, NH, 1, HID, **f32),
+                     torch.zeros(B, NH, HID, F, **f32), torch.zeros(B, NH, 1, F, **f32))
+    for name, gl in zip(("grad_L_W1_last", "grad_L_b1_last", "grad_L_W2_last", "grad_L_b2_last"), grad_last):
+        t[name] = gl.to(torch.float32).contiguous()
+    t["Out"] = torch.empty(B, NH, NC, CS, F, dtype=torch.bfloat16, device=dev)   # unused by the operator, must exist
+    t.update(alloc_backward_buffers(B, NH, NC, cgs, dev))
+    backward(t, cgs)
+    return {k: t[k] for k in GRAD_NAMES}
+
+
+def ttt_mlp(XQ, XK, XV, last_eta, ttt_norm_weight, ttt_norm_bias, W1, b1, W2, b2, checkpoint_group_size):
+    """Differentiable call: see TTTMLPFunction."""
+    return TTTMLPFunction.apply(XQ, XK, XV, last_eta, ttt_norm_weight, ttt_norm_bias, W1, b1, W2, b2, checkpoint_group_size)
