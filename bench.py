@@ -90,6 +90,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c4")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-overlap", action="store_true",
+                    help="backward with one workgroup per (batch, head) even where two fit the device")
     ap.add_argument("--cpu-sample-mb", type=int, default=1536, help="mini-batches in the CPU baseline sample")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy, so that a counter run has a kernel of known traffic")
@@ -109,6 +111,8 @@ def main():
     t.update(host.alloc_forward_buffers(B, NH, NC, cgs, dev))
     t.update(host.alloc_backward_buffers(B, NH, NC, cgs, dev))
     host.set_synchronize(False)           # time with events; the operator's default host sync is not part of the kernel
+    import test_time_training as ext
+    ext.set_overlap(not a.no_overlap)
 
     def step(ev=None):
         host.zero_accumulating_grads(t)
@@ -148,6 +152,7 @@ def main():
     bwd_tflops = BWD_G * G_FLOP * mb_steps / (bwd_ms * 1e-3) / 1e12
     fwd_tflops = FWD_G * G_FLOP * mb_steps / (fwd_ms * 1e-3) / 1e12
     all_tflops = (FWD_G + BWD_G) * G_FLOP * mb_steps / (ms_per_step * 1e-3) / 1e12
+    bwd_kernel = "ttt_mlp_bwd_split_kernel" if ext.last_backward_mode() == 1 else "ttt_mlp_bwd_kernel"
     out = {
         "metric": "TTT-MLP fwd+bwd tokens/sec on 1 MI355X (B=1,NH=48,256K tok); % bf16 MFMA peak",
         "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -157,7 +162,7 @@ def main():
                    "checkpoint_group_size": cgs},
         "fwd_ms": fwd_ms, "bwd_ms": bwd_ms, "fwd_tflops": fwd_tflops, "fwd_bwd_tflops": all_tflops,
         "pct_of_bf16_mfma_peak": 100.0 * all_tflops / PEAK_BF16_TFLOPS,
-        "roofline": {"bound": "mfma", "kernel": "ttt_mlp_bwd_kernel", "achieved": bwd_tflops, "peak": PEAK_BF16_TFLOPS,
+        "roofline": {"bound": "mfma", "kernel": bwd_kernel, "achieved": bwd_tflops, "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": bwd_tflops / PEAK_BF16_TFLOPS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload),
                      "flop_per_launch": BWD_G * G_FLOP * mb_steps, "avg_launch_ms": bwd_ms},

@@ -41,6 +41,8 @@ extern "C" {
 #define TTT_MLP_ERR_BAD_CKPT 1002  /* K != ceil(NC / checkpoint_group_size)       */
 #define TTT_MLP_ERR_ALIGN 1003     /* a pointer is not 16-byte aligned            */
 #define TTT_MLP_ERR_TOO_LARGE 1004 /* B*NH > 2^31-1, NC > 2^18 or cgs > 2^16         */
+#define TTT_MLP_ERR_NO_ROOM 1005   /* 2*B*NH workgroups exceed the CUs of the device */
+#define TTT_MLP_ERR_WORKSPACE 1006 /* workspace smaller than required              */
 
 /* Forward scan.  Replaces the 16 positional arguments of `ttt_forward`
  * (test_time_training.cpp:25-42).  bf16 tensors are passed as uint16_t bit patterns. */
@@ -127,6 +129,23 @@ int ttt_mlp_fwd_launch(const ttt_mlp_fwd_args* args, void* stream);
 
 /* Same for the remat backward. */
 int ttt_mlp_bwd_launch(const ttt_mlp_bwd_args* args, void* stream);
+
+/* The same backward (bit-identical results) with two workgroups per (batch, head):
+ * one recomputes checkpoint group after checkpoint group, the other walks each
+ * recomputed group backwards, so recomputation leaves the critical path.  The
+ * reference launcher (kernels/ttt_backward/ttt.cu:1451-1917) has no counterpart:
+ * it spreads one (batch, head) over a cluster of four thread blocks instead.
+ * The mode needs all 2*B*NH workgroups resident at once (one per CU) and a
+ * caller-owned device workspace of ttt_mlp_bwd_workspace_bytes() bytes, 256-byte
+ * aligned, contents unspecified before and after; calls that overlap in time
+ * need separate workspaces.  ttt_mlp_bwd_workspace_bytes() returns 0 when the
+ * mode does not fit the current device (then the launcher returns
+ * TTT_MLP_ERR_NO_ROOM and the caller uses ttt_mlp_bwd_launch).  The int at index
+ * B*NH*32 of the workspace is a status word: once the stream has drained it reads
+ * non-zero only if a workgroup waited 20 s for the other and gave up, in which
+ * case the outputs are invalid. */
+size_t ttt_mlp_bwd_workspace_bytes(int32_t B, int32_t NH, int32_t checkpoint_group_size);
+int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* args, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Human-readable text for a return code of the two launchers. */
 const char* ttt_mlp_error_string(int code);

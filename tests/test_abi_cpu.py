@@ -32,7 +32,8 @@ def declared_functions():
 
 
 def test_header_declares_the_expected_entry_points():
-    assert declared_functions() == ["ttt_mlp_abi_version", "ttt_mlp_bwd_launch", "ttt_mlp_error_string",
+    assert declared_functions() == ["ttt_mlp_abi_version", "ttt_mlp_bwd_launch", "ttt_mlp_bwd_launch_overlapped",
+                                    "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_error_string",
                                     "ttt_mlp_fwd_launch", "ttt_mlp_kernel_info"]
 
 
@@ -78,6 +79,20 @@ def test_forward_launch_rejects_bad_arguments_before_touching_the_gpu(lib):
     a.NC, a.checkpoint_group_size, a.K = 1 << 17, (1 << 16) + 1, 2
     assert lib.ttt_mlp_fwd_launch(ctypes.byref(a), None) == 1004
     assert lib.ttt_mlp_bwd_launch(None, None) == 1001
+
+
+def test_overlapped_backward_needs_a_device_with_room(lib):
+    """Without a GPU no device has room for two workgroups per (batch, head): the size query says 0 and
+    the launcher refuses before anything is enqueued."""
+    lib.ttt_mlp_bwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.ttt_mlp_error_string.restype = ctypes.c_char_p
+    assert lib.ttt_mlp_bwd_workspace_bytes(0, 2, 4) == 0
+    assert lib.ttt_mlp_bwd_workspace_bytes(1, 2, 0) == 0
+    assert lib.ttt_mlp_bwd_launch_overlapped(None, None, ctypes.c_size_t(0), None) == 1001
+    if not torch.cuda.is_available():
+        assert lib.ttt_mlp_bwd_workspace_bytes(1, 2, 4) == 0
+    assert b"ttt_mlp_bwd_launch" in lib.ttt_mlp_error_string(1005)
+    assert b"workspace" in lib.ttt_mlp_error_string(1006)
 
 
 def test_struct_layout_matches_header_field_order():

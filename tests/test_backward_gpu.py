@@ -14,10 +14,13 @@ FWD_KEYS = ("XQ", "XK", "XV", "last_eta", "ttt_norm_weight", "ttt_norm_bias", "W
 UP_KEYS = ("grad_L_W1_last", "grad_L_b1_last", "grad_L_W2_last", "grad_L_b2_last", "grad_L_XQW_mini_batch")
 
 
-def run_fwd_bwd(d, cgs, hw_forward=True, scratch_fill=None):
+def run_fwd_bwd(d, cgs, hw_forward=True, scratch_fill=None, overlap=None):
     """Forward on the GPU (or oracle checkpoints when hw_forward is False), then backward on the GPU.
-    scratch_fill: value written into the sixteen *_group workspace tensors before the backward."""
+    scratch_fill: value written into the sixteen *_group workspace tensors before the backward.
+    overlap: None = the operator's own choice; False / True = one / two workgroups per (batch, head),
+    and the mode that actually ran is asserted."""
     import ttt_mlp_host as host
+    import test_time_training as ext
     dev = torch.device("cuda:0")
     B, NH, NC = d["XQ"].shape[:3]
     t = {k: d[k].to(dev).contiguous() for k in FWD_KEYS + UP_KEYS}
@@ -35,7 +38,14 @@ def run_fwd_bwd(d, cgs, hw_forward=True, scratch_fill=None):
         for name, v in t.items():
             if name.endswith("_group"):
                 v.fill_(scratch_fill)
-    ret = host.backward(t, cgs)
+    if overlap is not None:
+        ext.set_overlap(bool(overlap))
+    try:
+        ret = host.backward(t, cgs)
+    finally:
+        ext.set_overlap(True)
+    if overlap is not None:
+        assert ext.last_backward_mode() == int(bool(overlap))
     assert ret.data_ptr() == t["Out"].data_ptr()
     assert torch.equal(t["Out"], out_before), "backward must leave Out untouched"
     return {k: v.float().cpu() for k, v in t.items()}
@@ -134,3 +144,23 @@ def test_bit_reproducible_and_independent_of_workspace_contents(B, NH, NC, cgs):
         for name in ("Out",) + GRADS:
             assert torch.isfinite(again[name]).all(), (name, fill)
             assert torch.equal(base[name], again[name]), (name, fill)
+
+
+@pytest.mark.parametrize("B,NH,NC,cgs", [
+    (1, 2, 4, 1),        # four groups of one mini-batch: the two sets alternate, the replay waits for the walk
+    (2, 3, 9, 4),        # ragged last group (walked first), (batch, head) count not a multiple of 8
+    (1, 8, 24, 8),       # multiple of 8: the two workgroups of a pair are placed on one XCD
+    (2, 8, 10, 5),       # two groups only
+    (1, 4, 33, 2),       # seventeen groups
+])
+def test_overlapped_backward_is_bit_identical(B, NH, NC, cgs):
+    """Recomputing the groups on a second workgroup changes the schedule, not one bit of the results."""
+    print(f"case B={B} NH={NH} NC={NC} cgs={cgs}", flush=True)
+    d = orc.make_inputs(B, NH, NC, seed=11)
+    randomize_affine(d, 11)
+    one = run_fwd_bwd(d, cgs, overlap=False)
+    two = run_fwd_bwd(d, cgs, overlap=True, scratch_fill=float("nan"))
+    import ttt_mlp_host as host
+    for k in host.GRAD_NAMES:
+        assert torch.isfinite(two[k]).all(), k
+        assert torch.equal(one[k], two[k]), k

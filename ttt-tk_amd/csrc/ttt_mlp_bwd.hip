@@ -62,7 +62,8 @@ constexpr int SB_BET = SB_GAM + FD * 4;       // ttt_norm_bias of this head
 constexpr int SB_ETA = SB_BET + FD * 4;
 constexpr int SB_DETA = SB_ETA + CS * 4;                  // [8 waves][64 tokens] partial dEta sums
 constexpr int SB_RED = SB_DETA + BW_NWAVE * CS * 4;       // [8 waves][2][64] norm-gradient accumulators
-constexpr int SM_BWD_BYTES = SB_RED + BW_NWAVE * 2 * FD * 4;
+constexpr int SB_FLAG = SB_RED + BW_NWAVE * 2 * FD * 4;   // outcome of a wait on the other workgroup
+constexpr int SM_BWD_BYTES = SB_FLAG + 16;
 static_assert(SM_BWD_BYTES <= 160 * 1024, "LDS budget of one gfx950 CU exceeded");
 
 #define WAVE_SYNC() TTT_WAVE_SYNC()
@@ -189,9 +190,7 @@ TTT_DEV float ln_normalize(float (&z)[8], float* std_out) {
 // all of them: a rotation by 8 inside each row of 16 lanes, then across the four rows.
 TTT_DEV float token_sum8(float x) {
   x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x128, 0xF, 0xF, false));  // row_ror:8
-  x += __shfl_xor(x, 16, 64);
-  x += __shfl_xor(x, 32, 64);
-  return x;
+  return half_sum_valu(row_pair_sum(x));
 }
 // acc[f0 + e] += sum over this wave's tokens of x[e]   (wave-private LDS vector)
 TTT_DEV void ln_token_sum_add(float* s_acc, const float (&x)[8], int q8, int f0) {
@@ -370,8 +369,43 @@ TTT_DEV bf16x8 w1_before(gptr_t img, gptr_t ck, unsigned ck_off, int j, int rb, 
   return r;
 }
 
-__global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams p) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+// ------------------------------------------------------------------ two workgroups per (batch, head)
+// The replay of a checkpoint group needs only the checkpoint, so it can run ahead of the reverse walk
+// on another CU: one workgroup replays group after group into two alternating sets of the per-group
+// tensors, the other walks each group backwards as soon as it is complete.  They signal through two
+// counters in HBM (agent scope); both are resident at once because the launcher uses this mode only
+// when the grid fits the CUs of the device.  A wait that sees no progress for SPIN_LIMIT ticks of the
+// 100 MHz clock raises the status word and both workgroups leave, so every wave always exits.
+constexpr uint64_t SPIN_LIMIT = 2000000000ull;   // 20 s
+TTT_DEV bool wait_at_least(int* word, int target, int* status, int* s_flag) {
+  if (threadIdx.x == 0) {
+    int ok = 1;
+    const uint64_t t0 = wall_clock64();
+    while (__hip_atomic_load(word, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < target) {
+      if (__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 || wall_clock64() - t0 > SPIN_LIMIT) {
+        __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ok = 0;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(32);
+    }
+    *s_flag = ok;
+  }
+  __syncthreads();
+  const int ok = *s_flag;
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  return ok != 0;
+}
+// Everything this workgroup has written (or read) so far is ordered before the new value of `word`.
+TTT_DEV void publish(int* word, int value) {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+  __syncthreads();
+  if (threadIdx.x == 0) __hip_atomic_store(word, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ROLE 0: replay and reverse walk of every group in one workgroup; 1: the replays only; 2: the reverse walks only.
+template <int ROLE>
+TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
   bf16* s_xq = reinterpret_cast<bf16*>(smem + SB_XQ);
   bf16* s_xk = reinterpret_cast<bf16*>(smem + SB_XK);
   bf16* s_gz2 = reinterpret_cast<bf16*>(smem + SB_GZ2);
@@ -393,7 +427,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
   const int pp = v & 3, r = v >> 2;                              // pair, index inside the pair
   const int tb[2] = {r, 1 - r};                                  // token block held in column block 0 / 1 of a Q tile
   const int q8 = lane >> 3, tok = 8 * v + q8, f0 = 8 * (lane & 7);   // LayerNorm ownership (token block r)
-  const int bh = blockIdx.x, head = bh % p.NH;
+  const int head = bh % p.NH;
   const int hid0 = BW_NS * v;
   float* s_own = s_P + (pp * 2 + r) * (32 * LDR);
   float* s_partner = s_P + (pp * 2 + (1 - r)) * (32 * LDR);
@@ -441,21 +475,23 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
   typedef const __attribute__((address_space(4))) BwdParams* KernArgs;
   KernArgs ka = (KernArgs)__builtin_amdgcn_kernarg_segment_ptr();
 #define REFRESH_OFFSETS() asm volatile("" : "+s"(ka), "+s"(ox), "+s"(oe), "+s"(of), "+s"(oh), "+s"(ot), "+s"(opk), "+s"(ock))
+  // per-group tensors: the caller's (set 0) or, in two-workgroup mode, the alternate set
+#define GRP(name) (set ? ka->alt_##name : ka->name)
 #define bXQ gbuf(ka->XQ + ox)
 #define bXK gbuf(ka->XK + ox)
 #define bXV gbuf(ka->XV + ox)
 #define bGO gbuf(ka->grad_L_XQW + ox)
 #define bETA gbuf(ka->last_eta + oe)
-#define bZ1 gbuf(ka->Z1_group + oh)
-#define bZ1B gbuf(ka->Z1_bar_group + oh)
-#define bIMG1 gbuf(ka->X2_group + oh)
-#define bIMG2 gbuf(ka->grad_l_wrt_Z1_group + oh)
-#define bXHF gbuf(ka->x_hat_fused_group + of)
-#define bGOF gbuf(ka->grad_output_fused_group + of)
-#define bGZ2 gbuf(ka->grad_l_wrt_Z2_group + of)
-#define bXHL gbuf(ka->x_hat_ln_group + of)
-#define bSDF gbuf(ka->std_fused_group + ot)
-#define bSDL gbuf(ka->std_ln_group + ot)
+#define bZ1 gbuf(GRP(Z1_group) + oh)
+#define bZ1B gbuf(GRP(Z1_bar_group) + oh)
+#define bIMG1 gbuf(GRP(X2_group) + oh)
+#define bIMG2 gbuf(GRP(grad_l_wrt_Z1_group) + oh)
+#define bXHF gbuf(GRP(x_hat_fused_group) + of)
+#define bGOF gbuf(GRP(grad_output_fused_group) + of)
+#define bGZ2 gbuf(GRP(grad_l_wrt_Z2_group) + of)
+#define bXHL gbuf(GRP(x_hat_ln_group) + of)
+#define bSDF gbuf(GRP(std_fused_group) + ot)
+#define bSDL gbuf(GRP(std_ln_group) + ot)
   // While a group is replayed the running gradients are parked in W*_init_group; during the reverse
   // walk the same two 64 KiB slots park what must survive the LayerNorm stage (three 32 KiB images).
 #define bPW1 gbuf(ka->W1_init_group + opk)
@@ -485,19 +521,32 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
   // running gradients wrt the state after the last mini-batch
   AccT<2, 1> gW1s;
   AccT<1, 2> gW2s;
-  acc_load_rows(gW1s, gbuf(p.grad_L_W1_last + (size_t)bh * FD * HID), 0, HID, 0, hid0, c, h);
-  acc_load_rows(gW2s, gbuf(p.grad_L_W2_last + (size_t)bh * HID * FD), 0, FD, hid0, 0, c, h);
+  if constexpr (ROLE != 1) {
+    acc_load_rows(gW1s, gbuf(p.grad_L_W1_last + (size_t)bh * FD * HID), 0, HID, 0, hid0, c, h);
+    acc_load_rows(gW2s, gbuf(p.grad_L_W2_last + (size_t)bh * HID * FD), 0, FD, hid0, 0, c, h);
+  }
+  int* const w_replayed = p.sync + (size_t)bh * BWD_SYNC_STRIDE;
+  int* const w_walked = w_replayed + 16;
+  int* const w_status = p.sync + (size_t)p.B * p.NH * BWD_SYNC_STRIDE;
+  int* const s_flag = reinterpret_cast<int*>(smem + SB_FLAG);
 
   for (int k = p.K - 1; k >= 0; k--) {
     const int n_mb = min(cgs, p.NC - k * cgs);
+    const int done = p.K - 1 - k;                    // groups already handled by this workgroup
+    const int set = ROLE == 0 ? 0 : (done & 1);
     REFRESH_OFFSETS();
     const size_t slot = (size_t)bh * p.K + k;
     const unsigned ckW = k * (FD * HID * 4);   // byte offset of this group's checkpoint in bCW1 / bCW2
     // ================================================================= replay
-    {
+    if constexpr (ROLE != 2) {
+      if constexpr (ROLE == 1) {   // the set is free once the reverse walk is done with the group before last
+        if (done >= 2 && !wait_at_least(w_walked, done - 1, w_status, s_flag)) return;
+      }
       // park the running gradients while the forward state needs the registers
-      acc_store_rows(gW1s, bPW1, 0, HID, 0, hid0, c, h);
-      acc_store_rows(gW2s, bPW2, 0, FD, hid0, 0, c, h);
+      if constexpr (ROLE == 0) {
+        acc_store_rows(gW1s, bPW1, 0, HID, 0, hid0, c, h);
+        acc_store_rows(gW2s, bPW2, 0, FD, hid0, 0, c, h);
+      }
       AccT<2, 1> W1s, W2t;
       AccT<1, 2> W2s;
       acc_load_rows(W1s, bCW1, ckW, HID, 0, hid0, c, h);
@@ -671,14 +720,21 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
         }
       }
       // running gradients back into registers
-      acc_load_rows(gW1s, bPW1, 0, HID, 0, hid0, c, h);
-      acc_load_rows(gW2s, bPW2, 0, FD, hid0, 0, c, h);
+      if constexpr (ROLE == 0) {
+        acc_load_rows(gW1s, bPW1, 0, HID, 0, hid0, c, h);
+        acc_load_rows(gW2s, bPW2, 0, FD, hid0, 0, c, h);
+      }
+      if constexpr (ROLE == 1) publish(w_replayed, done + 1);
     }
 
     // ================================================================= reverse walk
     // Operands are fetched from HBM right where they are consumed: with two waves per SIMD the other
     // wave covers the latency, while holding requests in registers across stages costs more in spills
     // than it gains (measured).
+    if constexpr (ROLE == 2) {
+      if (!wait_at_least(w_replayed, done + 1, w_status, s_flag)) return;
+    }
+    if constexpr (ROLE != 1)
     for (int j = n_mb - 1; j >= 0; j--) {
       const int mb = k * cgs + j;
       REFRESH_OFFSETS();
@@ -697,13 +753,18 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
         lds_put16(s_xk, tid, xk);
         lds_put16(s_gz2, tid, gz);
         if (tid < CS) s_eta[tid] = eta;
-        // operand tiles of the state after this step: T1 = W2 rows [hid][F], T2 = W1^T rows [F][hid]
+      }
+      // The state after this step enters as ready-made operands: the images the replay stored are in MFMA
+      // operand layout already, so their chunks go from HBM straight into the products below.
+      bf16x8 w2a[4], w1a[2][2];   // W2: lane = hid, contraction = F;  W1^T: lane = F, contraction = hid
+      {
+        LANE_VARS;
 #pragma unroll
-        for (int s = 0; s < 4; s++) store_piece_rows<LDF>(T1, 0, s, c, h, chunk_load(bIMG2, ho, s, t16));
+        for (int s = 0; s < 4; s++) w2a[s] = chunk_load(bIMG2, ho, s, t16);
 #pragma unroll
         for (int fb = 0; fb < 2; fb++)
 #pragma unroll
-          for (int s = 0; s < 2; s++) store_piece_rows<LDH>(T2, fb, s, c, h, chunk_load(bIMG1, ho, 2 * fb + s, t16));
+          for (int s = 0; s < 2; s++) w1a[fb][s] = chunk_load(bIMG1, ho, 2 * fb + s, t16);
       }
 
       // ---- output LayerNorm backward (LayerNorm lanes)
@@ -738,9 +799,8 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
           LANE_VARS;
           AccT<1, 2> gz1b;   // (gZ2_bar W2^T) * gelu'(Z1_bar): rows hid, lane = tok
           acc_zero(gz1b);
-          mma_jit<4>(gz1b, [&](int, int s) { return piece_rows<LDF>(T1, 0, s, c, h); },
+          mma_jit<4>(gz1b, [&](int, int s) { return w2a[s]; },
                      [&](int i, int s) { return piece_rows<LDX>(s_a, tb[i], s, c, h); });
-          WAVE_SYNC();   // T1 is overwritten below
 #pragma unroll
           for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -761,7 +821,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
         }
         WAVE_SYNC();
         acc_zero(dq);
-        mma_jit<2>(dq, [&](int rb, int s) { return piece_rows<LDH>(T2, rb, s, c, h); },        // W1 after: lane = F
+        mma_jit<2>(dq, [&](int rb, int s) { return w1a[rb][s]; },                              // W1 after: lane = F
                    [&](int i, int s) { return piece_rows<LDH>(T1, tb[i], s, c, h); });         // gZ1_bar: lane = tok
         mma_jit<4>(gW2s, [&](int, int s) { return piece_tr<LDH>(T0, 0, s, lane); },            // X2_bar^T: lane = hid
                    [&](int fb, int s) { return piece_tr<LDX>(s_a, fb, s, lane); });            // gZ2_bar: lane = F
@@ -1006,7 +1066,9 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
         g_st8h(bDXK, vln, xo, dxk_old);
       }
     }
+    if constexpr (ROLE == 2) publish(w_walked, done + 1);
   }
+  if constexpr (ROLE == 1) return;
 
   // ---- outputs that are written once
   acc_store_rows(gW1s, gbuf(p.grad_L_W1_init + (size_t)bh * FD * HID), 0, HID, 0, hid0, c, h);
@@ -1025,6 +1087,7 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
 }
 #undef REFRESH_OFFSETS
 #undef LANE_VARS
+#undef GRP
 #undef bXQ
 #undef bXK
 #undef bXV
@@ -1049,6 +1112,33 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams
 #undef bDXV
 #undef bDETA
 
+__global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  bwd_body<0>(p, smem, blockIdx.x);
+}
+
+// Two workgroups per (batch, head).  Workgroups are dealt to the 8 XCDs in turn, so with a multiple
+// of 8 (batch, head) pairs the two workgroups of a pair are placed 8 apart: same XCD, same L2.
+__global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_split_kernel(const BwdParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int b = blockIdx.x;
+  int bh, role;
+  if ((p.B * p.NH) % 8 == 0) {
+    bh = (b >> 4) * 8 + (b & 7);
+    role = (b >> 3) & 1;
+  } else {
+    bh = b >> 1;
+    role = b & 1;
+  }
+  if (role == 0) bwd_body<1>(p, smem, bh);
+  else bwd_body<2>(p, smem, bh);
+}
+
+__global__ void ttt_mlp_zero_words(int* w, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) w[i] = 0;
+}
+
 }  // namespace ttt
 
 extern "C" int ttt_mlp_bwd_threads() { return ttt::BW_THREADS; }
@@ -1058,6 +1148,15 @@ hipError_t ttt_mlp_bwd_enqueue(const ttt::BwdParams& p, hipStream_t stream) {
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(ttt::ttt_mlp_bwd_kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, ttt::SM_BWD_BYTES);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(ttt::ttt_mlp_bwd_kernel, dim3(p.B * p.NH), dim3(ttt::BW_THREADS), ttt::SM_BWD_BYTES, stream, p);
+  if (p.sync == nullptr) {
+    hipLaunchKernelGGL(ttt::ttt_mlp_bwd_kernel, dim3(p.B * p.NH), dim3(ttt::BW_THREADS), ttt::SM_BWD_BYTES, stream, p);
+    return hipGetLastError();
+  }
+  e = hipFuncSetAttribute(reinterpret_cast<const void*>(ttt::ttt_mlp_bwd_split_kernel),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, ttt::SM_BWD_BYTES);
+  if (e != hipSuccess) return e;
+  const int n = static_cast<int>(ttt::bwd_sync_ints((long long)p.B * p.NH));
+  hipLaunchKernelGGL(ttt::ttt_mlp_zero_words, dim3((n + 255) / 256), dim3(256), 0, stream, p.sync, n);
+  hipLaunchKernelGGL(ttt::ttt_mlp_bwd_split_kernel, dim3(2 * p.B * p.NH), dim3(ttt::BW_THREADS), ttt::SM_BWD_BYTES, stream, p);
   return hipGetLastError();
 }

@@ -36,6 +36,8 @@ extern "C" const char* ttt_mlp_error_string(int code) {
     case TTT_MLP_ERR_BAD_CKPT: return "ttt_mlp: number of checkpoints K must equal ceil(NC / checkpoint_group_size)";
     case TTT_MLP_ERR_ALIGN: return "ttt_mlp: every tensor pointer must be 16-byte aligned";
     case TTT_MLP_ERR_TOO_LARGE: return "ttt_mlp: B*NH exceeds the launch grid limit, or NC > 262144, or checkpoint_group_size > 65536";
+    case TTT_MLP_ERR_NO_ROOM: return "ttt_mlp: two workgroups per (batch, head) do not fit the compute units of this device; use ttt_mlp_bwd_launch";
+    case TTT_MLP_ERR_WORKSPACE: return "ttt_mlp: workspace smaller than ttt_mlp_bwd_workspace_bytes()";
     default: return hipGetErrorString(static_cast<hipError_t>(code));
   }
 }
@@ -59,7 +61,10 @@ extern "C" int ttt_mlp_fwd_launch(const ttt_mlp_fwd_args* a, void* stream) {
   return static_cast<int>(ttt_mlp_fwd_enqueue(p, static_cast<hipStream_t>(stream)));
 }
 
-extern "C" int ttt_mlp_bwd_launch(const ttt_mlp_bwd_args* a, void* stream) {
+namespace {
+
+// Validates the backward arguments and translates them for the kernels.
+int make_bwd_params(const ttt_mlp_bwd_args* a, ttt::BwdParams& p) {
   if (a == nullptr) return TTT_MLP_ERR_BAD_ARG;
   if (any_null(a->XQ, a->XK, a->XV, a->last_eta, a->ttt_norm_weight, a->ttt_norm_bias, a->W1_checkpoints,
                a->b1_checkpoints, a->W2_checkpoints, a->b2_checkpoints, a->W1_init_group, a->b1_init_group,
@@ -80,7 +85,7 @@ extern "C" int ttt_mlp_bwd_launch(const ttt_mlp_bwd_args* a, void* stream) {
                    a->grad_L_b1_init, a->grad_L_W2_init, a->grad_L_b2_init, a->grad_L_last_eta, a->grad_L_XQ,
                    a->grad_L_XK, a->grad_L_XV))
     return TTT_MLP_ERR_ALIGN;
-  ttt::BwdParams p;
+  p = ttt::BwdParams{};
   p.XQ = bf(a->XQ); p.XK = bf(a->XK); p.XV = bf(a->XV); p.last_eta = bf(a->last_eta);
   p.ttt_norm_weight = a->ttt_norm_weight; p.ttt_norm_bias = a->ttt_norm_bias;
   p.W1_ck = a->W1_checkpoints; p.b1_ck = a->b1_checkpoints; p.W2_ck = a->W2_checkpoints; p.b2_ck = a->b2_checkpoints;
@@ -101,6 +106,68 @@ extern "C" int ttt_mlp_bwd_launch(const ttt_mlp_bwd_args* a, void* stream) {
   p.grad_L_last_eta = bf(a->grad_L_last_eta);
   p.grad_L_XQ = bf(a->grad_L_XQ); p.grad_L_XK = bf(a->grad_L_XK); p.grad_L_XV = bf(a->grad_L_XV);
   p.B = a->B; p.NH = a->NH; p.NC = a->NC; p.K = a->K; p.cgs = a->checkpoint_group_size;
+  return TTT_MLP_OK;
+}
+
+// Two workgroups per (batch, head) wait for each other, so all of them must be resident at once:
+// one workgroup fills a CU (LDS), hence the grid may not exceed the CUs of the current device.
+bool two_workgroup_mode_fits(long long BH) {
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return false;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return false;
+  return BH > 0 && 2 * BH <= cus;
+}
+
+// Workspace of the two-workgroup mode: the synchronisation words, then the alternate set of the ten
+// per-group tensors that carry a replayed group to the reverse walk, each part 256-byte aligned.
+struct BwdWorkspace {
+  size_t off[11];
+  size_t total;
+  BwdWorkspace(long long BH, long long cgs) {
+    const size_t slot = (size_t)BH * (size_t)cgs;
+    const size_t tile = TTT_MLP_CS * TTT_MLP_F * 2, img = TTT_MLP_CS * TTT_MLP_HID * 2, vec = TTT_MLP_CS * 4;
+    const size_t bytes[11] = {ttt::bwd_sync_ints(BH) * sizeof(int), slot * tile, slot * vec, slot * img, slot * img, slot * img,
+                              slot * tile, slot * img, slot * tile, slot * tile, slot * vec};
+    size_t o = 0;
+    for (int i = 0; i < 11; i++) { off[i] = o; o += (bytes[i] + 255) & ~(size_t)255; }
+    total = o;
+  }
+};
+
+}  // namespace
+
+extern "C" int ttt_mlp_bwd_launch(const ttt_mlp_bwd_args* a, void* stream) {
+  ttt::BwdParams p;
+  if (int rc = make_bwd_params(a, p)) return rc;
+  return static_cast<int>(ttt_mlp_bwd_enqueue(p, static_cast<hipStream_t>(stream)));
+}
+
+extern "C" size_t ttt_mlp_bwd_workspace_bytes(int B, int NH, int checkpoint_group_size) {
+  if (B <= 0 || NH <= 0 || checkpoint_group_size <= 0 || checkpoint_group_size > (1 << 16)) return 0;
+  if (!two_workgroup_mode_fits((long long)B * NH)) return 0;
+  return BwdWorkspace((long long)B * NH, checkpoint_group_size).total;
+}
+
+extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* workspace, size_t workspace_bytes, void* stream) {
+  ttt::BwdParams p;
+  if (int rc = make_bwd_params(a, p)) return rc;
+  if (workspace == nullptr) return TTT_MLP_ERR_BAD_ARG;
+  if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return TTT_MLP_ERR_ALIGN;
+  if (!two_workgroup_mode_fits((long long)p.B * p.NH)) return TTT_MLP_ERR_NO_ROOM;
+  const BwdWorkspace w((long long)p.B * p.NH, p.cgs);
+  if (workspace_bytes < w.total) return TTT_MLP_ERR_WORKSPACE;
+  char* base = static_cast<char*>(workspace);
+  p.sync = reinterpret_cast<int*>(base + w.off[0]);
+  p.alt_x_hat_ln_group = reinterpret_cast<__bf16*>(base + w.off[1]);
+  p.alt_std_ln_group = reinterpret_cast<float*>(base + w.off[2]);
+  p.alt_X2_group = reinterpret_cast<__bf16*>(base + w.off[3]);
+  p.alt_Z1_group = reinterpret_cast<__bf16*>(base + w.off[4]);
+  p.alt_Z1_bar_group = reinterpret_cast<__bf16*>(base + w.off[5]);
+  p.alt_grad_l_wrt_Z2_group = reinterpret_cast<__bf16*>(base + w.off[6]);
+  p.alt_grad_l_wrt_Z1_group = reinterpret_cast<__bf16*>(base + w.off[7]);
+  p.alt_x_hat_fused_group = reinterpret_cast<__bf16*>(base + w.off[8]);
+  p.alt_grad_output_fused_group = reinterpret_cast<__bf16*>(base + w.off[9]);
+  p.alt_std_fused_group = reinterpret_cast<float*>(base + w.off[10]);
   return static_cast<int>(ttt_mlp_bwd_enqueue(p, static_cast<hipStream_t>(stream)));
 }
 

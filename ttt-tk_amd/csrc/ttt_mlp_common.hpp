@@ -161,6 +161,22 @@ TTT_DEV float quad_sum(float x) {
 }
 // Sum of lane l and lane l^32, result in both.
 TTT_DEV float half_sum(float x) { return x + __shfl_xor(x, 32, 64); }
+// The same sum without the LDS pipe, for stages that form many of them.  v_permlane32_swap exchanges the upper half of its
+// first register with the lower half of its second: starting from two copies of x, one register then
+// holds x[l % 32] and the other x[l % 32 + 32] in every lane.  (Written as asm: the builtin of this compiler adds the
+// first result to itself.)
+TTT_DEV float half_sum_valu(float x) {
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return a + b;
+}
+// Sum of lane l and lane l^16, result in both: v_permlane16_swap exchanges the odd rows of 16 lanes of
+// its first register with the even rows of its second.
+TTT_DEV float row_pair_sum(float x) {
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return a + b;
+}
 
 // ---------------------------------------------------------------------------- shape-generic tiles
 // Tiles whose extent along the hidden dimension is one 32-wide block (a wave that owns 32 hidden

@@ -31,11 +31,26 @@ struct BwdParams {
   float *grad_L_W1_init, *grad_L_b1_init, *grad_L_W2_init, *grad_L_b2_init;
   __bf16 *grad_L_last_eta, *grad_L_XQ, *grad_L_XK, *grad_L_XV;
   int B, NH, NC, K, cgs;
+  // Two-workgroup mode only (sync != nullptr): a second set of the per-group tensors that carry a
+  // replayed group to the reverse walk, and the words the two workgroups of a (batch, head) signal with.
+  __bf16* alt_x_hat_ln_group;
+  float* alt_std_ln_group;
+  __bf16 *alt_X2_group, *alt_Z1_group, *alt_Z1_bar_group;
+  __bf16 *alt_grad_l_wrt_Z2_group, *alt_grad_l_wrt_Z1_group;
+  __bf16 *alt_x_hat_fused_group, *alt_grad_output_fused_group;
+  float* alt_std_fused_group;
+  int* sync;
 };
+
+// Layout of `sync` (ints): 32 per (batch, head) - word 0 counts the groups replayed, word 16 the groups
+// the reverse walk has finished - then one status word (non-zero: a wait gave up).
+constexpr int BWD_SYNC_STRIDE = 32;
+inline size_t bwd_sync_ints(long long BH) { return (size_t)BH * BWD_SYNC_STRIDE + 32; }
 
 }  // namespace ttt
 
 hipError_t ttt_mlp_fwd_enqueue(const ttt::FwdParams& p, hipStream_t stream);
+// p.sync == nullptr: one workgroup per (batch, head); otherwise two (replay / reverse walk).
 hipError_t ttt_mlp_bwd_enqueue(const ttt::BwdParams& p, hipStream_t stream);
 extern "C" int ttt_mlp_fwd_lds_bytes();
 extern "C" int ttt_mlp_bwd_lds_bytes();
