@@ -447,10 +447,13 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
   }
   if (tid < HID) s_gb1[tid] = p.grad_L_b1_last[(size_t)bh * HID + tid];
   // Norm-weight / norm-bias gradients accumulate per wave in LDS (summed over the wave's 8 tokens
-  // with cross-lane adds in a fixed order); summed over the waves at the end.
+  // with cross-lane adds in a fixed order); summed over the waves at the end.  The replay and the
+  // reverse walk each contribute, and their sums are kept apart (so that the result does not depend on
+  // whether one workgroup does both): with one workgroup the sum that is not being added to waits in HBM.
   float* s_dgw = s_red + (v * 2 + 0) * FD;
   float* s_dbw = s_red + (v * 2 + 1) * FD;
   if (lane < FD) { s_dgw[lane] = 0.f; s_dbw[lane] = 0.f; }
+  const unsigned np_off = (v * 2 * FD + lane) * 4;   // this lane's two words of the wave's accumulators: +0, +FD*4
   float* s_gy = reinterpret_cast<float*>(smem + SB_XQ) + tok * FD + f0;   // this lane's part of the g_y park
   bf16x8 ones;
 #pragma unroll
@@ -483,15 +486,16 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
 #define bGO gbuf(ka->grad_L_XQW + ox)
 #define bETA gbuf(ka->last_eta + oe)
 #define bZ1 gbuf(GRP(Z1_group) + oh)
-#define bZ1B gbuf(GRP(Z1_bar_group) + oh)
+#define bGZ1B gbuf(GRP(Z1_bar_group) + oh)              // operand image of gZ1_bar = dL/dZ1_bar
+#define bX2B gbuf(GRP(X2_bar_group) + oh)               // operand image of X2_bar
+#define bGZB gbuf(GRP(grad_x_hat_fused_group) + of)     // gZ2_bar = dL/dZ2_bar, [tok][F] tiles
 #define bIMG1 gbuf(GRP(X2_group) + oh)
 #define bIMG2 gbuf(GRP(grad_l_wrt_Z1_group) + oh)
 #define bXHF gbuf(GRP(x_hat_fused_group) + of)
 #define bGOF gbuf(GRP(grad_output_fused_group) + of)
 #define bGZ2 gbuf(GRP(grad_l_wrt_Z2_group) + of)
-#define bXHL gbuf(GRP(x_hat_ln_group) + of)
+#define bNP gbuf(ka->x_hat_ln_group + of)                // one workgroup per (batch, head): park of norm-gradient sums
 #define bSDF gbuf(GRP(std_fused_group) + ot)
-#define bSDL gbuf(GRP(std_ln_group) + ot)
   // While a group is replayed the running gradients are parked in W*_init_group; during the reverse
   // walk the same two 64 KiB slots park what must survive the LayerNorm stage (three 32 KiB images).
 #define bPW1 gbuf(ka->W1_init_group + opk)
@@ -530,6 +534,22 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
   int* const w_status = p.sync + (size_t)p.B * p.NH * BWD_SYNC_STRIDE;
   int* const s_flag = reinterpret_cast<int*>(smem + SB_FLAG);
 
+  if constexpr (ROLE == 0) {   // the replay's sum starts at zero
+    g_stf(bNP, np_off, 0, 0.f);
+    g_stf(bNP, np_off, FD * 4, 0.f);
+  }
+  // Exchanges the wave's LDS accumulators with the parked sum (every lane owns two words of both).
+  auto norm_swap = [&]() {
+    WAVE_SYNC();
+    const float a0 = s_dgw[lane], a1 = s_dbw[lane];
+    const float p0 = g_ldf(bNP, np_off, 0), p1 = g_ldf(bNP, np_off, FD * 4);
+    s_dgw[lane] = p0;
+    s_dbw[lane] = p1;
+    g_stf(bNP, np_off, 0, a0);
+    g_stf(bNP, np_off, FD * 4, a1);
+    WAVE_SYNC();
+  };
+
   for (int k = p.K - 1; k >= 0; k--) {
     const int n_mb = min(cgs, p.NC - k * cgs);
     const int done = p.K - 1 - k;                    // groups already handled by this workgroup
@@ -546,6 +566,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
       if constexpr (ROLE == 0) {
         acc_store_rows(gW1s, bPW1, 0, HID, 0, hid0, c, h);
         acc_store_rows(gW2s, bPW2, 0, FD, hid0, 0, c, h);
+        norm_swap();
       }
       AccT<2, 1> W1s, W2t;
       AccT<1, 2> W2s;
@@ -556,11 +577,14 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
       if (tid < HID) s_b1[tid] = p.b1_ck[slot * HID + tid];
       if (tid < FD) s_b2[tid] = p.b2_ck[slot * FD + tid];
 
-      Staged3 st;
-      stage3_load(st, bXQ, bXK, bXV, bETA, k * cgs, tid, t16);
-      stage3_store(st, s_xq, s_xk, s_e2, s_eta, tid);
+      {
+        Staged3 st;
+        stage3_load(st, bXQ, bXK, bXV, bETA, k * cgs, tid, t16);
+        stage3_store(st, s_xq, s_xk, s_e2, s_eta, tid);
+      }
       for (int j = 0; j < n_mb; j++) {
         const int mb = k * cgs + j;
+        Staged3 st;   // the next mini-batch's inputs on their way from HBM to LDS (not carried around the loop)
         REFRESH_OFFSETS();
         LANE_VARS;
         __syncthreads();   // the staged inputs (and, for j = 0, the biases) are visible
@@ -679,7 +703,8 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
 #pragma unroll
             for (int s = 0; s < 2; s++) chunk_store(bIMG1, j * IMG_BYTES, 2 * fb + s, t16, piece_tr<LDF>(T2, fb, s, lane));
         }
-        // post-update forward on XQ
+        // post-update forward on XQ; X2_bar rows [tok][hid] -> T0, gelu'(Z1_bar) packed
+        bf16x8 d1b[2][2];
         {
           LANE_VARS;
           AccT<1, 2> z1b;
@@ -687,42 +712,118 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
           mma_jit<4>(z1b, [&](int, int s) { return piece_state(W1s, 0, s); },
                      [&](int i, int s) { return piece_rows<LDX>(s_xq, tb[i], s, c, h); });
           bf16x8 x2bQ[2][2];
+          WAVE_SYNC();   // the weight step's readers of T0 are done
 #pragma unroll
           for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int t = 0; t < 2; t++) {
-              chunk_store(bZ1B, j * IMG_BYTES, 2 * tb[i] + t, t16, pack8(z1b.b[0][i], t));
 #pragma unroll
-              for (int jj = 0; jj < 8; jj++) x2bQ[i][t][jj] = (bf16)gelu_f(z1b.b[0][i][8 * t + jj]);
+              for (int jj = 0; jj < 8; jj++) {
+                float g, d;
+                gelu_fd(z1b.b[0][i][8 * t + jj], g, d);
+                x2bQ[i][t][jj] = (bf16)g;
+                d1b[i][t][jj] = (bf16)d;
+              }
+              store_piece_rows<LDH>(T0, tb[i], t, c, h, x2bQ[i][t]);
             }
           AccT<2, 2> z2;
           acc_zero(z2);
           mma_jit<2>(z2, [&](int rb, int s) { return piece_state(W2s, rb, s); },
                      [&](int i, int s) { return x2bQ[i][s]; });
-          if (j + 1 < n_mb)
-            stage3_load(st, bXQ, bXK, bXV, bETA, mb + 1, tid, t16);
           WAVE_SYNC();   // this wave's readers of T1 / T2 are done
           pair_sum(s_own, s_partner, z2, c, h);
-          // every reader of this mini-batch's XQ / XK / XV tiles is past the barriers above
+        }
+        // ---- the output branch, backwards: it needs the state after this step, which is in registers
+        //      right now, and nothing of the running gradients.  Output LayerNorm forward and backward:
+        float gO[8];
+        {
+          LANE_VARS;
+          // Every reader of this mini-batch's XQ / XK / XV tiles is past the barriers of the pair sum: the
+          // next ones are fetched now and land in LDS at the end of this stage, which covers their latency.
+          // (Fetched any earlier they would sit in registers across the pair sum, and be spilled.)
+          if (j + 1 < n_mb) stage3_load(st, bXQ, bXK, bXV, bETA, mb + 1, tid, t16);
+          float z[8], gx[8], gam[8];
+          {
+            float b2v[8];
+            ln_gather(z, s_lnrow);
+            ln_load_f32(b2v, s_b2 + f0);
+#pragma unroll
+            for (int e = 0; e < 8; e++) z[e] += b2v[e];
+          }
+          ln_cvt8(gO, g_ld8h(bGO, vln, mb * TILE_BYTES));
+          float sd;
+          ln_normalize(z, &sd);   // z = x_hat
+          ln_load_f32(gam, s_gam + f0);
+#pragma unroll
+          for (int e = 0; e < 8; e++) gx[e] = gO[e] * z[e];
+          ln_token_sum_add(s_dbw, gO, q8, f0);
+          ln_token_sum_add(s_dgw, gx, q8, f0);
+#pragma unroll
+          for (int e = 0; e < 8; e++) gx[e] = gO[e] * gam[e];
+          const float s1 = oct_sum(sum8(gx)), s2 = oct_sum(dot8(gx, z));
+          const float sc = 1.f / (FD * sd);
+#pragma unroll
+          for (int e = 0; e < 8; e++) gx[e] = (FD * gx[e] - s1 - z[e] * s2) * sc;
+          ln_store(s_a + tok * LDX + f0, gx);            // gZ2_bar
+          ln_store_g(bGZB, vln, j * TILE_BYTES, gx);
           if (j + 1 < n_mb) stage3_store(st, s_xq, s_xk, s_e2, s_eta, tid);
+        }
+        __syncthreads();
+        {
+          LANE_VARS;
+          {
+            LANE_VARS;
+            AccT<1, 2> gz1b;   // (gZ2_bar W2^T) * gelu'(Z1_bar): rows hid, lane = tok
+            acc_zero(gz1b);
+            mma_jit<4>(gz1b, [&](int, int s) { return piece_state(W2t, 0, s); },
+                       [&](int i, int s) { return piece_rows<LDX>(s_a, tb[i], s, c, h); });
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+              for (int t = 0; t < 2; t++) {
+                bf16x8 gzb;
+#pragma unroll
+                for (int jj = 0; jj < 8; jj++) gzb[jj] = (bf16)(gz1b.b[0][i][8 * t + jj] * (float)d1b[i][t][jj]);
+                store_piece_rows<LDH>(T1, tb[i], t, c, h, gzb);    // gZ1_bar rows [tok][hid]
+              }
+          }
+          WAVE_SYNC();
+          AccT<2, 2> dq;
+          acc_zero(dq);
+          mma_jit<2>(dq, [&](int rb, int s) { return chunk_load(bIMG1, j * IMG_BYTES, 2 * rb + s, t16); },   // W1 after: lane = F
+                     [&](int i, int s) { return piece_rows<LDH>(T1, tb[i], s, c, h); });                   // gZ1_bar: lane = tok
+          // what the reverse walk adds to the running gradients, as ready-made operands (lane = hid, contraction = tok)
+#pragma unroll
+          for (int s = 0; s < 4; s++) {
+            chunk_store(bX2B, j * IMG_BYTES, s, t16, piece_tr<LDH>(T0, 0, s, lane));
+            chunk_store(bGZ1B, j * IMG_BYTES, s, t16, piece_tr<LDH>(T1, 0, s, lane));
+          }
+          WAVE_SYNC();   // every reader of T1 / T2 is done before the pair sum takes their place
+          pair_sum(s_own, s_partner, dq, c, h);
         }
         {
           LANE_VARS;
-          float z[8], b2v[8];
+          float z[8];
           ln_gather(z, s_lnrow);
-          ln_load_f32(b2v, s_b2 + f0);
+          bf16x8 dxq_old = g_ld8h(bDXQ, vln, mb * TILE_BYTES);
 #pragma unroll
-          for (int e = 0; e < 8; e++) z[e] += b2v[e];
-          float sd;
-          ln_normalize(z, &sd);
-          ln_store_g(bXHL, vln, j * TILE_BYTES, z);
-          if ((lane & 7) == 0) g_stf(bSDL, vtok, j * (CS * 4), sd);
+          for (int e = 0; e < 8; e++) dxq_old[e] = (bf16)((float)dxq_old[e] + (z[e] + gO[e]));
+          g_st8h(bDXQ, vln, mb * TILE_BYTES, dxq_old);
+        }
+      }
+      if constexpr (ROLE == 1) {
+        if (k == 0) {   // hand this workgroup's norm-gradient sums to the one that writes the result
+          WAVE_SYNC();
+          float* np = p.norm_partial + (size_t)bh * (BW_NWAVE * 2 * FD) + v * 2 * FD;
+          np[lane] = s_dgw[lane];
+          np[FD + lane] = s_dbw[lane];
         }
       }
       // running gradients back into registers
       if constexpr (ROLE == 0) {
         acc_load_rows(gW1s, bPW1, 0, HID, 0, hid0, c, h);
         acc_load_rows(gW2s, bPW2, 0, FD, hid0, 0, c, h);
+        norm_swap();
       }
       if constexpr (ROLE == 1) publish(w_replayed, done + 1);
     }
@@ -748,101 +849,34 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
       {
         LANE_VARS;
         const u32x4 xq = g_ld16(bXQ, t16, xo), xk = g_ld16(bXK, t16, xo), gz = g_ld16(bGZ2, t16, so);
+        const u32x4 gzb = g_ld16(bGZB, t16, so);
         const float eta = bf2f(g_ldh(bETA, 2 * (tid & (CS - 1)), mb * (CS * 2)));
         lds_put16(s_xq, tid, xq);
         lds_put16(s_xk, tid, xk);
         lds_put16(s_gz2, tid, gz);
+        lds_put16(s_a, tid, gzb);
         if (tid < CS) s_eta[tid] = eta;
-      }
-      // The state after this step enters as ready-made operands: the images the replay stored are in MFMA
-      // operand layout already, so their chunks go from HBM straight into the products below.
-      bf16x8 w2a[4], w1a[2][2];   // W2: lane = hid, contraction = F;  W1^T: lane = F, contraction = hid
-      {
-        LANE_VARS;
-#pragma unroll
-        for (int s = 0; s < 4; s++) w2a[s] = chunk_load(bIMG2, ho, s, t16);
-#pragma unroll
-        for (int fb = 0; fb < 2; fb++)
-#pragma unroll
-          for (int s = 0; s < 2; s++) w1a[fb][s] = chunk_load(bIMG1, ho, 2 * fb + s, t16);
-      }
-
-      // ---- output LayerNorm backward (LayerNorm lanes)
-      float gO[8];
-      {
-        LANE_VARS;
-        float xh[8], gx[8], gam[8];
-        ln_cvt8(gO, g_ld8h(bGO, vln, xo));
-        ln_cvt8(xh, g_ld8h(bXHL, vln, so));
-        ln_load_f32(gam, s_gam + f0);
-        const float sd = g_ldf(bSDL, vtok, j * (CS * 4));
-#pragma unroll
-        for (int e = 0; e < 8; e++) gx[e] = gO[e] * xh[e];
-        ln_token_sum_add(s_dbw, gO, q8, f0);
-        ln_token_sum_add(s_dgw, gx, q8, f0);
-#pragma unroll
-        for (int e = 0; e < 8; e++) gx[e] = gO[e] * gam[e];
-        const float s1 = oct_sum(sum8(gx)), s2 = oct_sum(dot8(gx, xh));
-        const float sc = 1.f / (FD * sd);
-#pragma unroll
-        for (int e = 0; e < 8; e++) gx[e] = (FD * gx[e] - s1 - xh[e] * s2) * sc;
-        ln_store(s_a + tok * LDX + f0, gx);  // gZ2_bar
       }
       __syncthreads();
 
-      // ---- post-update forward, backwards (uses the state AFTER this mini-batch)
-      bf16x8 dxq_old;            // the output rows this lane accumulates into
+      // ---- what the output branch adds to the running gradients.  The replay has taken that branch
+      //      backwards already and left gZ2_bar (now in LDS) and X2_bar^T, gZ1_bar^T as operand images.
       {
         LANE_VARS;
-        AccT<2, 2> dq;
-        {
-          LANE_VARS;
-          AccT<1, 2> gz1b;   // (gZ2_bar W2^T) * gelu'(Z1_bar): rows hid, lane = tok
-          acc_zero(gz1b);
-          mma_jit<4>(gz1b, [&](int, int s) { return w2a[s]; },
-                     [&](int i, int s) { return piece_rows<LDX>(s_a, tb[i], s, c, h); });
+        bf16x8 x2b[4], g1b[4];   // lane = hid, contraction = tok
 #pragma unroll
-          for (int i = 0; i < 2; i++)
-#pragma unroll
-            for (int t = 0; t < 2; t++) {
-              bf16x8 x2b, gzb;
-              bf16x8 zcb[2][2];
-              zcb[i][t] = chunk_load(bZ1B, ho, 2 * tb[i] + t, t16);
-#pragma unroll
-              for (int jj = 0; jj < 8; jj++) {
-                float g, d;
-                gelu_fd((float)zcb[i][t][jj], g, d);
-                x2b[jj] = (bf16)g;
-                gzb[jj] = (bf16)(gz1b.b[0][i][8 * t + jj] * d);
-              }
-              store_piece_rows<LDH>(T0, tb[i], t, c, h, x2b);    // X2_bar  rows [tok][hid]
-              store_piece_rows<LDH>(T1, tb[i], t, c, h, gzb);    // gZ1_bar rows [tok][hid]
-            }
+        for (int s = 0; s < 4; s++) {
+          x2b[s] = chunk_load(bX2B, ho, s, t16);
+          g1b[s] = chunk_load(bGZ1B, ho, s, t16);
         }
-        WAVE_SYNC();
-        acc_zero(dq);
-        mma_jit<2>(dq, [&](int rb, int s) { return w1a[rb][s]; },                              // W1 after: lane = F
-                   [&](int i, int s) { return piece_rows<LDH>(T1, tb[i], s, c, h); });         // gZ1_bar: lane = tok
-        mma_jit<4>(gW2s, [&](int, int s) { return piece_tr<LDH>(T0, 0, s, lane); },            // X2_bar^T: lane = hid
+        mma_jit<4>(gW2s, [&](int, int s) { return x2b[s]; },                                   // X2_bar^T: lane = hid
                    [&](int fb, int s) { return piece_tr<LDX>(s_a, fb, s, lane); });            // gZ2_bar: lane = F
         if (v < 2) lds_rowsum_add_jit(s_gb2 + 32 * v, [&](int s) { return piece_tr<LDX>(s_a, v, s, lane); }, ones, c, h);
         mma_jit<4>(gW1s, [&](int fb, int s) { return piece_tr<LDX>(s_xq, fb, s, lane); },      // XQ^T: lane = F
-                   [&](int, int s) { return piece_tr<LDH>(T1, 0, s, lane); });                 // gZ1_bar: lane = hid
-        lds_rowsum_add_jit(s_gb1w, [&](int s) { return piece_tr<LDH>(T1, 0, s, lane); }, ones, c, h);
-        WAVE_SYNC();   // every reader of T1 / T2 is done before the pair sum takes their place
-        pair_sum(s_own, s_partner, dq, c, h);
+                   [&](int, int s) { return g1b[s]; });                                        // gZ1_bar: lane = hid
+        lds_rowsum_add_jit(s_gb1w, [&](int s) { return g1b[s]; }, ones, c, h);
       }
-      // pair sums of dXQ complete; gb2 holds its value after the first update
-      {
-        LANE_VARS;
-        float z[8];
-        ln_gather(z, s_lnrow);
-        dxq_old = g_ld8h(bDXQ, vln, xo);
-#pragma unroll
-        for (int e = 0; e < 8; e++) dxq_old[e] = (bf16)((float)dxq_old[e] + (z[e] + gO[e]));
-        g_st8h(bDXQ, vln, xo, dxq_old);
-      }
-      __syncthreads();  // dXQ readers of the regions are done: T1 / T2 are free again
+      // gb2 holds its value after the first update
 
       // ---- the weight step, backwards (uses the state BEFORE this mini-batch).
       //      Parked across the LayerNorm stage: X2 in T0; packed d1 = gelu'(Z1), g1 = -eta * dl/dZ1 and
@@ -1077,12 +1111,19 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
   if (tid < HID) p.grad_L_b1_init[(size_t)bh * HID + tid] = s_gb1[tid];
   if (tid < FD) p.grad_L_b2_init[(size_t)bh * FD + tid] = s_gb2[tid];
   // norm-weight / norm-bias gradients: sum the per-wave LDS accumulators
+  // (the replay's share: parked in HBM by this workgroup, or handed over by the replaying one, whose last
+  // count this workgroup has acquired before it walked the last group)
   if (tid < 2 * FD) {
     const int which = tid / FD, f = tid % FD;
-    float s = 0.f;
+    const float* rp = ROLE == 0 ? reinterpret_cast<const float*>(p.x_hat_ln_group + (size_t)bh * cgs * (CS * FD))
+                                : p.norm_partial + (size_t)bh * (BW_NWAVE * 2 * FD);
+    float s = 0.f, sr = 0.f;
 #pragma unroll
-    for (int u = 0; u < BW_NWAVE; u++) s += s_red[(u * 2 + which) * FD + f];
-    (which == 0 ? p.grad_L_ttt_norm_weight : p.grad_L_ttt_norm_bias)[(size_t)bh * FD + f] = s;
+    for (int u = 0; u < BW_NWAVE; u++) {
+      s += s_red[(u * 2 + which) * FD + f];
+      sr += rp[(u * 2 + which) * FD + f];
+    }
+    (which == 0 ? p.grad_L_ttt_norm_weight : p.grad_L_ttt_norm_bias)[(size_t)bh * FD + f] = sr + s;
   }
 }
 #undef REFRESH_OFFSETS
@@ -1094,15 +1135,16 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
 #undef bGO
 #undef bETA
 #undef bZ1
-#undef bZ1B
+#undef bGZ1B
+#undef bX2B
+#undef bGZB
+#undef bNP
 #undef bIMG1
 #undef bIMG2
 #undef bXHF
 #undef bGOF
 #undef bGZ2
-#undef bXHL
 #undef bSDF
-#undef bSDL
 #undef bPW1
 #undef bPW2
 #undef bCW1

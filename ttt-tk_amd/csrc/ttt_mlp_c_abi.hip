@@ -118,16 +118,18 @@ bool two_workgroup_mode_fits(long long BH) {
   return BH > 0 && 2 * BH <= cus;
 }
 
-// Workspace of the two-workgroup mode: the synchronisation words, then the alternate set of the ten
-// per-group tensors that carry a replayed group to the reverse walk, each part 256-byte aligned.
+// Workspace of the two-workgroup mode: the synchronisation words, the replaying workgroups' share of the
+// norm gradients, then the alternate set of the ten per-group tensors that carry a replayed group to the
+// reverse walk; each part 256-byte aligned.
 struct BwdWorkspace {
   size_t off[11];
   size_t total;
   BwdWorkspace(long long BH, long long cgs) {
     const size_t slot = (size_t)BH * (size_t)cgs;
     const size_t tile = TTT_MLP_CS * TTT_MLP_F * 2, img = TTT_MLP_CS * TTT_MLP_HID * 2, vec = TTT_MLP_CS * 4;
-    const size_t bytes[11] = {ttt::bwd_sync_ints(BH) * sizeof(int), slot * tile, slot * vec, slot * img, slot * img, slot * img,
-                              slot * tile, slot * img, slot * tile, slot * tile, slot * vec};
+    const size_t bytes[11] = {ttt::bwd_sync_ints(BH) * sizeof(int), (size_t)BH * 8 * 2 * TTT_MLP_F * sizeof(float),
+                              slot * img, slot * img, slot * img, slot * img, slot * tile, slot * img, slot * tile,
+                              slot * tile + slot * tile, slot * vec};
     size_t o = 0;
     for (int i = 0; i < 11; i++) { off[i] = o; o += (bytes[i] + 255) & ~(size_t)255; }
     total = o;
@@ -157,16 +159,18 @@ extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* wo
   const BwdWorkspace w((long long)p.B * p.NH, p.cgs);
   if (workspace_bytes < w.total) return TTT_MLP_ERR_WORKSPACE;
   char* base = static_cast<char*>(workspace);
+  const size_t slot_elems = (size_t)p.B * p.NH * p.cgs * (TTT_MLP_CS * TTT_MLP_F);   // one [B,NH,cgs,CS,F] tensor
   p.sync = reinterpret_cast<int*>(base + w.off[0]);
-  p.alt_x_hat_ln_group = reinterpret_cast<__bf16*>(base + w.off[1]);
-  p.alt_std_ln_group = reinterpret_cast<float*>(base + w.off[2]);
-  p.alt_X2_group = reinterpret_cast<__bf16*>(base + w.off[3]);
-  p.alt_Z1_group = reinterpret_cast<__bf16*>(base + w.off[4]);
-  p.alt_Z1_bar_group = reinterpret_cast<__bf16*>(base + w.off[5]);
+  p.norm_partial = reinterpret_cast<float*>(base + w.off[1]);
+  p.alt_X2_group = reinterpret_cast<__bf16*>(base + w.off[2]);
+  p.alt_Z1_group = reinterpret_cast<__bf16*>(base + w.off[3]);
+  p.alt_Z1_bar_group = reinterpret_cast<__bf16*>(base + w.off[4]);
+  p.alt_X2_bar_group = reinterpret_cast<__bf16*>(base + w.off[5]);
   p.alt_grad_l_wrt_Z2_group = reinterpret_cast<__bf16*>(base + w.off[6]);
   p.alt_grad_l_wrt_Z1_group = reinterpret_cast<__bf16*>(base + w.off[7]);
   p.alt_x_hat_fused_group = reinterpret_cast<__bf16*>(base + w.off[8]);
-  p.alt_grad_output_fused_group = reinterpret_cast<__bf16*>(base + w.off[9]);
+  p.alt_grad_x_hat_fused_group = reinterpret_cast<__bf16*>(base + w.off[9]);
+  p.alt_grad_output_fused_group = p.alt_grad_x_hat_fused_group + slot_elems;
   p.alt_std_fused_group = reinterpret_cast<float*>(base + w.off[10]);
   return static_cast<int>(ttt_mlp_bwd_enqueue(p, static_cast<hipStream_t>(stream)));
 }

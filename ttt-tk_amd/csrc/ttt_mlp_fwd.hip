@@ -173,13 +173,16 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
   const gptr_t gXQ = gbuf(p.XQ + x_base), gXK = gbuf(p.XK + x_base), gXV = gbuf(p.XV + x_base), gOut = gbuf(p.Out + x_base);
   const gptr_t gEta = gbuf(p.last_eta + uni64((size_t)bh * p.NC * CS));
   const gptr_t gW1ck = gbuf(p.W1_ck + uni64((size_t)bh * p.K * FD * HID)), gW2ck = gbuf(p.W2_ck + uni64((size_t)bh * p.K * HID * FD));
-  Staged st;
-  stage_load(st, gXQ, gXK, gXV, gEta, 0, tid);
-  stage_store(st, smem, 0, tid);
+  {
+    Staged st;
+    stage_load(st, gXQ, gXK, gXV, gEta, 0, tid);
+    stage_store(st, smem, 0, tid);
+  }
   __syncthreads();
 
   for (int mb = 0; mb < p.NC; mb++) {
     LANE_VARS;
+    Staged st;   // the next mini-batch's inputs on their way from HBM to LDS (not carried around the loop)
     const bf16* s_xq = reinterpret_cast<const bf16*>(smem + SM_XQ + (mb & 1) * SM_TILE);
 
     // ---- checkpoint: the state before this mini-batch
@@ -290,11 +293,6 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
       for (int e = 0; e < 8; e++) o[e] = (bf16)((FD * gx[e] - s1 - z[e] * s2) * scale);
       lds_put16(s_g2 + tok * FLD + f0, __builtin_bit_cast(u32x4, o));
     }
-    // the next mini-batch's inputs leave HBM now and are written to LDS at the end of this one
-    {
-      LANE_VARS;
-      if (mb + 1 < p.NC) stage_load(st, gXQ, gXK, gXV, gEta, mb + 1, tid);
-    }
     __syncthreads();
 
     // ---- G1 = (G2 W2^T) * gelu'(Z1);  state += X^T G
@@ -370,6 +368,9 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
       AccT<2, 2> z2;
       acc_zero(z2);
       mma(z2, w2A, x2bB);                          // rows F, lane = tok
+      // The next mini-batch's inputs leave HBM now and are written to LDS at the end of this one.  (Fetched
+      // before the weight step they would be spilled at once, each spill waiting for its load.)
+      if (mb + 1 < p.NC) stage_load(st, gXQ, gXK, gXV, gEta, mb + 1, tid);
       pair_sum_to_lds(s_Pp, z2, pr, c, h);
     }
 

@@ -33,17 +33,17 @@ struct BwdParams {
   int B, NH, NC, K, cgs;
   // Two-workgroup mode only (sync != nullptr): a second set of the per-group tensors that carry a
   // replayed group to the reverse walk, and the words the two workgroups of a (batch, head) signal with.
-  __bf16* alt_x_hat_ln_group;
-  float* alt_std_ln_group;
-  __bf16 *alt_X2_group, *alt_Z1_group, *alt_Z1_bar_group;
+  __bf16 *alt_X2_group, *alt_Z1_group, *alt_Z1_bar_group, *alt_X2_bar_group;
   __bf16 *alt_grad_l_wrt_Z2_group, *alt_grad_l_wrt_Z1_group;
-  __bf16 *alt_x_hat_fused_group, *alt_grad_output_fused_group;
+  __bf16 *alt_x_hat_fused_group, *alt_grad_x_hat_fused_group, *alt_grad_output_fused_group;
   float* alt_std_fused_group;
+  float* norm_partial;   // [B*NH][8 waves][2][64]: the replaying workgroup's share of the norm-weight / norm-bias gradients
   int* sync;
 };
 
-// Layout of `sync` (ints): 32 per (batch, head) - word 0 counts the groups replayed, word 16 the groups
-// the reverse walk has finished - then one status word (non-zero: a wait gave up).
+// Layout of `sync` (ints): 32 per (batch, head) - word 0 counts the groups replayed (norm_partial is
+// written before the last count), word 16 the groups the reverse walk has finished - then one status
+// word (non-zero: a wait gave up).
 constexpr int BWD_SYNC_STRIDE = 32;
 inline size_t bwd_sync_ints(long long BH) { return (size_t)BH * BWD_SYNC_STRIDE + 32; }
 
