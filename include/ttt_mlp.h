@@ -145,6 +145,14 @@ int ttt_mlp_bwd_launch(const ttt_mlp_bwd_args* args, void* stream);
  * non-zero only if a workgroup waited 20 s for the other and gave up, in which
  * case the outputs are invalid. */
 size_t ttt_mlp_bwd_workspace_bytes(int32_t B, int32_t NH, int32_t checkpoint_group_size);
+
+/* The forward with two workgroups per (batch, head), under the same conditions and with the same
+ * conventions (workspace, status word at int index B*NH*32, TTT_MLP_ERR_NO_ROOM, bit-identical
+ * results): one workgroup carries the state through the mini-batches and leaves every new state
+ * in the workspace as bf16 operands, the other computes Out from them, eight mini-batches behind.
+ * No counterpart in the reference launcher (kernels/ttt/ttt.cu:594-721). */
+size_t ttt_mlp_fwd_workspace_bytes(int32_t B, int32_t NH);
+int ttt_mlp_fwd_launch_overlapped(const ttt_mlp_fwd_args* args, void* workspace, size_t workspace_bytes, void* stream);
 int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* args, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Human-readable text for a return code of the two launchers. */

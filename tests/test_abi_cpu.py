@@ -34,7 +34,8 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points():
     assert declared_functions() == ["ttt_mlp_abi_version", "ttt_mlp_bwd_launch", "ttt_mlp_bwd_launch_overlapped",
                                     "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_error_string",
-                                    "ttt_mlp_fwd_launch", "ttt_mlp_kernel_info"]
+                                    "ttt_mlp_fwd_launch", "ttt_mlp_fwd_launch_overlapped",
+                                    "ttt_mlp_fwd_workspace_bytes", "ttt_mlp_kernel_info"]
 
 
 def test_library_exports_every_declared_symbol(lib):
@@ -89,6 +90,11 @@ def test_overlapped_backward_needs_a_device_with_room(lib):
     assert lib.ttt_mlp_bwd_workspace_bytes(0, 2, 4) == 0
     assert lib.ttt_mlp_bwd_workspace_bytes(1, 2, 0) == 0
     assert lib.ttt_mlp_bwd_launch_overlapped(None, None, ctypes.c_size_t(0), None) == 1001
+    lib.ttt_mlp_fwd_workspace_bytes.restype = ctypes.c_size_t
+    assert lib.ttt_mlp_fwd_workspace_bytes(0, 2) == 0
+    assert lib.ttt_mlp_fwd_launch_overlapped(None, None, ctypes.c_size_t(0), None) == 1001
+    if not torch.cuda.is_available():
+        assert lib.ttt_mlp_fwd_workspace_bytes(1, 2) == 0
     if not torch.cuda.is_available():
         assert lib.ttt_mlp_bwd_workspace_bytes(1, 2, 4) == 0
     assert b"ttt_mlp_bwd_launch" in lib.ttt_mlp_error_string(1005)

@@ -14,8 +14,9 @@ namespace {
 
 constexpr int64_t F = TTT_MLP_F, CS = TTT_MLP_CS, HID = TTT_MLP_HID;
 bool g_synchronize = true;  // upstream blocks the host until the kernel has finished
-bool g_overlap = true;      // backward: two workgroups per (batch, head) whenever they fit the device
-int g_last_backward_mode = -1;   // 0 = one workgroup per (batch, head), 1 = two
+bool g_overlap = true;      // two workgroups per (batch, head) whenever they fit the device
+int g_last_forward_mode = -1;    // 0 = one workgroup per (batch, head), 1 = two
+int g_last_backward_mode = -1;
 
 void check_tensor(const torch::Tensor& t, const char* name, c10::ScalarType dtype, std::initializer_list<int64_t> shape) {
   TORCH_CHECK(t.device().is_cuda(), "Invalid dims for ", name, ": not a GPU tensor");
@@ -87,8 +88,20 @@ torch::Tensor ttt_forward(const torch::Tensor XQ, const torch::Tensor XK, const 
   a.Out = bfp_mut(Out);
   a.checkpoint_group_size = checkpoint_group_size;
   a.B = (int32_t)B; a.NH = (int32_t)NH; a.NC = (int32_t)NC; a.K = (int32_t)K;
+  const c10::DeviceGuard guard(XQ.device());
   hipStream_t stream = c10::hip::getCurrentHIPStream(XQ.device().index()).stream();
-  finish(ttt_mlp_fwd_launch(&a, stream), stream, "ttt_forward");
+  // With few (batch, head) pairs most CUs would idle: then a second workgroup per pair computes Out behind
+  // the state recurrence.  Its workspace comes from torch's caching allocator, which orders its reuse
+  // after this launch on the same stream.
+  const size_t ws_bytes = (g_overlap && NC >= 2) ? ttt_mlp_fwd_workspace_bytes((int32_t)B, (int32_t)NH) : 0;
+  if (ws_bytes > 0) {
+    torch::Tensor ws = torch::empty({(int64_t)ws_bytes}, torch::TensorOptions().dtype(torch::kUInt8).device(XQ.device()));
+    g_last_forward_mode = 1;
+    finish(ttt_mlp_fwd_launch_overlapped(&a, ws.data_ptr(), ws_bytes, stream), stream, "ttt_forward");
+  } else {
+    g_last_forward_mode = 0;
+    finish(ttt_mlp_fwd_launch(&a, stream), stream, "ttt_forward");
+  }
   return Out;
 }
 
@@ -211,9 +224,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   // the host synchronisation the upstream operator performs on every call.
   m.def("set_synchronize", [](bool on) { g_synchronize = on; }, "Block the host after each launch (default true).");
   m.def("abi_version", []() { return ttt_mlp_abi_version(); });
-  // Also not upstream: choice of the backward's launch shape (results are bit-identical either way).
+  // Also not upstream: choice of the launch shape (results are bit-identical either way).
   m.def("set_overlap", [](bool on) { g_overlap = on; },
-        "Backward: recompute checkpoint groups on a second workgroup per (batch, head) when the device has room (default true).");
+        "Use a second workgroup per (batch, head) when the device has room: the forward's output branch, the "
+        "backward's recomputation of checkpoint groups (default true).");
+  m.def("last_forward_mode", []() { return g_last_forward_mode; },
+        "0: the last ttt_forward used one workgroup per (batch, head); 1: two; -1: none yet.");
   m.def("last_backward_mode", []() { return g_last_backward_mode; },
         "0: the last ttt_backward used one workgroup per (batch, head); 1: two; -1: none yet.");
 }

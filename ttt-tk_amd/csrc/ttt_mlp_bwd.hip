@@ -376,33 +376,6 @@ TTT_DEV bf16x8 w1_before(gptr_t img, gptr_t ck, unsigned ck_off, int j, int rb, 
 // counters in HBM (agent scope); both are resident at once because the launcher uses this mode only
 // when the grid fits the CUs of the device.  A wait that sees no progress for SPIN_LIMIT ticks of the
 // 100 MHz clock raises the status word and both workgroups leave, so every wave always exits.
-constexpr uint64_t SPIN_LIMIT = 2000000000ull;   // 20 s
-TTT_DEV bool wait_at_least(int* word, int target, int* status, int* s_flag) {
-  if (threadIdx.x == 0) {
-    int ok = 1;
-    const uint64_t t0 = wall_clock64();
-    while (__hip_atomic_load(word, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < target) {
-      if (__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 || wall_clock64() - t0 > SPIN_LIMIT) {
-        __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        ok = 0;
-        break;
-      }
-      __builtin_amdgcn_s_sleep(32);
-    }
-    *s_flag = ok;
-  }
-  __syncthreads();
-  const int ok = *s_flag;
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-  return ok != 0;
-}
-// Everything this workgroup has written (or read) so far is ordered before the new value of `word`.
-TTT_DEV void publish(int* word, int value) {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-  __syncthreads();
-  if (threadIdx.x == 0) __hip_atomic_store(word, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-}
-
 // ROLE 0: replay and reverse walk of every group in one workgroup; 1: the replays only; 2: the reverse walks only.
 template <int ROLE>
 TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {

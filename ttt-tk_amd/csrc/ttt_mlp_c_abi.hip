@@ -42,7 +42,8 @@ extern "C" const char* ttt_mlp_error_string(int code) {
   }
 }
 
-extern "C" int ttt_mlp_fwd_launch(const ttt_mlp_fwd_args* a, void* stream) {
+namespace {
+int make_fwd_params(const ttt_mlp_fwd_args* a, ttt::FwdParams& p) {
   if (a == nullptr) return TTT_MLP_ERR_BAD_ARG;
   if (any_null(a->XQ, a->XK, a->XV, a->last_eta, a->ttt_norm_weight, a->ttt_norm_bias, a->W1, a->b1, a->W2, a->b2,
                a->W1_checkpoints, a->b1_checkpoints, a->W2_checkpoints, a->b2_checkpoints, a->Out))
@@ -51,15 +52,16 @@ extern "C" int ttt_mlp_fwd_launch(const ttt_mlp_fwd_args* a, void* stream) {
   if (!all_aligned(a->XQ, a->XK, a->XV, a->last_eta, a->ttt_norm_weight, a->ttt_norm_bias, a->W1, a->b1, a->W2,
                    a->b2, a->W1_checkpoints, a->b1_checkpoints, a->W2_checkpoints, a->b2_checkpoints, a->Out))
     return TTT_MLP_ERR_ALIGN;
-  ttt::FwdParams p;
+  p = ttt::FwdParams{};
   p.XQ = bf(a->XQ); p.XK = bf(a->XK); p.XV = bf(a->XV); p.last_eta = bf(a->last_eta);
   p.ttt_norm_weight = a->ttt_norm_weight; p.ttt_norm_bias = a->ttt_norm_bias;
   p.W1 = a->W1; p.b1 = a->b1; p.W2 = a->W2; p.b2 = a->b2;
   p.W1_ck = a->W1_checkpoints; p.b1_ck = a->b1_checkpoints; p.W2_ck = a->W2_checkpoints; p.b2_ck = a->b2_checkpoints;
   p.Out = bf(a->Out);
   p.B = a->B; p.NH = a->NH; p.NC = a->NC; p.K = a->K; p.cgs = a->checkpoint_group_size;
-  return static_cast<int>(ttt_mlp_fwd_enqueue(p, static_cast<hipStream_t>(stream)));
+  return TTT_MLP_OK;
 }
+}  // namespace
 
 namespace {
 
@@ -173,6 +175,50 @@ extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* wo
   p.alt_grad_output_fused_group = p.alt_grad_x_hat_fused_group + slot_elems;
   p.alt_std_fused_group = reinterpret_cast<float*>(base + w.off[10]);
   return static_cast<int>(ttt_mlp_bwd_enqueue(p, static_cast<hipStream_t>(stream)));
+}
+
+// Workspace of the forward's two-workgroup mode: synchronisation words, then per (batch, head) a ring of
+// 2 * FWD_RING slots of state images and of bias vectors.
+namespace {
+struct FwdWorkspace {
+  size_t off[3];
+  size_t total;
+  explicit FwdWorkspace(long long BH) {
+    const size_t slots = (size_t)BH * 2 * ttt::FWD_RING;
+    const size_t bytes[3] = {ttt::bwd_sync_ints(BH) * sizeof(int), slots * ttt::FWD_IMG_BYTES,
+                             slots * ttt::FWD_BIAS_FLOATS * sizeof(float)};
+    size_t o = 0;
+    for (int i = 0; i < 3; i++) { off[i] = o; o += (bytes[i] + 255) & ~(size_t)255; }
+    total = o;
+  }
+};
+}  // namespace
+
+extern "C" int ttt_mlp_fwd_launch(const ttt_mlp_fwd_args* a, void* stream) {
+  ttt::FwdParams p;
+  if (int rc = make_fwd_params(a, p)) return rc;
+  return static_cast<int>(ttt_mlp_fwd_enqueue(p, static_cast<hipStream_t>(stream)));
+}
+
+extern "C" size_t ttt_mlp_fwd_workspace_bytes(int B, int NH) {
+  if (B <= 0 || NH <= 0) return 0;
+  if (!two_workgroup_mode_fits((long long)B * NH)) return 0;
+  return FwdWorkspace((long long)B * NH).total;
+}
+
+extern "C" int ttt_mlp_fwd_launch_overlapped(const ttt_mlp_fwd_args* a, void* workspace, size_t workspace_bytes, void* stream) {
+  ttt::FwdParams p;
+  if (int rc = make_fwd_params(a, p)) return rc;
+  if (workspace == nullptr) return TTT_MLP_ERR_BAD_ARG;
+  if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return TTT_MLP_ERR_ALIGN;
+  if (!two_workgroup_mode_fits((long long)p.B * p.NH)) return TTT_MLP_ERR_NO_ROOM;
+  const FwdWorkspace w((long long)p.B * p.NH);
+  if (workspace_bytes < w.total) return TTT_MLP_ERR_WORKSPACE;
+  char* base = static_cast<char*>(workspace);
+  p.sync = reinterpret_cast<int*>(base + w.off[0]);
+  p.state_img = reinterpret_cast<__bf16*>(base + w.off[1]);
+  p.bias_img = reinterpret_cast<float*>(base + w.off[2]);
+  return static_cast<int>(ttt_mlp_fwd_enqueue(p, static_cast<hipStream_t>(stream)));
 }
 
 extern "C" int ttt_mlp_kernel_info(int which, int* lds_bytes, int* threads_per_workgroup) {

@@ -352,4 +352,43 @@ TTT_DEV void gelu_fdd(float x, float& g, float& d1, float& d2) {
   d2 = s * (__builtin_fmaf(u, 2.f * GK2, GK0) - x * t * q * q);
 }
 
+// ---------------------------------------------------------------------------- workgroups that wait for each other
+// Two workgroups of one (batch, head) hand work over through counters in HBM (agent scope).  Both are
+// resident at once because the launchers use such a mode only when the grid fits the CUs of the device.
+// A wait that sees no progress for SPIN_LIMIT ticks of the 100 MHz clock raises the status word and
+// makes both workgroups leave, so every wave always exits.
+constexpr uint64_t SPIN_LIMIT = 2000000000ull;   // 20 s
+TTT_DEV bool wait_at_least(int* word, int target, int* status, int* s_flag) {
+  if (threadIdx.x == 0) {
+    int ok = 1;
+    const uint64_t t0 = wall_clock64();
+    // polled without acquire semantics (an acquire at agent scope invalidates caches on every poll);
+    // one acquire fence once the value is there
+    while (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+      if (__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 || wall_clock64() - t0 > SPIN_LIMIT) {
+        __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ok = 0;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(32);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    *s_flag = ok;
+  }
+  // The other waves share this CU's caches with thread 0 and are ordered after its fence by the barrier.
+  __syncthreads();
+  return *s_flag != 0;
+}
+// Everything this workgroup has written (or read) so far is ordered before the new value of `word`: every
+// wave's accesses are complete at the barrier, then one thread releases them at agent scope (a release by
+// every wave would write the L2 back eight times over).
+TTT_DEV void publish(int* word, int value) {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    __hip_atomic_store(word, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 }  // namespace ttt

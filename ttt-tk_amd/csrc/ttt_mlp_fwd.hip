@@ -43,7 +43,8 @@ constexpr int SM_B2 = SM_B1 + HID * 4;
 constexpr int SM_ETA = SM_B2 + FD * 4;
 constexpr int SM_GAM = SM_ETA + CS * 4;
 constexpr int SM_BET = SM_GAM + FD * 4;
-constexpr int SM_FWD_BYTES = SM_BET + FD * 4;
+constexpr int SM_FLAG = SM_BET + FD * 4;                 // outcome of a wait on the other workgroup
+constexpr int SM_FWD_BYTES = SM_FLAG + 16;
 static_assert(SM_FWD_BYTES <= 160 * 1024, "forward LDS budget");
 
 // 16 bytes to / from an 8-byte aligned LDS address.
@@ -111,15 +112,53 @@ TTT_DEV void pair_sum_to_lds(float* tile, const AccT<2, 2>& z, int r, int c, int
   __syncthreads();
 }
 
-__global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams p) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const bf16* s_xk = reinterpret_cast<const bf16*>(smem + SM_XK);
-  const bf16* s_xv = reinterpret_cast<const bf16*>(smem + SM_XV);
+// Output LayerNorm + residual for the 8 features [f0, f0+8) of token `tok`: Out = XQ + LN(sum of the four
+// pair sums + b2).  8 lanes per token, 8 tokens per wave.
+TTT_DEV void output_layernorm(const float* s_P, const float* s_b2, const float* s_gam, const float* s_bet,
+                              const bf16* s_xq, gptr_t gOut, int mb, int tok, int f0) {
+  float z[8];
+  {
+    f32x4 a0 = *reinterpret_cast<const f32x4*>(s_b2 + f0);
+    f32x4 a1 = *reinterpret_cast<const f32x4*>(s_b2 + f0 + 4);
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      a0 += *reinterpret_cast<const f32x4*>(s_P + t * 64 * LDP + tok * LDP + f0);
+      a1 += *reinterpret_cast<const f32x4*>(s_P + t * 64 * LDP + tok * LDP + f0 + 4);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; e++) { z[e] = a0[e]; z[4 + e] = a1[e]; }
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; e++) sum += z[e];
+  const float mu = oct_sum(sum) * (1.f / FD);
+  float var = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; e++) { z[e] -= mu; var = __builtin_fmaf(z[e], z[e], var); }
+  const float rstd = __builtin_amdgcn_rsqf(oct_sum(var) * (1.f / FD) + LN_EPS);
+  const bf16x8 qv = lds_get8h(s_xq + tok * FLD + f0);
+  float gam[8], bet[8];
+#pragma unroll
+  for (int q = 0; q < 2; q++) {
+    const f32x4 gq = *reinterpret_cast<const f32x4*>(s_gam + f0 + 4 * q);
+    const f32x4 bq = *reinterpret_cast<const f32x4*>(s_bet + f0 + 4 * q);
+#pragma unroll
+    for (int e = 0; e < 4; e++) { gam[4 * q + e] = gq[e]; bet[4 * q + e] = bq[e]; }
+  }
+  bf16x8 o;
+#pragma unroll
+  for (int e = 0; e < 8; e++) o[e] = (bf16)(bf2f(qv[e]) + __builtin_fmaf(gam[e], z[e] * rstd, bet[e]));
+  g_st8h(gOut, (tok * FD + f0) * 2, mb * TILE_BYTES, o);
+}
+
+// ROLE 0: the whole scan in one workgroup.  ROLE 1: the state recurrence only - after every mini-batch
+// the new state is left in HBM as ready-made bf16 operands for the workgroup that runs fwd_output_branch.
+template <int ROLE>
+TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
   bf16* s_g2 = reinterpret_cast<bf16*>(smem + SM_G2);
   float* s_P = reinterpret_cast<float*>(smem + SM_P);
   float* s_b1 = reinterpret_cast<float*>(smem + SM_B1);
   float* s_b2 = reinterpret_cast<float*>(smem + SM_B2);
-  const float* s_eta = reinterpret_cast<const float*>(smem + SM_ETA);
   float* s_gam = reinterpret_cast<float*>(smem + SM_GAM);
   float* s_bet = reinterpret_cast<float*>(smem + SM_BET);
 
@@ -127,7 +166,7 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
   const int v = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave index, in a scalar register
   const int pr = v >> 2;                                    // index inside the wave pair (v & 3)
   const int tok = 8 * v + (lane >> 3), f0 = 8 * (lane & 7); // LayerNorm ownership: 8 lanes per token, 8 features each
-  const int bh = blockIdx.x, head = bh % p.NH;
+  const int head = bh % p.NH;
   const int hid0 = FW_NS * v;
   float* s_Pp = s_P + (v & 3) * 64 * LDP;
   bf16* s_x2t = reinterpret_cast<bf16*>(smem + SM_X2T + v * SM_X2T_TILE);
@@ -180,14 +219,34 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
   }
   __syncthreads();
 
+  int* const w_given = p.sync + (size_t)bh * BWD_SYNC_STRIDE;   // groups handed to the output branch
+  int* const w_taken = w_given + 16;                             // groups it has finished
+  int* const w_status = p.sync + (size_t)p.B * p.NH * BWD_SYNC_STRIDE;
+  int* const s_flag = reinterpret_cast<int*>(smem + SM_FLAG);
+
   for (int mb = 0; mb < p.NC; mb++) {
     LANE_VARS;
     Staged st;   // the next mini-batch's inputs on their way from HBM to LDS (not carried around the loop)
     const bf16* s_xq = reinterpret_cast<const bf16*>(smem + SM_XQ + (mb & 1) * SM_TILE);
+    // ROLE 1 has no use for XQ (nor for b1 in LDS): their space holds a second XK / XV / eta buffer, so that
+    // the next mini-batch's inputs can be written while this one's are still being read.
+    const int alt = ROLE == 1 ? (mb & 1) : 0;
+    const bf16* s_xk = reinterpret_cast<const bf16*>(smem + (alt ? SM_XQ : SM_XK));
+    const bf16* s_xv = reinterpret_cast<const bf16*>(smem + (alt ? SM_XQ + SM_TILE : SM_XV));
+    const float* s_eta = reinterpret_cast<const float*>(smem + (alt ? SM_B1 : SM_ETA));
+    // ROLE 1: where the state after this mini-batch goes (a ring of 2 * FWD_RING slots)
+    const int grp = mb / FWD_RING, slot = (grp & 1) * FWD_RING + mb % FWD_RING;
+    float* const gB = p.bias_img + ((size_t)bh * 2 * FWD_RING + slot) * FWD_BIAS_FLOATS;
+    if constexpr (ROLE == 1) {
+      if (mb % FWD_RING == 0 && grp >= 2) {   // the set is free once the output branch is done with the group before last
+        if (!wait_at_least(w_taken, grp - 1, w_status, s_flag)) return;
+      }
+    }
 
     // ---- checkpoint: the state before this mini-batch
     if (mb % p.cgs == 0) {
       LANE_VARS;
+      if constexpr (ROLE == 1) __syncthreads();   // b2 as waves 0 and 1 left it (no barrier ends a mini-batch in this role)
       const size_t slot = (size_t)bh * p.K + mb / p.cgs;
       const unsigned ck = (mb / p.cgs) * (FD * HID * 4);   // byte offset of the slot in gW1ck / gW2ck
 #pragma unroll
@@ -244,6 +303,13 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
     // ---- LayerNorm-fused reconstruction-loss gradient: 8 tokens per wave, 8 lanes per token
     {
       LANE_VARS;
+      if constexpr (ROLE == 1) {   // next XK / XV / eta leave HBM now and land in the other buffers at the end of this stage
+        if (mb + 1 < p.NC) {
+          st.k = g_ld16(gXK, 16 * tid, (mb + 1) * TILE_BYTES);
+          st.v = g_ld16(gXV, 16 * tid, (mb + 1) * TILE_BYTES);
+          st.eta = bf2f(g_ldh(gEta, 2 * (tid & (CS - 1)), (mb + 1) * (CS * 2)));
+        }
+      }
       float z[8];
       {
         f32x4 a0 = *reinterpret_cast<const f32x4*>(s_b2 + f0);
@@ -292,6 +358,14 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
 #pragma unroll
       for (int e = 0; e < 8; e++) o[e] = (bf16)((FD * gx[e] - s1 - z[e] * s2) * scale);
       lds_put16(s_g2 + tok * FLD + f0, __builtin_bit_cast(u32x4, o));
+      if constexpr (ROLE == 1) {
+        if (mb + 1 < p.NC) {
+          const int off = ((tid >> 3) * FLD + (tid & 7) * 8) * 2;
+          lds_put16(smem + (alt ? SM_XK : SM_XQ) + off, st.k);
+          lds_put16(smem + (alt ? SM_XV : SM_XQ + SM_TILE) + off, st.v);
+          if (tid < CS) reinterpret_cast<float*>(smem + (alt ? SM_ETA : SM_B1))[tid] = st.eta;
+        }
+      }
     }
     __syncthreads();
 
@@ -332,17 +406,38 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
           for (int g = 0; g < 4; g++) {
             f32x4 x = {b2acc[4 * g], b2acc[4 * g + 1], b2acc[4 * g + 2], b2acc[4 * g + 3]};
             *reinterpret_cast<f32x4*>(s_b2 + 32 * v + 8 * g + 4 * h) = x;
+            if constexpr (ROLE == 1) *reinterpret_cast<f32x4*>(gB + HID + 32 * v + 8 * g + 4 * h) = x;
           }
         }
       }
       const OpdT<2, 4> xkT = lds_tr_kappa<2, 4>(s_xk, FLD, lane);      // lane = F, contraction = tok
       mma(W1s, xkT, g1op);                                             // W1[:,shard]   += XK^T G1
     }
-    {
+    if constexpr (ROLE != 1) {
       LANE_VARS;
       if (h == 0) s_b1[hid0 + c] = b1L;      // read back below by this wave only
     }
     TTT_WAVE_SYNC();
+
+    if constexpr (ROLE == 1) {
+      // ---- hand the state after this mini-batch to the output branch: W1s and W2s exactly as the
+      //      post-update forward would convert them, and the two bias vectors
+      LANE_VARS;
+      const gptr_t gImg = gbuf(p.state_img + ((size_t)bh * 2 * FWD_RING + slot) * (FWD_IMG_BYTES / 2));
+      const OpdT<1, 4> w1A = cvt_chain(W1s);
+      const OpdT<2, 2> w2A = cvt_chain(W2s);
+#pragma unroll
+      for (int s = 0; s < 4; s++) g_st8h(gImg, 16 * tid, s * 8192, w1A.v[0][s]);
+#pragma unroll
+      for (int fb = 0; fb < 2; fb++)
+#pragma unroll
+        for (int s = 0; s < 2; s++) g_st8h(gImg, 16 * tid, (4 + 2 * fb + s) * 8192, w2A.v[fb][s]);
+      if (h == 0) gB[hid0 + c] = b1L;
+      if (mb % FWD_RING == FWD_RING - 1 || mb == p.NC - 1) publish(w_given, grp + 1);
+      // No barrier ends a mini-batch here: every LDS buffer written from now on was last read before a
+      // barrier that its writers have yet to pass (the pair sum's, or the one after the LayerNorm stage).
+      continue;
+    }
 
     // ---- post-update forward on XQ, transposed: Z1b^T = W1s^T XQ^T (rows hid, lane = tok)
     {
@@ -377,39 +472,7 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
     // ---- output LayerNorm + residual, 8 tokens per wave; next mini-batch's inputs into LDS
     {
       LANE_VARS;
-      float z[8];
-      {
-        f32x4 a0 = *reinterpret_cast<const f32x4*>(s_b2 + f0);
-        f32x4 a1 = *reinterpret_cast<const f32x4*>(s_b2 + f0 + 4);
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-          a0 += *reinterpret_cast<const f32x4*>(s_P + t * 64 * LDP + tok * LDP + f0);
-          a1 += *reinterpret_cast<const f32x4*>(s_P + t * 64 * LDP + tok * LDP + f0 + 4);
-        }
-#pragma unroll
-        for (int e = 0; e < 4; e++) { z[e] = a0[e]; z[4 + e] = a1[e]; }
-      }
-      float sum = 0.f;
-#pragma unroll
-      for (int e = 0; e < 8; e++) sum += z[e];
-      const float mu = oct_sum(sum) * (1.f / FD);
-      float var = 0.f;
-#pragma unroll
-      for (int e = 0; e < 8; e++) { z[e] -= mu; var = __builtin_fmaf(z[e], z[e], var); }
-      const float rstd = __builtin_amdgcn_rsqf(oct_sum(var) * (1.f / FD) + LN_EPS);
-      const bf16x8 qv = lds_get8h(s_xq + tok * FLD + f0);
-      float gam[8], bet[8];
-#pragma unroll
-      for (int q = 0; q < 2; q++) {
-        const f32x4 gq = *reinterpret_cast<const f32x4*>(s_gam + f0 + 4 * q);
-        const f32x4 bq = *reinterpret_cast<const f32x4*>(s_bet + f0 + 4 * q);
-#pragma unroll
-        for (int e = 0; e < 4; e++) { gam[4 * q + e] = gq[e]; bet[4 * q + e] = bq[e]; }
-      }
-      bf16x8 o;
-#pragma unroll
-      for (int e = 0; e < 8; e++) o[e] = (bf16)(bf2f(qv[e]) + __builtin_fmaf(gam[e], z[e] * rstd, bet[e]));
-      g_st8h(gOut, (tok * FD + f0) * 2, mb * TILE_BYTES, o);
+      output_layernorm(s_P, s_b2, s_gam, s_bet, s_xq, gOut, mb, tok, f0);
     }
     // XK / XV were last read before the pair sum above; the XQ buffer written here is the other one.
     {
@@ -418,7 +481,121 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams
     }
     __syncthreads();
   }
+}
+
+// The output branch of the forward on its own workgroup: Out[mb] = XQ + LN(gelu(XQ W1' + b1') W2' + b2')
+// with the state after mini-batch mb, taken from the operand images the recurrence leaves behind.  Nothing
+// is carried from one mini-batch to the next here.
+TTT_DEV void fwd_output_branch(const FwdParams& p, unsigned char* smem, const int bh) {
+  float* s_P = reinterpret_cast<float*>(smem + SM_P);
+  float* s_b1 = reinterpret_cast<float*>(smem + SM_B1);
+  float* s_b2 = reinterpret_cast<float*>(smem + SM_B2);   // two buffers: the second takes the place of the eta vector
+  static_assert(SM_ETA == SM_B2 + FD * 4, "the second b2 buffer aliases the eta vector");
+  float* s_gam = reinterpret_cast<float*>(smem + SM_GAM);
+  float* s_bet = reinterpret_cast<float*>(smem + SM_BET);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int v = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int pr = v >> 2;
+  const int head = bh % p.NH;
+  const int hid0 = FW_NS * v;
+  float* s_Pp = s_P + (v & 3) * 64 * LDP;
+  int lane_v = lane;
+  if (tid < FD) {
+    s_gam[tid] = p.ttt_norm_weight[head * FD + tid];
+    s_bet[tid] = p.ttt_norm_bias[head * FD + tid];
+  }
+  const size_t x_base = uni64((size_t)bh * p.NC * (CS * FD));
+  const gptr_t gXQ = gbuf(p.XQ + x_base), gOut = gbuf(p.Out + x_base);
+  int* const w_given = p.sync + (size_t)bh * BWD_SYNC_STRIDE;
+  int* const w_taken = w_given + 16;
+  int* const w_status = p.sync + (size_t)p.B * p.NH * BWD_SYNC_STRIDE;
+  int* const s_flag = reinterpret_cast<int*>(smem + SM_FLAG);
+
+  for (int mb = 0; mb < p.NC; mb++) {
+    LANE_VARS;
+    const int grp = mb / FWD_RING, slot = (grp & 1) * FWD_RING + mb % FWD_RING;
+    if (mb % FWD_RING == 0) {
+      if (!wait_at_least(w_given, grp + 1, w_status, s_flag)) return;
+    }
+    bf16* s_xq = reinterpret_cast<bf16*>(smem + SM_XQ + (mb & 1) * SM_TILE);
+    const gptr_t gImg = gbuf(p.state_img + ((size_t)bh * 2 * FWD_RING + slot) * (FWD_IMG_BYTES / 2));
+    const float* gB = p.bias_img + ((size_t)bh * 2 * FWD_RING + slot) * FWD_BIAS_FLOATS;
+    {
+      LANE_VARS;
+      // XQ and b2 alternate between two LDS buffers: other waves may still be in the previous mini-batch's
+      // LayerNorm, which reads both.  (b1 is read before the pair sum's barriers only.)
+      const u32x4 q = g_ld16(gXQ, 16 * tid, mb * TILE_BYTES);
+      float bv = 0.f;
+      if (tid < FWD_BIAS_FLOATS) bv = gB[tid];
+      lds_put16(smem + SM_XQ + (mb & 1) * SM_TILE + ((tid >> 3) * FLD + (tid & 7) * 8) * 2, q);
+      if (tid < HID) s_b1[tid] = bv;
+      else if (tid < FWD_BIAS_FLOATS) s_b2[(mb & 1) * FD + tid - HID] = bv;
+    }
+    __syncthreads();   // XQ and the biases are visible; the previous mini-batch's readers of s_P are done
+    {
+      LANE_VARS;
+      OpdT<1, 4> w1A;
+      OpdT<2, 2> w2A;
+#pragma unroll
+      for (int s = 0; s < 4; s++) w1A.v[0][s] = g_ld8h(gImg, 16 * tid, s * 8192);
+#pragma unroll
+      for (int fb = 0; fb < 2; fb++)
+#pragma unroll
+        for (int s = 0; s < 2; s++) w2A.v[fb][s] = g_ld8h(gImg, 16 * tid, (4 + 2 * fb + s) * 8192);
+      const OpdT<2, 4> xqB = lds_rows_kappa<2, 4>(s_xq, FLD, c, h);
+      AccT<1, 2> z1b;
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const f32x4 bv = *reinterpret_cast<const f32x4*>(s_b1 + hid0 + 8 * g + 4 * h);
+#pragma unroll
+        for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) z1b.b[0][cb][4 * g + e] = bv[e];
+      }
+      mma(z1b, w1A, xqB);
+#pragma unroll
+      for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) z1b.b[0][cb][i] = gelu_f(z1b.b[0][cb][i]);
+      const OpdT<2, 2> x2bB = cvt_chain(z1b);      // lane = tok, contraction = hid
+      AccT<2, 2> z2;
+      acc_zero(z2);
+      mma(z2, w2A, x2bB);                          // rows F, lane = tok
+      pair_sum_to_lds(s_Pp, z2, pr, c, h);
+    }
+    {
+      LANE_VARS;
+      output_layernorm(s_P, s_b2 + (mb & 1) * FD, s_gam, s_bet, s_xq, gOut, mb, tok, f0);
+    }
+    if (mb % FWD_RING == FWD_RING - 1 || mb == p.NC - 1) publish(w_taken, grp + 1);
+  }
 #undef LANE_VARS
+}
+
+__global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  fwd_body<0>(p, smem, blockIdx.x);
+}
+
+// Two workgroups per (batch, head), placed like those of the backward (same XCD where the count allows).
+__global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_split_kernel(const FwdParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int b = blockIdx.x;
+  int bh, role;
+  if ((p.B * p.NH) % 8 == 0) {
+    bh = (b >> 4) * 8 + (b & 7);
+    role = (b >> 3) & 1;
+  } else {
+    bh = b >> 1;
+    role = b & 1;
+  }
+  if (role == 0) fwd_body<1>(p, smem, bh);
+  else fwd_output_branch(p, smem, bh);
+}
+
+__global__ void ttt_mlp_fwd_zero_words(int* w, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) w[i] = 0;
 }
 
 }  // namespace ttt
@@ -428,9 +605,18 @@ extern "C" int ttt_mlp_fwd_threads() { return ttt::FW_THREADS; }
 
 hipError_t ttt_mlp_fwd_enqueue(const ttt::FwdParams& p, hipStream_t stream) {
   // Per-device attribute; cheap enough to set on every launch.
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(ttt::ttt_mlp_fwd_kernel),
+  if (p.sync == nullptr) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(ttt::ttt_mlp_fwd_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, ttt::SM_FWD_BYTES);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(ttt::ttt_mlp_fwd_kernel, dim3(p.B * p.NH), dim3(ttt::FW_THREADS), ttt::SM_FWD_BYTES, stream, p);
+    return hipGetLastError();
+  }
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(ttt::ttt_mlp_fwd_split_kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, ttt::SM_FWD_BYTES);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(ttt::ttt_mlp_fwd_kernel, dim3(p.B * p.NH), dim3(ttt::FW_THREADS), ttt::SM_FWD_BYTES, stream, p);
+  const int n = static_cast<int>(ttt::bwd_sync_ints((long long)p.B * p.NH));
+  hipLaunchKernelGGL(ttt::ttt_mlp_fwd_zero_words, dim3((n + 255) / 256), dim3(256), 0, stream, p.sync, n);
+  hipLaunchKernelGGL(ttt::ttt_mlp_fwd_split_kernel, dim3(2 * p.B * p.NH), dim3(ttt::FW_THREADS), ttt::SM_FWD_BYTES, stream, p);
   return hipGetLastError();
 }

@@ -12,7 +12,16 @@ struct FwdParams {
   float *W1_ck, *b1_ck, *W2_ck, *b2_ck;
   __bf16* Out;
   int B, NH, NC, K, cgs;
+  // Two-workgroup mode only (sync != nullptr): per (batch, head) a ring of 2 * FWD_RING mini-batch slots
+  // with the bf16 operand images (64 KiB) and the bias vectors (256 + 64 floats) of the state after a
+  // mini-batch, and the words the two workgroups signal with (layout as in the backward).
+  __bf16* state_img;
+  float* bias_img;
+  int* sync;
 };
+constexpr int FWD_RING = 8;                    // mini-batches per hand-over
+constexpr int FWD_IMG_BYTES = 64 * 256 * 2 * 2;  // W1 and W2 as bf16 operands
+constexpr int FWD_BIAS_FLOATS = 256 + 64;
 
 struct BwdParams {
   const __bf16 *XQ, *XK, *XV, *last_eta;
@@ -49,6 +58,7 @@ inline size_t bwd_sync_ints(long long BH) { return (size_t)BH * BWD_SYNC_STRIDE 
 
 }  // namespace ttt
 
+// p.sync == nullptr: one workgroup per (batch, head); otherwise two (state recurrence / output branch).
 hipError_t ttt_mlp_fwd_enqueue(const ttt::FwdParams& p, hipStream_t stream);
 // p.sync == nullptr: one workgroup per (batch, head); otherwise two (replay / reverse walk).
 hipError_t ttt_mlp_bwd_enqueue(const ttt::BwdParams& p, hipStream_t stream);
