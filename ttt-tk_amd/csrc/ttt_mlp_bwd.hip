@@ -818,12 +818,12 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
       const unsigned ho = j * IMG_BYTES;         // its slot in the [cgs][64][256] scratch tensors
       // eta of the token this lane holds in column block i of a Q-orientation tile
       const float eta_i[2] = {bf2f(g_ldh(bETA, 2 * c, mb * (CS * 2) + 64 * tb[0])), bf2f(g_ldh(bETA, 2 * c, mb * (CS * 2) + 64 * tb[1]))};
-      __syncthreads();
       {
         LANE_VARS;
         const u32x4 xq = g_ld16(bXQ, t16, xo), xk = g_ld16(bXK, t16, xo), gz = g_ld16(bGZ2, t16, so);
         const u32x4 gzb = g_ld16(bGZB, t16, so);
         const float eta = bf2f(g_ldh(bETA, 2 * (tid & (CS - 1)), mb * (CS * 2)));
+        __syncthreads();   // the previous mini-batch's readers of these tiles are done (the loads are under way)
         lds_put16(s_xq, tid, xq);
         lds_put16(s_xk, tid, xk);
         lds_put16(s_gz2, tid, gz);
@@ -834,6 +834,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
 
       // ---- what the output branch adds to the running gradients.  The replay has taken that branch
       //      backwards already and left gZ2_bar (now in LDS) and X2_bar^T, gZ1_bar^T as operand images.
+      bf16x8 w2bf[4];   // W2 before this step (lane = hid, contraction = F): fetched now, needed by the next stage
       {
         LANE_VARS;
         bf16x8 x2b[4], g1b[4];   // lane = hid, contraction = tok
@@ -842,6 +843,8 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
           x2b[s] = chunk_load(bX2B, ho, s, t16);
           g1b[s] = chunk_load(bGZ1B, ho, s, t16);
         }
+#pragma unroll
+        for (int s = 0; s < 4; s++) w2bf[s] = w2_before(bIMG2, bCW2, ckW, j, s, hid0, c, h, t16);
         mma_jit<4>(gW2s, [&](int, int s) { return x2b[s]; },                                   // X2_bar^T: lane = hid
                    [&](int fb, int s) { return piece_tr<LDX>(s_a, fb, s, lane); });            // gZ2_bar: lane = F
         if (v < 2) lds_rowsum_add_jit(s_gb2 + 32 * v, [&](int s) { return piece_tr<LDX>(s_a, v, s, lane); }, ones, c, h);
@@ -861,7 +864,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
         // T1 = W2 before the step, rows [hid][F]; T2 = gW1, rows [hid][F]
 #pragma unroll
         for (int s = 0; s < 4; s++)
-          store_piece_rows<LDF>(T1, 0, s, c, h, w2_before(bIMG2, bCW2, ckW, j, s, hid0, c, h, t16));
+          store_piece_rows<LDF>(T1, 0, s, c, h, w2bf[s]);
         store_state_rows<LDF>(T2, gW1s, c, h);
         WAVE_SYNC();
         AccT<2, 2> pz;
@@ -1038,6 +1041,11 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
               uhp[i][t][jj] = (bf16)(-eta_i[i] * S.b[0][0][8 * t + jj] * d1v);
             }
         }
+        bf16x8 w1bf[2][2];   // W1^T before the step (lane = F, contraction = hid), for the product after the next fence
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+          for (int s = 0; s < 2; s++) w1bf[rb][s] = w1_before(bIMG1, bCW1, ckW, j, rb, s, hid0, c, h, t16);
         WAVE_SYNC();   // S, P2 and gW1 G1^T have consumed T2 / T1
 #pragma unroll
         for (int i = 0; i < 2; i++)
@@ -1047,8 +1055,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
             store_piece_rows<LDH>(T2, tb[i], t, c, h, uhp[i][t]);   // -eta u rows [tok][hid]
           }
         WAVE_SYNC();
-        mma_jit<2>(dk, [&](int rb, int s) {                                                    // + W1 dZ1^T, W1 before the step
-                     return w1_before(bIMG1, bCW1, ckW, j, rb, s, hid0, c, h, t16); },
+        mma_jit<2>(dk, [&](int rb, int s) { return w1bf[rb][s]; },                             // + W1 dZ1^T, W1 before the step
                    [&](int i, int s) { return dzp[i][s]; });
         mma_jit<4>(gW2s, [&](int, int s) { return piece_tr<LDH>(T2, 0, s, lane); },            // (-eta u)^T: lane = hid
                    [&](int fb, int s) { return piece_tr<LDX>(s_gz2, fb, s, lane); });          // gZ2: lane = F
