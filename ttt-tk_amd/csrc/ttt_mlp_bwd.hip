@@ -504,7 +504,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
   }
   int* const w_replayed = p.sync + (size_t)bh * BWD_SYNC_STRIDE;
   int* const w_walked = w_replayed + 16;
-  int* const w_status = p.sync + (size_t)p.B * p.NH * BWD_SYNC_STRIDE;
+  int* const w_status = p.status;
   int* const s_flag = reinterpret_cast<int*>(smem + SB_FLAG);
 
   if constexpr (ROLE == 0) {   // the replay's sum starts at zero
@@ -1136,7 +1136,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
 
 __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  bwd_body<0>(p, smem, blockIdx.x);
+  bwd_body<0>(p, smem, p.bh0 + blockIdx.x);
 }
 
 // Two workgroups per (batch, head).  Workgroups are dealt to the 8 XCDs in turn, so with a multiple
@@ -1145,13 +1145,14 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_split_kernel(const Bwd
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int b = blockIdx.x;
   int bh, role;
-  if ((p.B * p.NH) % 8 == 0) {
+  if (p.nbh % 8 == 0) {
     bh = (b >> 4) * 8 + (b & 7);
     role = (b >> 3) & 1;
   } else {
     bh = b >> 1;
     role = b & 1;
   }
+  bh += p.bh0;
   if (role == 0) bwd_body<1>(p, smem, bh);
   else bwd_body<2>(p, smem, bh);
 }
@@ -1171,14 +1172,15 @@ hipError_t ttt_mlp_bwd_enqueue(const ttt::BwdParams& p, hipStream_t stream) {
                                      hipFuncAttributeMaxDynamicSharedMemorySize, ttt::SM_BWD_BYTES);
   if (e != hipSuccess) return e;
   if (p.sync == nullptr) {
-    hipLaunchKernelGGL(ttt::ttt_mlp_bwd_kernel, dim3(p.B * p.NH), dim3(ttt::BW_THREADS), ttt::SM_BWD_BYTES, stream, p);
+    hipLaunchKernelGGL(ttt::ttt_mlp_bwd_kernel, dim3(p.nbh), dim3(ttt::BW_THREADS), ttt::SM_BWD_BYTES, stream, p);
     return hipGetLastError();
   }
   e = hipFuncSetAttribute(reinterpret_cast<const void*>(ttt::ttt_mlp_bwd_split_kernel),
                           hipFuncAttributeMaxDynamicSharedMemorySize, ttt::SM_BWD_BYTES);
   if (e != hipSuccess) return e;
-  const int n = static_cast<int>(ttt::bwd_sync_ints((long long)p.B * p.NH));
-  hipLaunchKernelGGL(ttt::ttt_mlp_zero_words, dim3((n + 255) / 256), dim3(256), 0, stream, p.sync, n);
-  hipLaunchKernelGGL(ttt::ttt_mlp_bwd_split_kernel, dim3(2 * p.B * p.NH), dim3(ttt::BW_THREADS), ttt::SM_BWD_BYTES, stream, p);
+  const int n = static_cast<int>(ttt::bwd_sync_ints(p.nbh));
+  int* const words = p.status - (size_t)p.nbh * ttt::BWD_SYNC_STRIDE;   // p.sync itself is moved back by bh0 entries
+  hipLaunchKernelGGL(ttt::ttt_mlp_zero_words, dim3((n + 255) / 256), dim3(256), 0, stream, words, n);
+  hipLaunchKernelGGL(ttt::ttt_mlp_bwd_split_kernel, dim3(2 * p.nbh), dim3(ttt::BW_THREADS), ttt::SM_BWD_BYTES, stream, p);
   return hipGetLastError();
 }

@@ -111,25 +111,43 @@ int make_bwd_params(const ttt_mlp_bwd_args* a, ttt::BwdParams& p) {
   return TTT_MLP_OK;
 }
 
-// Two workgroups per (batch, head) wait for each other, so all of them must be resident at once:
-// one workgroup fills a CU (LDS), hence the grid may not exceed the CUs of the current device.
-bool two_workgroup_mode_fits(long long BH) {
+// Two workgroups per (batch, head) wait for each other, so all of them must be resident at once: one
+// workgroup fills a CU (LDS), hence such a launch may not exceed the CUs of the current device.  The
+// (batch, head) pairs are therefore covered by two launches in a row: as many full rounds of one
+// workgroup per pair as there are (a multiple of the CU count), then the rest - with two workgroups per
+// pair if that fits the device (split), otherwise with one.
+struct LaunchPlan {
+  long long n_single = 0;   // pairs 0 .. n_single-1: one workgroup each
+  long long n_rest = 0;     // pairs n_single .. n_single+n_rest-1
+  bool rest_split = false;
+};
+// `after_full_rounds`: whether the rest may be split when full rounds precede it.  That pays for the
+// backward; the forward's gain from splitting is smaller than what a full device costs it (measured).
+LaunchPlan plan_launches(long long BH, bool after_full_rounds) {
+  LaunchPlan pl;
   int dev = 0, cus = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return false;
-  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return false;
-  return BH > 0 && 2 * BH <= cus;
+  if (BH <= 0 || hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+    pl.n_single = BH > 0 ? BH : 0;
+    return pl;
+  }
+  pl.n_single = BH / cus * cus;
+  pl.n_rest = BH - pl.n_single;
+  pl.rest_split = pl.n_rest > 0 && 2 * pl.n_rest <= cus && (after_full_rounds || pl.n_single == 0);
+  if (!pl.rest_split) { pl.n_single = BH; pl.n_rest = 0; }
+  return pl;
 }
 
-// Workspace of the two-workgroup mode: the synchronisation words, the replaying workgroups' share of the
-// norm gradients, then the alternate set of the ten per-group tensors that carry a replayed group to the
-// reverse walk; each part 256-byte aligned.
+// Workspace of the backward's two-workgroup mode for n (batch, head) pairs: the synchronisation words,
+// the replaying workgroups' share of the norm gradients, then the alternate set of the ten per-group
+// tensors that carry a replayed group to the reverse walk; each part 256-byte aligned.
 struct BwdWorkspace {
   size_t off[11];
   size_t total;
-  BwdWorkspace(long long BH, long long cgs) {
-    const size_t slot = (size_t)BH * (size_t)cgs;
+  BwdWorkspace(long long n, long long cgs) {
+    const size_t slot = (size_t)n * (size_t)cgs;
     const size_t tile = TTT_MLP_CS * TTT_MLP_F * 2, img = TTT_MLP_CS * TTT_MLP_HID * 2, vec = TTT_MLP_CS * 4;
-    const size_t bytes[11] = {ttt::bwd_sync_ints(BH) * sizeof(int), (size_t)BH * 8 * 2 * TTT_MLP_F * sizeof(float),
+    const size_t bytes[11] = {ttt::bwd_sync_ints(n) * sizeof(int), (size_t)n * 8 * 2 * TTT_MLP_F * sizeof(float),
                               slot * img, slot * img, slot * img, slot * img, slot * tile, slot * img, slot * tile,
                               slot * tile + slot * tile, slot * vec};
     size_t o = 0;
@@ -138,86 +156,116 @@ struct BwdWorkspace {
   }
 };
 
-}  // namespace
-
-extern "C" int ttt_mlp_bwd_launch(const ttt_mlp_bwd_args* a, void* stream) {
-  ttt::BwdParams p;
-  if (int rc = make_bwd_params(a, p)) return rc;
-  return static_cast<int>(ttt_mlp_bwd_enqueue(p, static_cast<hipStream_t>(stream)));
-}
-
-extern "C" size_t ttt_mlp_bwd_workspace_bytes(int B, int NH, int checkpoint_group_size) {
-  if (B <= 0 || NH <= 0 || checkpoint_group_size <= 0 || checkpoint_group_size > (1 << 16)) return 0;
-  if (!two_workgroup_mode_fits((long long)B * NH)) return 0;
-  return BwdWorkspace((long long)B * NH, checkpoint_group_size).total;
-}
-
-extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* workspace, size_t workspace_bytes, void* stream) {
-  ttt::BwdParams p;
-  if (int rc = make_bwd_params(a, p)) return rc;
-  if (workspace == nullptr) return TTT_MLP_ERR_BAD_ARG;
-  if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return TTT_MLP_ERR_ALIGN;
-  if (!two_workgroup_mode_fits((long long)p.B * p.NH)) return TTT_MLP_ERR_NO_ROOM;
-  const BwdWorkspace w((long long)p.B * p.NH, p.cgs);
-  if (workspace_bytes < w.total) return TTT_MLP_ERR_WORKSPACE;
-  char* base = static_cast<char*>(workspace);
-  const size_t slot_elems = (size_t)p.B * p.NH * p.cgs * (TTT_MLP_CS * TTT_MLP_F);   // one [B,NH,cgs,CS,F] tensor
-  p.sync = reinterpret_cast<int*>(base + w.off[0]);
-  p.norm_partial = reinterpret_cast<float*>(base + w.off[1]);
-  p.alt_X2_group = reinterpret_cast<__bf16*>(base + w.off[2]);
-  p.alt_Z1_group = reinterpret_cast<__bf16*>(base + w.off[3]);
-  p.alt_Z1_bar_group = reinterpret_cast<__bf16*>(base + w.off[4]);
-  p.alt_X2_bar_group = reinterpret_cast<__bf16*>(base + w.off[5]);
-  p.alt_grad_l_wrt_Z2_group = reinterpret_cast<__bf16*>(base + w.off[6]);
-  p.alt_grad_l_wrt_Z1_group = reinterpret_cast<__bf16*>(base + w.off[7]);
-  p.alt_x_hat_fused_group = reinterpret_cast<__bf16*>(base + w.off[8]);
-  p.alt_grad_x_hat_fused_group = reinterpret_cast<__bf16*>(base + w.off[9]);
-  p.alt_grad_output_fused_group = p.alt_grad_x_hat_fused_group + slot_elems;
-  p.alt_std_fused_group = reinterpret_cast<float*>(base + w.off[10]);
-  return static_cast<int>(ttt_mlp_bwd_enqueue(p, static_cast<hipStream_t>(stream)));
-}
-
 // Workspace of the forward's two-workgroup mode: synchronisation words, then per (batch, head) a ring of
 // 2 * FWD_RING slots of state images and of bias vectors.
-namespace {
 struct FwdWorkspace {
   size_t off[3];
   size_t total;
-  explicit FwdWorkspace(long long BH) {
-    const size_t slots = (size_t)BH * 2 * ttt::FWD_RING;
-    const size_t bytes[3] = {ttt::bwd_sync_ints(BH) * sizeof(int), slots * ttt::FWD_IMG_BYTES,
+  explicit FwdWorkspace(long long n) {
+    const size_t slots = (size_t)n * 2 * ttt::FWD_RING;
+    const size_t bytes[3] = {ttt::bwd_sync_ints(n) * sizeof(int), slots * ttt::FWD_IMG_BYTES,
                              slots * ttt::FWD_BIAS_FLOATS * sizeof(float)};
     size_t o = 0;
     for (int i = 0; i < 3; i++) { off[i] = o; o += (bytes[i] + 255) & ~(size_t)255; }
     total = o;
   }
 };
+
+int check_workspace(const void* workspace) {
+  if (workspace == nullptr) return TTT_MLP_ERR_BAD_ARG;
+  if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return TTT_MLP_ERR_ALIGN;
+  return TTT_MLP_OK;
+}
+
 }  // namespace
+
+extern "C" int ttt_mlp_bwd_launch(const ttt_mlp_bwd_args* a, void* stream) {
+  ttt::BwdParams p;
+  if (int rc = make_bwd_params(a, p)) return rc;
+  p.bh0 = 0;
+  p.nbh = p.B * p.NH;
+  return static_cast<int>(ttt_mlp_bwd_enqueue(p, static_cast<hipStream_t>(stream)));
+}
+
+extern "C" size_t ttt_mlp_bwd_workspace_bytes(int B, int NH, int checkpoint_group_size) {
+  if (B <= 0 || NH <= 0 || checkpoint_group_size <= 0 || checkpoint_group_size > (1 << 16)) return 0;
+  const LaunchPlan pl = plan_launches((long long)B * NH, true);
+  return pl.rest_split ? BwdWorkspace(pl.n_rest, checkpoint_group_size).total : 0;
+}
+
+extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* workspace, size_t workspace_bytes, void* stream) {
+  ttt::BwdParams p;
+  if (int rc = make_bwd_params(a, p)) return rc;
+  if (int rc = check_workspace(workspace)) return rc;
+  const LaunchPlan pl = plan_launches((long long)p.B * p.NH, true);
+  if (!pl.rest_split) return TTT_MLP_ERR_NO_ROOM;
+  const BwdWorkspace w(pl.n_rest, p.cgs);
+  if (workspace_bytes < w.total) return TTT_MLP_ERR_WORKSPACE;
+  if (pl.n_single > 0) {
+    p.bh0 = 0;
+    p.nbh = static_cast<int>(pl.n_single);
+    if (hipError_t e = ttt_mlp_bwd_enqueue(p, static_cast<hipStream_t>(stream))) return static_cast<int>(e);
+  }
+  // The kernels index the workspace by the global pair number: every pointer is moved back by bh0 entries.
+  char* base = static_cast<char*>(workspace);
+  const size_t b0 = (size_t)pl.n_single;
+  const size_t slot_elems = (size_t)pl.n_rest * p.cgs * (TTT_MLP_CS * TTT_MLP_F);   // one [n_rest,cgs,CS,F] tensor
+  const size_t tile = (size_t)p.cgs * TTT_MLP_CS * TTT_MLP_F, img = (size_t)p.cgs * TTT_MLP_CS * TTT_MLP_HID, vec = (size_t)p.cgs * TTT_MLP_CS;
+  p.bh0 = static_cast<int>(pl.n_single);
+  p.nbh = static_cast<int>(pl.n_rest);
+  int* words = reinterpret_cast<int*>(base + w.off[0]);
+  p.status = words + (size_t)pl.n_rest * ttt::BWD_SYNC_STRIDE;
+  p.sync = words - b0 * ttt::BWD_SYNC_STRIDE;
+  p.norm_partial = reinterpret_cast<float*>(base + w.off[1]) - b0 * (8 * 2 * TTT_MLP_F);
+  p.alt_X2_group = reinterpret_cast<__bf16*>(base + w.off[2]) - b0 * img;
+  p.alt_Z1_group = reinterpret_cast<__bf16*>(base + w.off[3]) - b0 * img;
+  p.alt_Z1_bar_group = reinterpret_cast<__bf16*>(base + w.off[4]) - b0 * img;
+  p.alt_X2_bar_group = reinterpret_cast<__bf16*>(base + w.off[5]) - b0 * img;
+  p.alt_grad_l_wrt_Z2_group = reinterpret_cast<__bf16*>(base + w.off[6]) - b0 * tile;
+  p.alt_grad_l_wrt_Z1_group = reinterpret_cast<__bf16*>(base + w.off[7]) - b0 * img;
+  p.alt_x_hat_fused_group = reinterpret_cast<__bf16*>(base + w.off[8]) - b0 * tile;
+  p.alt_grad_x_hat_fused_group = reinterpret_cast<__bf16*>(base + w.off[9]) - b0 * tile;
+  p.alt_grad_output_fused_group = reinterpret_cast<__bf16*>(base + w.off[9]) + slot_elems - b0 * tile;
+  p.alt_std_fused_group = reinterpret_cast<float*>(base + w.off[10]) - b0 * vec;
+  return static_cast<int>(ttt_mlp_bwd_enqueue(p, static_cast<hipStream_t>(stream)));
+}
 
 extern "C" int ttt_mlp_fwd_launch(const ttt_mlp_fwd_args* a, void* stream) {
   ttt::FwdParams p;
   if (int rc = make_fwd_params(a, p)) return rc;
+  p.bh0 = 0;
+  p.nbh = p.B * p.NH;
   return static_cast<int>(ttt_mlp_fwd_enqueue(p, static_cast<hipStream_t>(stream)));
 }
 
 extern "C" size_t ttt_mlp_fwd_workspace_bytes(int B, int NH) {
   if (B <= 0 || NH <= 0) return 0;
-  if (!two_workgroup_mode_fits((long long)B * NH)) return 0;
-  return FwdWorkspace((long long)B * NH).total;
+  const LaunchPlan pl = plan_launches((long long)B * NH, false);
+  return pl.rest_split ? FwdWorkspace(pl.n_rest).total : 0;
 }
 
 extern "C" int ttt_mlp_fwd_launch_overlapped(const ttt_mlp_fwd_args* a, void* workspace, size_t workspace_bytes, void* stream) {
   ttt::FwdParams p;
   if (int rc = make_fwd_params(a, p)) return rc;
-  if (workspace == nullptr) return TTT_MLP_ERR_BAD_ARG;
-  if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return TTT_MLP_ERR_ALIGN;
-  if (!two_workgroup_mode_fits((long long)p.B * p.NH)) return TTT_MLP_ERR_NO_ROOM;
-  const FwdWorkspace w((long long)p.B * p.NH);
+  if (int rc = check_workspace(workspace)) return rc;
+  const LaunchPlan pl = plan_launches((long long)p.B * p.NH, false);
+  if (!pl.rest_split) return TTT_MLP_ERR_NO_ROOM;
+  const FwdWorkspace w(pl.n_rest);
   if (workspace_bytes < w.total) return TTT_MLP_ERR_WORKSPACE;
+  if (pl.n_single > 0) {
+    p.bh0 = 0;
+    p.nbh = static_cast<int>(pl.n_single);
+    if (hipError_t e = ttt_mlp_fwd_enqueue(p, static_cast<hipStream_t>(stream))) return static_cast<int>(e);
+  }
   char* base = static_cast<char*>(workspace);
-  p.sync = reinterpret_cast<int*>(base + w.off[0]);
-  p.state_img = reinterpret_cast<__bf16*>(base + w.off[1]);
-  p.bias_img = reinterpret_cast<float*>(base + w.off[2]);
+  const size_t b0 = (size_t)pl.n_single;
+  p.bh0 = static_cast<int>(pl.n_single);
+  p.nbh = static_cast<int>(pl.n_rest);
+  int* words = reinterpret_cast<int*>(base + w.off[0]);
+  p.status = words + (size_t)pl.n_rest * ttt::BWD_SYNC_STRIDE;
+  p.sync = words - b0 * ttt::BWD_SYNC_STRIDE;
+  p.state_img = reinterpret_cast<__bf16*>(base + w.off[1]) - b0 * 2 * ttt::FWD_RING * (ttt::FWD_IMG_BYTES / 2);
+  p.bias_img = reinterpret_cast<float*>(base + w.off[2]) - b0 * 2 * ttt::FWD_RING * ttt::FWD_BIAS_FLOATS;
   return static_cast<int>(ttt_mlp_fwd_enqueue(p, static_cast<hipStream_t>(stream)));
 }
 

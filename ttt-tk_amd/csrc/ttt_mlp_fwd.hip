@@ -221,7 +221,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
 
   int* const w_given = p.sync + (size_t)bh * BWD_SYNC_STRIDE;   // groups handed to the output branch
   int* const w_taken = w_given + 16;                             // groups it has finished
-  int* const w_status = p.sync + (size_t)p.B * p.NH * BWD_SYNC_STRIDE;
+  int* const w_status = p.status;
   int* const s_flag = reinterpret_cast<int*>(smem + SM_FLAG);
 
   for (int mb = 0; mb < p.NC; mb++) {
@@ -508,7 +508,7 @@ TTT_DEV void fwd_output_branch(const FwdParams& p, unsigned char* smem, const in
   const gptr_t gXQ = gbuf(p.XQ + x_base), gOut = gbuf(p.Out + x_base);
   int* const w_given = p.sync + (size_t)bh * BWD_SYNC_STRIDE;
   int* const w_taken = w_given + 16;
-  int* const w_status = p.sync + (size_t)p.B * p.NH * BWD_SYNC_STRIDE;
+  int* const w_status = p.status;
   int* const s_flag = reinterpret_cast<int*>(smem + SM_FLAG);
 
   for (int mb = 0; mb < p.NC; mb++) {
@@ -574,7 +574,7 @@ TTT_DEV void fwd_output_branch(const FwdParams& p, unsigned char* smem, const in
 
 __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  fwd_body<0>(p, smem, blockIdx.x);
+  fwd_body<0>(p, smem, p.bh0 + blockIdx.x);
 }
 
 // Two workgroups per (batch, head), placed like those of the backward (same XCD where the count allows).
@@ -582,13 +582,14 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_split_kernel(const Fwd
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int b = blockIdx.x;
   int bh, role;
-  if ((p.B * p.NH) % 8 == 0) {
+  if (p.nbh % 8 == 0) {
     bh = (b >> 4) * 8 + (b & 7);
     role = (b >> 3) & 1;
   } else {
     bh = b >> 1;
     role = b & 1;
   }
+  bh += p.bh0;
   if (role == 0) fwd_body<1>(p, smem, bh);
   else fwd_output_branch(p, smem, bh);
 }
@@ -609,14 +610,15 @@ hipError_t ttt_mlp_fwd_enqueue(const ttt::FwdParams& p, hipStream_t stream) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(ttt::ttt_mlp_fwd_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, ttt::SM_FWD_BYTES);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(ttt::ttt_mlp_fwd_kernel, dim3(p.B * p.NH), dim3(ttt::FW_THREADS), ttt::SM_FWD_BYTES, stream, p);
+    hipLaunchKernelGGL(ttt::ttt_mlp_fwd_kernel, dim3(p.nbh), dim3(ttt::FW_THREADS), ttt::SM_FWD_BYTES, stream, p);
     return hipGetLastError();
   }
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(ttt::ttt_mlp_fwd_split_kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, ttt::SM_FWD_BYTES);
   if (e != hipSuccess) return e;
-  const int n = static_cast<int>(ttt::bwd_sync_ints((long long)p.B * p.NH));
-  hipLaunchKernelGGL(ttt::ttt_mlp_fwd_zero_words, dim3((n + 255) / 256), dim3(256), 0, stream, p.sync, n);
-  hipLaunchKernelGGL(ttt::ttt_mlp_fwd_split_kernel, dim3(2 * p.B * p.NH), dim3(ttt::FW_THREADS), ttt::SM_FWD_BYTES, stream, p);
+  const int n = static_cast<int>(ttt::bwd_sync_ints(p.nbh));
+  int* const words = p.status - (size_t)p.nbh * ttt::BWD_SYNC_STRIDE;   // p.sync itself is moved back by bh0 entries
+  hipLaunchKernelGGL(ttt::ttt_mlp_fwd_zero_words, dim3((n + 255) / 256), dim3(256), 0, stream, words, n);
+  hipLaunchKernelGGL(ttt::ttt_mlp_fwd_split_kernel, dim3(2 * p.nbh), dim3(ttt::FW_THREADS), ttt::SM_FWD_BYTES, stream, p);
   return hipGetLastError();
 }

@@ -15,9 +15,13 @@ struct FwdParams {
   // Two-workgroup mode only (sync != nullptr): per (batch, head) a ring of 2 * FWD_RING mini-batch slots
   // with the bf16 operand images (64 KiB) and the bias vectors (256 + 64 floats) of the state after a
   // mini-batch, and the words the two workgroups signal with (layout as in the backward).
+  // The workspace pointers are indexed by the global (batch, head) number like everything else: the
+  // launcher passes them moved back by bh0 entries.
   __bf16* state_img;
   float* bias_img;
   int* sync;
+  int* status;    // the status word behind the synchronisation words
+  int bh0, nbh;   // this launch covers (batch, head) pairs bh0 .. bh0 + nbh - 1
 };
 constexpr int FWD_RING = 8;                    // mini-batches per hand-over
 constexpr int FWD_IMG_BYTES = 64 * 256 * 2 * 2;  // W1 and W2 as bf16 operands
@@ -48,6 +52,8 @@ struct BwdParams {
   float* alt_std_fused_group;
   float* norm_partial;   // [B*NH][8 waves][2][64]: the replaying workgroup's share of the norm-weight / norm-bias gradients
   int* sync;
+  int* status;    // the status word behind the synchronisation words
+  int bh0, nbh;   // this launch covers (batch, head) pairs bh0 .. bh0 + nbh - 1 (workspace pointers moved back by bh0 entries)
 };
 
 // Layout of `sync` (ints): 32 per (batch, head) - word 0 counts the groups replayed (norm_partial is
