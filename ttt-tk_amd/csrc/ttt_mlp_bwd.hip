@@ -5,8 +5,9 @@
 // group, last to first, the forward is replayed from the checkpoint while the per-mini-batch
 // activations are saved, then the group is walked backwards producing the ten output gradients.
 //
-// Mapping: one workgroup of 8 wavefronts (two per SIMD, at most 256 registers each) per (batch,
-// head); wave v owns hidden columns [32v, 32v+32).  All [tokens x hidden] activations live in
+// Mapping: workgroups of 8 wavefronts (two per SIMD, at most 256 registers each); one per (batch,
+// head), or two where the device has CUs to spare - then one replays the checkpoint groups and the
+// other walks them backwards, a group behind.  Wave v owns hidden columns [32v, 32v+32).  All [tokens x hidden] activations live in
 // registers in the "Q" orientation (accumulator rows = hidden, lane = token), so per-token scalars
 // (eta, dEta partial sums) are per-lane values.  An activation that is also needed with tokens as the
 // contraction index is bounced once through a wave-private LDS tile (row store + transposing read).
@@ -23,11 +24,16 @@
 //            stores the operand images of W1^T[shard] and W2[shard]^T, and the walk reads the image of
 //            the state after and before the step (before the first step of a group: converted straight
 //            from the fp32 checkpoint).
-// While a group is replayed the running gradients are parked in the caller's W*_init_group scratch.
-// Saved per mini-batch (caller's *_group scratch): Z1 and Z1_bar as bf16 register images (Z1_group,
-// Z1_bar_group); the two weight operand images (X2_group: W1^T[shard], grad_l_wrt_Z1_group:
-// W2[shard]^T); x_hat / grad_output of the fused LayerNorm loss, dl/dZ2 and the output LayerNorm's
-// x_hat as bf16 [tok][F] tiles; the two std vectors in fp32.
+// The output branch (Out depends on the state after a step, nothing later depends on it) is taken
+// backwards inside the replay, where that state is still in registers: the replay writes dXQ and
+// leaves dL/dZ2_bar and the operands X2_bar^T, (dL/dZ1_bar)^T, so that the walk only accumulates their
+// products into the running gradients.
+// While a group is replayed by the workgroup that also walks, the running gradients are parked in the
+// caller's W*_init_group scratch.
+// Saved per mini-batch (caller's *_group scratch): Z1 as a bf16 register image (Z1_group); the operand
+// images X2_bar^T (X2_bar_group) and (dL/dZ1_bar)^T (Z1_bar_group); the two weight operand images
+// (X2_group: W1^T[shard], grad_l_wrt_Z1_group: W2[shard]^T); x_hat / grad_output of the fused LayerNorm
+// loss, dl/dZ2 and dL/dZ2_bar (grad_x_hat_fused_group) as bf16 [tok][F] tiles; the fused std in fp32.
 #include "ttt_mlp_common.hpp"
 #include "ttt_mlp_kernels.hpp"
 

@@ -5,8 +5,9 @@
 // (W1,b1,W2,b2) is carried through NC mini-batches of 64 tokens; before mini-batch i with
 // i % checkpoint_group_size == 0 the state is stored at checkpoint slot i / checkpoint_group_size.
 //
-// Mapping: one workgroup of 8 wavefronts (two per SIMD, at most 256 registers each) per (batch,
-// head); wave v owns hidden columns [32v, 32v+32).  The state lives in registers for the whole scan
+// Mapping: workgroups of 8 wavefronts (two per SIMD, at most 256 registers each); one per (batch,
+// head), or two where the device has CUs to spare - then one carries the state and the other computes
+// Out from the states it leaves behind.  Wave v owns hidden columns [32v, 32v+32).  The state lives in registers for the whole scan
 // as MFMA accumulator tiles:
 //   W1s = W1[:, shard]      (rows F,   columns hid)  -> chained operand of XK*W1 and of (XQ*W1)^T
 //   W2s = W2[shard, :]      (rows hid, columns F)    -> chained operand of (X2*W2)^T
