@@ -1,0 +1,72 @@
+"""The two-workgroup launchers called directly through the C ABI (ctypes): shapes the operator module never
+routes there (a single mini-batch, a single checkpoint group), the status word, and the error codes."""
+import ctypes
+import os
+
+import pytest
+import torch
+
+from oracle import ttt_mlp_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "ttt-tk_amd", "libttt_mlp.so")
+FWD_KEYS = ("XQ", "XK", "XV", "last_eta", "ttt_norm_weight", "ttt_norm_bias", "W1", "b1", "W2", "b2")
+UP_KEYS = ("grad_L_W1_last", "grad_L_b1_last", "grad_L_W2_last", "grad_L_b2_last", "grad_L_XQW_mini_batch")
+SIZES = ("checkpoint_group_size", "B", "NH", "NC", "K")
+
+
+def _lib():
+    lib = ctypes.CDLL(LIB)
+    lib.ttt_mlp_fwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.ttt_mlp_bwd_workspace_bytes.restype = ctypes.c_size_t
+    return lib
+
+
+def _args(order, t, cgs, B, NH, NC, K):
+    class Args(ctypes.Structure):
+        _fields_ = [(n, ctypes.c_void_p) for n in order] + [(n, ctypes.c_int32) for n in SIZES]
+    return Args(*[t[k].data_ptr() for k in order], cgs, B, NH, NC, K)
+
+
+@pytest.mark.parametrize("B,NH,NC,cgs", [(1, 2, 1, 1), (1, 3, 5, 8), (2, 2, 17, 4)])
+def test_overlapped_launchers_through_ctypes(B, NH, NC, cgs):
+    print(f"case B={B} NH={NH} NC={NC} cgs={cgs}", flush=True)
+    import ttt_mlp_host as host
+    lib = _lib()
+    dev = torch.device("cuda:0")
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    K = host.num_checkpoints(NC, cgs)
+    d = orc.make_inputs(B, NH, NC, seed=31)
+    results = []
+    for overlapped in (False, True):
+        t = {k: d[k].to(dev).contiguous() for k in FWD_KEYS + UP_KEYS}
+        t.update(host.alloc_forward_buffers(B, NH, NC, cgs, dev))
+        t.update(host.alloc_backward_buffers(B, NH, NC, cgs, dev))
+        fa = _args(host.FWD_ORDER, t, cgs, B, NH, NC, K)
+        ba = _args(host.BWD_ORDER, t, cgs, B, NH, NC, K)
+        if not overlapped:
+            assert lib.ttt_mlp_fwd_launch(ctypes.byref(fa), stream) == 0
+            assert lib.ttt_mlp_bwd_launch(ctypes.byref(ba), stream) == 0
+        else:
+            for which, a in (("fwd", fa), ("bwd", ba)):
+                nbytes = (lib.ttt_mlp_fwd_workspace_bytes(B, NH) if which == "fwd"
+                          else lib.ttt_mlp_bwd_workspace_bytes(B, NH, cgs))
+                assert nbytes > 0 and nbytes % 256 == 0
+                ws = torch.full((nbytes + 256,), 0xA5, dtype=torch.uint8, device=dev)
+                base = (ws.data_ptr() + 255) // 256 * 256
+                launch = getattr(lib, f"ttt_mlp_{which}_launch_overlapped")
+                # too small / misaligned / missing workspace are refused before anything is enqueued
+                assert launch(ctypes.byref(a), ctypes.c_void_p(base), ctypes.c_size_t(nbytes - 1), stream) == 1006
+                assert launch(ctypes.byref(a), ctypes.c_void_p(base + 16), ctypes.c_size_t(nbytes), stream) == 1003
+                assert launch(ctypes.byref(a), None, ctypes.c_size_t(nbytes), stream) == 1001
+                assert launch(ctypes.byref(a), ctypes.c_void_p(base), ctypes.c_size_t(nbytes), stream) == 0
+                torch.cuda.synchronize()
+                status = ws[base - ws.data_ptr():].view(torch.int32)[B * NH * 32].item()
+                assert status == 0, "a workgroup gave up waiting for the other"
+        torch.cuda.synchronize()
+        results.append({k: t[k].float().cpu() for k in ("Out", "W1_checkpoints", "b2_checkpoints") + host.GRAD_NAMES})
+    for k in results[0]:
+        assert torch.isfinite(results[1][k]).all(), k
+        assert torch.equal(results[0][k], results[1][k]), k
