@@ -147,12 +147,13 @@ def test_bit_reproducible_and_independent_of_workspace_contents(B, NH, NC, cgs):
 
 
 @pytest.mark.parametrize("B,NH,NC,cgs", [
-    (1, 2, 4, 1),        # four groups of one mini-batch: the two sets alternate, the replay waits for the walk
+    (1, 2, 9, 1),        # nine groups of one mini-batch: the sets are reused, the replays wait for the walk
     (2, 3, 9, 4),        # ragged last group (walked first), (batch, head) count not a multiple of 8
     (1, 8, 24, 8),       # multiple of 8: the two workgroups of a pair are placed on one XCD
     (2, 8, 10, 5),       # two groups only
     (1, 4, 33, 2),       # seventeen groups
-    (2, 130, 5, 2),      # more pairs than CUs: 256 with one workgroup each, then the last 4 with two
+    (2, 130, 5, 2),      # more pairs than CUs: 256 with one workgroup each, then the last 4 with three
+    (1, 96, 5, 2),       # too many pairs for three workgroups each: one replays all groups, one walks
 ])
 def test_overlapped_backward_is_bit_identical(B, NH, NC, cgs):
     """Recomputing the groups on a second workgroup changes the schedule, not one bit of the results."""

@@ -382,9 +382,10 @@ TTT_DEV bf16x8 w1_before(gptr_t img, gptr_t ck, unsigned ck_off, int j, int rb, 
 // counters in HBM (agent scope); both are resident at once because the launcher uses this mode only
 // when the grid fits the CUs of the device.  A wait that sees no progress for SPIN_LIMIT ticks of the
 // 100 MHz clock raises the status word and both workgroups leave, so every wave always exits.
-// ROLE 0: replay and reverse walk of every group in one workgroup; 1: the replays only; 2: the reverse walks only.
+// ROLE 0: replay and reverse walk of every group in one workgroup; 1: replays only - every n_replay-th group,
+// starting with group number `turn` (counted from the end of the sequence); 2: the reverse walks only.
 template <int ROLE>
-TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
+TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, const int turn) {
   bf16* s_xq = reinterpret_cast<bf16*>(smem + SB_XQ);
   bf16* s_xk = reinterpret_cast<bf16*>(smem + SB_XK);
   bf16* s_gz2 = reinterpret_cast<bf16*>(smem + SB_GZ2);
@@ -458,7 +459,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
   KernArgs ka = (KernArgs)__builtin_amdgcn_kernarg_segment_ptr();
 #define REFRESH_OFFSETS() asm volatile("" : "+s"(ka), "+s"(ox), "+s"(oe), "+s"(of), "+s"(oh), "+s"(ot), "+s"(opk), "+s"(ock))
   // per-group tensors: the caller's (set 0) or, in two-workgroup mode, the alternate set
-#define GRP(name) (set ? ka->alt_##name : ka->name)
+#define GRP(name) (set ? ka->alt_##name[set - 1] : ka->name)
 #define bXQ gbuf(ka->XQ + ox)
 #define bXK gbuf(ka->XK + ox)
 #define bXV gbuf(ka->XV + ox)
@@ -473,7 +474,6 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
 #define bXHF gbuf(GRP(x_hat_fused_group) + of)
 #define bGOF gbuf(GRP(grad_output_fused_group) + of)
 #define bGZ2 gbuf(GRP(grad_l_wrt_Z2_group) + of)
-#define bNP gbuf(ka->x_hat_ln_group + of)                // one workgroup per (batch, head): park of norm-gradient sums
 #define bSDF gbuf(GRP(std_fused_group) + ot)
   // While a group is replayed the running gradients are parked in W*_init_group; during the reverse
   // walk the same two 64 KiB slots park what must survive the LayerNorm stage (three 32 KiB images).
@@ -508,44 +508,61 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
     acc_load_rows(gW1s, gbuf(p.grad_L_W1_last + (size_t)bh * FD * HID), 0, HID, 0, hid0, c, h);
     acc_load_rows(gW2s, gbuf(p.grad_L_W2_last + (size_t)bh * HID * FD), 0, FD, hid0, 0, c, h);
   }
-  int* const w_replayed = p.sync + (size_t)bh * BWD_SYNC_STRIDE;
-  int* const w_walked = w_replayed + 16;
+  int* const w_sync = p.sync + (size_t)bh * BWD_SYNC_STRIDE;   // + 0, + 8: groups replayed by workgroup 0 / 1
+  int* const w_walked = w_sync + 16;
+  const int n_replay = ROLE == 0 ? 1 : p.n_replay, n_sets = 2 * n_replay;
   int* const w_status = p.status;
   int* const s_flag = reinterpret_cast<int*>(smem + SB_FLAG);
 
-  if constexpr (ROLE == 0) {   // the replay's sum starts at zero
-    g_stf(bNP, np_off, 0, 0.f);
-    g_stf(bNP, np_off, FD * 4, 0.f);
+  // The replay's share of the norm gradients is kept as two sums, of the even and of the odd groups (counted
+  // from the end of the sequence), whoever replays them; the walk's share is a third.  A workgroup that adds
+  // to more than one of them keeps the others parked in HBM, 4 KiB each: one workgroup per (batch, head) in
+  // two slots of the caller's x_hat_ln_group, a single replaying workgroup in the workspace.
+  const gptr_t gPark = ROLE == 0 ? gbuf(p.x_hat_ln_group + (size_t)bh * cgs * (CS * FD))
+                                 : gbuf(p.norm_park + (size_t)bh * (BW_NWAVE * 2 * FD));
+  constexpr unsigned PARK_BYTES = BW_NWAVE * 2 * FD * 4;
+  if (ROLE == 0 || (ROLE == 1 && n_replay == 1)) {   // parked sums start at zero
+    g_stf(gPark, np_off, 0, 0.f);
+    g_stf(gPark, np_off, FD * 4, 0.f);
+    if constexpr (ROLE == 0) {
+      g_stf(gPark, np_off, PARK_BYTES, 0.f);
+      g_stf(gPark, np_off, PARK_BYTES + FD * 4, 0.f);
+    }
   }
-  // Exchanges the wave's LDS accumulators with the parked sum (every lane owns two words of both).
-  auto norm_swap = [&]() {
+  // Exchanges the wave's LDS accumulators with a parked sum (every lane owns two words of both).
+  auto norm_swap = [&](unsigned slot) {
     WAVE_SYNC();
     const float a0 = s_dgw[lane], a1 = s_dbw[lane];
-    const float p0 = g_ldf(bNP, np_off, 0), p1 = g_ldf(bNP, np_off, FD * 4);
+    const float p0 = g_ldf(gPark, np_off, slot * PARK_BYTES), p1 = g_ldf(gPark, np_off, slot * PARK_BYTES + FD * 4);
     s_dgw[lane] = p0;
     s_dbw[lane] = p1;
-    g_stf(bNP, np_off, 0, a0);
-    g_stf(bNP, np_off, FD * 4, a1);
+    g_stf(gPark, np_off, slot * PARK_BYTES, a0);
+    g_stf(gPark, np_off, slot * PARK_BYTES + FD * 4, a1);
     WAVE_SYNC();
   };
 
   for (int k = p.K - 1; k >= 0; k--) {
     const int n_mb = min(cgs, p.NC - k * cgs);
-    const int done = p.K - 1 - k;                    // groups already handled by this workgroup
-    const int set = ROLE == 0 ? 0 : (done & 1);
+    const int done = p.K - 1 - k;                    // number of this group, counted from the end of the sequence
+    if (ROLE == 1 && done % n_replay != turn) continue;
+    const int set = ROLE == 0 ? 0 : done % n_sets;
+    int* const w_replayed = w_sync + 8 * (done % n_replay);
     REFRESH_OFFSETS();
     const size_t slot = (size_t)bh * p.K + k;
     const unsigned ckW = k * (FD * HID * 4);   // byte offset of this group's checkpoint in bCW1 / bCW2
     // ================================================================= replay
     if constexpr (ROLE != 2) {
-      if constexpr (ROLE == 1) {   // the set is free once the reverse walk is done with the group before last
-        if (done >= 2 && !wait_at_least(w_walked, done - 1, w_status, s_flag)) return;
+      if constexpr (ROLE == 1) {   // the set is free once the reverse walk is done with the group that used it last
+        if (done >= n_sets && !wait_at_least(w_walked, done - n_sets + 1, w_status, s_flag)) return;
+        // a single replaying workgroup adds to the sum of this group's parity: the groups alternate, so from
+        // the second group on the live sum and the parked one change places
+        if (n_replay == 1 && done > 0) norm_swap(0);
       }
       // park the running gradients while the forward state needs the registers
       if constexpr (ROLE == 0) {
         acc_store_rows(gW1s, bPW1, 0, HID, 0, hid0, c, h);
         acc_store_rows(gW2s, bPW2, 0, FD, hid0, 0, c, h);
-        norm_swap();
+        norm_swap(done & 1);   // the walk's sum out, the replay's sum of this parity in
       }
       AccT<2, 1> W1s, W2t;
       AccT<1, 2> W2s;
@@ -791,20 +808,25 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
         }
       }
       if constexpr (ROLE == 1) {
-        if (k == 0) {   // hand this workgroup's norm-gradient sums to the one that writes the result
+        if (done + n_replay >= p.K) {   // this workgroup's last group: hand its norm-gradient sums to the walk
           WAVE_SYNC();
-          float* np = p.norm_partial + (size_t)bh * (BW_NWAVE * 2 * FD) + v * 2 * FD;
+          float* np = p.norm_partial + ((size_t)bh * 2 + (done & 1)) * (BW_NWAVE * 2 * FD) + v * 2 * FD;
           np[lane] = s_dgw[lane];
           np[FD + lane] = s_dbw[lane];
+          if (n_replay == 1) {   // and the sum of the other parity (zero if there was one group only)
+            float* no = p.norm_partial + ((size_t)bh * 2 + (1 - (done & 1))) * (BW_NWAVE * 2 * FD) + v * 2 * FD;
+            no[lane] = g_ldf(gPark, np_off, 0);
+            no[FD + lane] = g_ldf(gPark, np_off, FD * 4);
+          }
         }
       }
       // running gradients back into registers
       if constexpr (ROLE == 0) {
         acc_load_rows(gW1s, bPW1, 0, HID, 0, hid0, c, h);
         acc_load_rows(gW2s, bPW2, 0, FD, hid0, 0, c, h);
-        norm_swap();
+        norm_swap(done & 1);
       }
-      if constexpr (ROLE == 1) publish(w_replayed, done + 1);
+      if constexpr (ROLE == 1) publish(w_replayed, done / n_replay + 1);
     }
 
     // ================================================================= reverse walk
@@ -812,7 +834,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
     // wave covers the latency, while holding requests in registers across stages costs more in spills
     // than it gains (measured).
     if constexpr (ROLE == 2) {
-      if (!wait_at_least(w_replayed, done + 1, w_status, s_flag)) return;
+      if (!wait_at_least(w_replayed, done / n_replay + 1, w_status, s_flag)) return;
     }
     if constexpr (ROLE != 1)
     for (int j = n_mb - 1; j >= 0; j--) {
@@ -1097,19 +1119,22 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
   if (tid < HID) p.grad_L_b1_init[(size_t)bh * HID + tid] = s_gb1[tid];
   if (tid < FD) p.grad_L_b2_init[(size_t)bh * FD + tid] = s_gb2[tid];
   // norm-weight / norm-bias gradients: sum the per-wave LDS accumulators
-  // (the replay's share: parked in HBM by this workgroup, or handed over by the replaying one, whose last
-  // count this workgroup has acquired before it walked the last group)
+  // The replay's two sums: parked in HBM by this workgroup, or handed over by the replaying workgroups, whose
+  // last counts this workgroup has acquired (a second replaying workgroup has nothing to hand over if there is
+  // one group only).
   if (tid < 2 * FD) {
     const int which = tid / FD, f = tid % FD;
     const float* rp = ROLE == 0 ? reinterpret_cast<const float*>(p.x_hat_ln_group + (size_t)bh * cgs * (CS * FD))
-                                : p.norm_partial + (size_t)bh * (BW_NWAVE * 2 * FD);
-    float s = 0.f, sr = 0.f;
+                                : p.norm_partial + (size_t)bh * 2 * (BW_NWAVE * 2 * FD);
+    const bool have_odd = ROLE == 0 || p.K > 1 || n_replay == 1;
+    float s = 0.f, sr0 = 0.f, sr1 = 0.f;
 #pragma unroll
     for (int u = 0; u < BW_NWAVE; u++) {
       s += s_red[(u * 2 + which) * FD + f];
-      sr += rp[(u * 2 + which) * FD + f];
+      sr0 += rp[(u * 2 + which) * FD + f];
+      if (have_odd) sr1 += rp[BW_NWAVE * 2 * FD + (u * 2 + which) * FD + f];
     }
-    (which == 0 ? p.grad_L_ttt_norm_weight : p.grad_L_ttt_norm_bias)[(size_t)bh * FD + f] = sr + s;
+    (which == 0 ? p.grad_L_ttt_norm_weight : p.grad_L_ttt_norm_bias)[(size_t)bh * FD + f] = (sr0 + sr1) + s;
   }
 }
 #undef REFRESH_OFFSETS
@@ -1124,7 +1149,6 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
 #undef bGZ1B
 #undef bX2B
 #undef bGZB
-#undef bNP
 #undef bIMG1
 #undef bIMG2
 #undef bXHF
@@ -1142,25 +1166,25 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh) {
 
 __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  bwd_body<0>(p, smem, p.bh0 + blockIdx.x);
+  bwd_body<0>(p, smem, p.bh0 + blockIdx.x, 0);
 }
 
-// Two workgroups per (batch, head).  Workgroups are dealt to the 8 XCDs in turn, so with a multiple
-// of 8 (batch, head) pairs the two workgroups of a pair are placed 8 apart: same XCD, same L2.
+// n_replay + 1 workgroups per (batch, head).  Workgroups are dealt to the 8 XCDs in turn, so with a multiple
+// of 8 (batch, head) pairs the workgroups of a pair are placed 8 apart: same XCD, same L2.
 __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_split_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int b = blockIdx.x;
+  const int b = blockIdx.x, per = p.n_replay + 1;
   int bh, role;
   if (p.nbh % 8 == 0) {
-    bh = (b >> 4) * 8 + (b & 7);
-    role = (b >> 3) & 1;
+    bh = (b / (8 * per)) * 8 + (b & 7);
+    role = (b >> 3) % per;
   } else {
-    bh = b >> 1;
-    role = b & 1;
+    bh = b / per;
+    role = b % per;
   }
   bh += p.bh0;
-  if (role == 0) bwd_body<1>(p, smem, bh);
-  else bwd_body<2>(p, smem, bh);
+  if (role < p.n_replay) bwd_body<1>(p, smem, bh, role);
+  else bwd_body<2>(p, smem, bh, 0);
 }
 
 __global__ void ttt_mlp_zero_words(int* w, int n) {
@@ -1187,6 +1211,6 @@ hipError_t ttt_mlp_bwd_enqueue(const ttt::BwdParams& p, hipStream_t stream) {
   const int n = static_cast<int>(ttt::bwd_sync_ints(p.nbh));
   int* const words = p.status - (size_t)p.nbh * ttt::BWD_SYNC_STRIDE;   // p.sync itself is moved back by bh0 entries
   hipLaunchKernelGGL(ttt::ttt_mlp_zero_words, dim3((n + 255) / 256), dim3(256), 0, stream, words, n);
-  hipLaunchKernelGGL(ttt::ttt_mlp_bwd_split_kernel, dim3(2 * p.nbh), dim3(ttt::BW_THREADS), ttt::SM_BWD_BYTES, stream, p);
+  hipLaunchKernelGGL(ttt::ttt_mlp_bwd_split_kernel, dim3((p.n_replay + 1) * p.nbh), dim3(ttt::BW_THREADS), ttt::SM_BWD_BYTES, stream, p);
   return hipGetLastError();
 }

@@ -120,10 +120,11 @@ struct LaunchPlan {
   long long n_single = 0;   // pairs 0 .. n_single-1: one workgroup each
   long long n_rest = 0;     // pairs n_single .. n_single+n_rest-1
   bool rest_split = false;
+  int per_pair = 1;         // workgroups per pair of the rest: 2, or 3 where the kernel can use them and they fit
 };
 // `after_full_rounds`: whether the rest may be split when full rounds precede it.  That pays for the
 // backward; the forward's gain from splitting is smaller than what a full device costs it (measured).
-LaunchPlan plan_launches(long long BH, bool after_full_rounds) {
+LaunchPlan plan_launches(long long BH, bool after_full_rounds, bool three_way) {
   LaunchPlan pl;
   int dev = 0, cus = 0;
   if (BH <= 0 || hipGetDevice(&dev) != hipSuccess ||
@@ -135,23 +136,32 @@ LaunchPlan plan_launches(long long BH, bool after_full_rounds) {
   pl.n_rest = BH - pl.n_single;
   pl.rest_split = pl.n_rest > 0 && 2 * pl.n_rest <= cus && (after_full_rounds || pl.n_single == 0);
   if (!pl.rest_split) { pl.n_single = BH; pl.n_rest = 0; }
+  else pl.per_pair = (three_way && 3 * pl.n_rest <= cus) ? 3 : 2;
   return pl;
 }
 
-// Workspace of the backward's two-workgroup mode for n (batch, head) pairs: the synchronisation words,
-// the replaying workgroups' share of the norm gradients, then the alternate set of the ten per-group
-// tensors that carry a replayed group to the reverse walk; each part 256-byte aligned.
+// Workspace of the backward with 2 or 3 workgroups per pair, for n (batch, head) pairs: the synchronisation
+// words, the replay's shares of the norm gradients (two sums per pair + one parking slot), then 1 or 3
+// alternate sets of the ten per-group tensors that carry a replayed group to the reverse walk; each part
+// 256-byte aligned.
 struct BwdWorkspace {
-  size_t off[11];
+  static constexpr int PARTS = 3 + 10 * 3;
+  size_t off[PARTS];
   size_t total;
-  BwdWorkspace(long long n, long long cgs) {
+  BwdWorkspace(long long n, long long cgs, int alt_sets) {
     const size_t slot = (size_t)n * (size_t)cgs;
     const size_t tile = TTT_MLP_CS * TTT_MLP_F * 2, img = TTT_MLP_CS * TTT_MLP_HID * 2, vec = TTT_MLP_CS * 4;
-    const size_t bytes[11] = {ttt::bwd_sync_ints(n) * sizeof(int), (size_t)n * 8 * 2 * TTT_MLP_F * sizeof(float),
-                              slot * img, slot * img, slot * img, slot * img, slot * tile, slot * img, slot * tile,
-                              slot * tile + slot * tile, slot * vec};
+    const size_t norm = (size_t)n * 8 * 2 * TTT_MLP_F * sizeof(float);
+    // per set: X2, Z1, Z1_bar, X2_bar (images), gZ2 (tile), gZ1 (image), x_hat_fused, g_x_hat_fused, g_out_fused (tiles), std_fused
+    const size_t per_set[10] = {slot * img, slot * img, slot * img, slot * img, slot * tile, slot * img,
+                                slot * tile, slot * tile, slot * tile, slot * vec};
     size_t o = 0;
-    for (int i = 0; i < 11; i++) { off[i] = o; o += (bytes[i] + 255) & ~(size_t)255; }
+    auto put = [&](int i, size_t bytes) { off[i] = o; o += (bytes + 255) & ~(size_t)255; };
+    put(0, ttt::bwd_sync_ints(n) * sizeof(int));
+    put(1, 2 * norm);
+    put(2, norm);
+    for (int s = 0; s < 3; s++)
+      for (int t = 0; t < 10; t++) put(3 + 10 * s + t, s < alt_sets ? per_set[t] : 0);
     total = o;
   }
 };
@@ -189,17 +199,18 @@ extern "C" int ttt_mlp_bwd_launch(const ttt_mlp_bwd_args* a, void* stream) {
 
 extern "C" size_t ttt_mlp_bwd_workspace_bytes(int B, int NH, int checkpoint_group_size) {
   if (B <= 0 || NH <= 0 || checkpoint_group_size <= 0 || checkpoint_group_size > (1 << 16)) return 0;
-  const LaunchPlan pl = plan_launches((long long)B * NH, true);
-  return pl.rest_split ? BwdWorkspace(pl.n_rest, checkpoint_group_size).total : 0;
+  const LaunchPlan pl = plan_launches((long long)B * NH, true, true);
+  return pl.rest_split ? BwdWorkspace(pl.n_rest, checkpoint_group_size, 2 * (pl.per_pair - 1) - 1).total : 0;
 }
 
 extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* workspace, size_t workspace_bytes, void* stream) {
   ttt::BwdParams p;
   if (int rc = make_bwd_params(a, p)) return rc;
   if (int rc = check_workspace(workspace)) return rc;
-  const LaunchPlan pl = plan_launches((long long)p.B * p.NH, true);
+  const LaunchPlan pl = plan_launches((long long)p.B * p.NH, true, true);
   if (!pl.rest_split) return TTT_MLP_ERR_NO_ROOM;
-  const BwdWorkspace w(pl.n_rest, p.cgs);
+  const int n_replay = pl.per_pair - 1, alt_sets = 2 * n_replay - 1;
+  const BwdWorkspace w(pl.n_rest, p.cgs, alt_sets);
   if (workspace_bytes < w.total) return TTT_MLP_ERR_WORKSPACE;
   if (pl.n_single > 0) {
     p.bh0 = 0;
@@ -209,24 +220,29 @@ extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* wo
   // The kernels index the workspace by the global pair number: every pointer is moved back by bh0 entries.
   char* base = static_cast<char*>(workspace);
   const size_t b0 = (size_t)pl.n_single;
-  const size_t slot_elems = (size_t)pl.n_rest * p.cgs * (TTT_MLP_CS * TTT_MLP_F);   // one [n_rest,cgs,CS,F] tensor
   const size_t tile = (size_t)p.cgs * TTT_MLP_CS * TTT_MLP_F, img = (size_t)p.cgs * TTT_MLP_CS * TTT_MLP_HID, vec = (size_t)p.cgs * TTT_MLP_CS;
+  const size_t norm = 8 * 2 * TTT_MLP_F;
   p.bh0 = static_cast<int>(pl.n_single);
   p.nbh = static_cast<int>(pl.n_rest);
+  p.n_replay = n_replay;
   int* words = reinterpret_cast<int*>(base + w.off[0]);
   p.status = words + (size_t)pl.n_rest * ttt::BWD_SYNC_STRIDE;
   p.sync = words - b0 * ttt::BWD_SYNC_STRIDE;
-  p.norm_partial = reinterpret_cast<float*>(base + w.off[1]) - b0 * (8 * 2 * TTT_MLP_F);
-  p.alt_X2_group = reinterpret_cast<__bf16*>(base + w.off[2]) - b0 * img;
-  p.alt_Z1_group = reinterpret_cast<__bf16*>(base + w.off[3]) - b0 * img;
-  p.alt_Z1_bar_group = reinterpret_cast<__bf16*>(base + w.off[4]) - b0 * img;
-  p.alt_X2_bar_group = reinterpret_cast<__bf16*>(base + w.off[5]) - b0 * img;
-  p.alt_grad_l_wrt_Z2_group = reinterpret_cast<__bf16*>(base + w.off[6]) - b0 * tile;
-  p.alt_grad_l_wrt_Z1_group = reinterpret_cast<__bf16*>(base + w.off[7]) - b0 * img;
-  p.alt_x_hat_fused_group = reinterpret_cast<__bf16*>(base + w.off[8]) - b0 * tile;
-  p.alt_grad_x_hat_fused_group = reinterpret_cast<__bf16*>(base + w.off[9]) - b0 * tile;
-  p.alt_grad_output_fused_group = reinterpret_cast<__bf16*>(base + w.off[9]) + slot_elems - b0 * tile;
-  p.alt_std_fused_group = reinterpret_cast<float*>(base + w.off[10]) - b0 * vec;
+  p.norm_partial = reinterpret_cast<float*>(base + w.off[1]) - b0 * 2 * norm;
+  p.norm_park = reinterpret_cast<float*>(base + w.off[2]) - b0 * norm;
+  for (int s = 0; s < alt_sets; s++) {
+    const size_t* o = w.off + 3 + 10 * s;
+    p.alt_X2_group[s] = reinterpret_cast<__bf16*>(base + o[0]) - b0 * img;
+    p.alt_Z1_group[s] = reinterpret_cast<__bf16*>(base + o[1]) - b0 * img;
+    p.alt_Z1_bar_group[s] = reinterpret_cast<__bf16*>(base + o[2]) - b0 * img;
+    p.alt_X2_bar_group[s] = reinterpret_cast<__bf16*>(base + o[3]) - b0 * img;
+    p.alt_grad_l_wrt_Z2_group[s] = reinterpret_cast<__bf16*>(base + o[4]) - b0 * tile;
+    p.alt_grad_l_wrt_Z1_group[s] = reinterpret_cast<__bf16*>(base + o[5]) - b0 * img;
+    p.alt_x_hat_fused_group[s] = reinterpret_cast<__bf16*>(base + o[6]) - b0 * tile;
+    p.alt_grad_x_hat_fused_group[s] = reinterpret_cast<__bf16*>(base + o[7]) - b0 * tile;
+    p.alt_grad_output_fused_group[s] = reinterpret_cast<__bf16*>(base + o[8]) - b0 * tile;
+    p.alt_std_fused_group[s] = reinterpret_cast<float*>(base + o[9]) - b0 * vec;
+  }
   return static_cast<int>(ttt_mlp_bwd_enqueue(p, static_cast<hipStream_t>(stream)));
 }
 
@@ -240,7 +256,7 @@ extern "C" int ttt_mlp_fwd_launch(const ttt_mlp_fwd_args* a, void* stream) {
 
 extern "C" size_t ttt_mlp_fwd_workspace_bytes(int B, int NH) {
   if (B <= 0 || NH <= 0) return 0;
-  const LaunchPlan pl = plan_launches((long long)B * NH, false);
+  const LaunchPlan pl = plan_launches((long long)B * NH, false, false);
   return pl.rest_split ? FwdWorkspace(pl.n_rest).total : 0;
 }
 
@@ -248,7 +264,7 @@ extern "C" int ttt_mlp_fwd_launch_overlapped(const ttt_mlp_fwd_args* a, void* wo
   ttt::FwdParams p;
   if (int rc = make_fwd_params(a, p)) return rc;
   if (int rc = check_workspace(workspace)) return rc;
-  const LaunchPlan pl = plan_launches((long long)p.B * p.NH, false);
+  const LaunchPlan pl = plan_launches((long long)p.B * p.NH, false, false);
   if (!pl.rest_split) return TTT_MLP_ERR_NO_ROOM;
   const FwdWorkspace w(pl.n_rest);
   if (workspace_bytes < w.total) return TTT_MLP_ERR_WORKSPACE;

@@ -44,21 +44,25 @@ struct BwdParams {
   float *grad_L_W1_init, *grad_L_b1_init, *grad_L_W2_init, *grad_L_b2_init;
   __bf16 *grad_L_last_eta, *grad_L_XQ, *grad_L_XK, *grad_L_XV;
   int B, NH, NC, K, cgs;
-  // Two-workgroup mode only (sync != nullptr): a second set of the per-group tensors that carry a
-  // replayed group to the reverse walk, and the words the two workgroups of a (batch, head) signal with.
-  __bf16 *alt_X2_group, *alt_Z1_group, *alt_Z1_bar_group, *alt_X2_bar_group;
-  __bf16 *alt_grad_l_wrt_Z2_group, *alt_grad_l_wrt_Z1_group;
-  __bf16 *alt_x_hat_fused_group, *alt_grad_x_hat_fused_group, *alt_grad_output_fused_group;
-  float* alt_std_fused_group;
-  float* norm_partial;   // [B*NH][8 waves][2][64]: the replaying workgroup's share of the norm-weight / norm-bias gradients
+  // Several workgroups per (batch, head) only (sync != nullptr): n_replay = 1 or 2 workgroups replay the
+  // checkpoint groups (taking turns), one walks them backwards.  Group number g (0 = the last group of the
+  // sequence) is replayed into set g % (2 * n_replay) of the per-group tensors that carry it to the walk:
+  // set 0 = the caller's tensors, sets 1.. = alt_*[set - 1] from the workspace.
+  __bf16 *alt_X2_group[3], *alt_Z1_group[3], *alt_Z1_bar_group[3], *alt_X2_bar_group[3];
+  __bf16 *alt_grad_l_wrt_Z2_group[3], *alt_grad_l_wrt_Z1_group[3];
+  __bf16 *alt_x_hat_fused_group[3], *alt_grad_x_hat_fused_group[3], *alt_grad_output_fused_group[3];
+  float* alt_std_fused_group[3];
+  float* norm_partial;   // [B*NH][2][8 waves][2][64]: the replay's share of the norm-weight / norm-bias gradients, by group parity
+  float* norm_park;      // [B*NH][8 waves][2][64]: n_replay = 1: the share of the parity that is not being added to
+  int n_replay;
   int* sync;
   int* status;    // the status word behind the synchronisation words
   int bh0, nbh;   // this launch covers (batch, head) pairs bh0 .. bh0 + nbh - 1 (workspace pointers moved back by bh0 entries)
 };
 
-// Layout of `sync` (ints): 32 per (batch, head) - word 0 counts the groups replayed (norm_partial is
-// written before the last count), word 16 the groups the reverse walk has finished - then one status
-// word (non-zero: a wait gave up).
+// Layout of `sync` (ints): 32 per (batch, head) - words 0 and 8 count the groups replayed by the first /
+// second replaying workgroup (norm_partial is written before the last count), word 16 the groups the
+// reverse walk has finished - then one status word (non-zero: a wait gave up).
 constexpr int BWD_SYNC_STRIDE = 32;
 inline size_t bwd_sync_ints(long long BH) { return (size_t)BH * BWD_SYNC_STRIDE + 32; }
 
