@@ -83,6 +83,19 @@ constexpr unsigned IMG_BYTES = CS * HID * 2;          // 32 KiB
 constexpr unsigned CHUNK_BYTES = BW_THREADS * 16;     // 8 KiB
 constexpr unsigned TILE_BYTES = CS * FD * 2;          // one [64][64] bf16 tile in HBM: 8 KiB
 TTT_DEV void chunk_store(gptr_t b, unsigned img, int n, unsigned t16, bf16x8 v) { g_st8h(b, t16, img + n * CHUNK_BYTES, v); }
+// The replay's images: written once and read a checkpoint group later.  When another workgroup reads them
+// (STREAM) they bypass the cache hierarchy as far as the hardware lets them, so that they do not push out
+// lines that are re-used; with one workgroup per (batch, head) keeping them cached measured faster.
+template <bool STREAM>
+TTT_DEV void image_store(gptr_t b, unsigned img, int n, unsigned t16, bf16x8 v) {
+  if constexpr (STREAM) g_st_stream<bf16x8>(b, t16, img + n * CHUNK_BYTES, v);
+  else g_st8h(b, t16, img + n * CHUNK_BYTES, v);
+}
+template <bool STREAM>
+TTT_DEV bf16x8 image_load(gptr_t b, unsigned img, int n, unsigned t16) {
+  if constexpr (STREAM) return g_ld_stream<bf16x8>(b, t16, img + n * CHUNK_BYTES);
+  else return g_ld8h(b, t16, img + n * CHUNK_BYTES);
+}
 TTT_DEV bf16x8 chunk_load(gptr_t b, unsigned img, int n, unsigned t16) { return g_ld8h(b, t16, img + n * CHUNK_BYTES); }
 
 // fp32 accumulator tile <-> HBM in the caller's row-major layout.  `ld` = row length, (r0, c0) =
@@ -140,11 +153,13 @@ TTT_DEV void ln_store(bf16* p, const float (&x)[8]) {
   *reinterpret_cast<bf16x4*>(p + 4) = b;
 }
 // 8 features of this lane's token to / from a [tok][F] bf16 tile in HBM (16 bytes per lane).
+template <bool STREAM = false>
 TTT_DEV void ln_store_g(gptr_t b, unsigned voff, unsigned soff, const float (&x)[8]) {
   bf16x8 v;
 #pragma unroll
   for (int e = 0; e < 8; e++) v[e] = (bf16)x[e];
-  g_st8h(b, voff, soff, v);
+  if constexpr (STREAM) g_st_stream<bf16x8>(b, voff, soff, v);
+  else g_st8h(b, voff, soff, v);
 }
 TTT_DEV void ln_cvt8(float (&x)[8], bf16x8 v) {
 #pragma unroll
@@ -477,9 +492,12 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
 #define bSDF gbuf(GRP(std_fused_group) + ot)
   // While a group is replayed the running gradients are parked in W*_init_group; during the reverse
   // walk the same two 64 KiB slots park what must survive the LayerNorm stage (three 32 KiB images).
+  // Several workgroups per (batch, head): slot j of W1_init_group (of the set) carries gelu'(Z1) and gelu''(Z1)
+  // of mini-batch j as two register images, and Z1_group carries gelu(Z1) instead of Z1.
+#define bDD gbuf(GRP(W1_init_group) + opk)
 #define bPW1 gbuf(ka->W1_init_group + opk)
 #define bPW2 gbuf(ka->W2_init_group + opk)
-  constexpr unsigned PARK_D1 = 0, PARK_T2 = IMG_BYTES, PARK_G1 = 0;   // d1, t2 in bPW1; g1 in bPW2
+  constexpr unsigned PARK_D1 = 0, PARK_T2 = IMG_BYTES, PARK_G1 = 0;   // d1 in bPW1 (one workgroup only); g1, t2 in bPW2
 #define bCW1 gbuf(ka->W1_ck + ock)
 #define bCW2 gbuf(ka->W2_ck + ock)
 #define bDXQ gbuf(ka->grad_L_XQ + ox)
@@ -597,7 +615,25 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int t = 0; t < 2; t++) {
-              chunk_store(bZ1, j * IMG_BYTES, 2 * tb[i] + t, t16, pack8(x2.b[0][i], t));
+              const bf16x8 zr = pack8(x2.b[0][i], t);
+              if constexpr (ROLE == 0) {
+                image_store<ROLE != 0>(bZ1, j * IMG_BYTES, 2 * tb[i] + t, t16, zr);
+              } else {
+                // The walk needs gelu, gelu' and gelu'' of the ROUNDED Z1 (what it would compute from the image
+                // of Z1); a replaying workgroup has the time to do that for it.
+                bf16x8 gv, av, bv;
+#pragma unroll
+                for (int jj = 0; jj < 8; jj++) {
+                  float g, a, b;
+                  gelu_fdd((float)zr[jj], g, a, b);
+                  gv[jj] = (bf16)g;
+                  av[jj] = (bf16)a;
+                  bv[jj] = (bf16)b;
+                }
+                image_store<ROLE != 0>(bZ1, j * IMG_BYTES, 2 * tb[i] + t, t16, gv);
+                image_store<ROLE != 0>(bDD, j * (2 * IMG_BYTES), 2 * tb[i] + t, t16, av);
+                image_store<ROLE != 0>(bDD, j * (2 * IMG_BYTES) + IMG_BYTES, 2 * tb[i] + t, t16, bv);
+              }
               bf16x8 xv;
 #pragma unroll
               for (int jj = 0; jj < 8; jj++) {
@@ -644,13 +680,13 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
               gx[e] = go[e] * gam[e];
             }
           }
-          ln_store_g(bXHF, vln, j * TILE_BYTES, z);
-          ln_store_g(bGOF, vln, j * TILE_BYTES, go);
+          ln_store_g<ROLE != 0>(bXHF, vln, j * TILE_BYTES, z);
+          ln_store_g<ROLE != 0>(bGOF, vln, j * TILE_BYTES, go);
           const float s1 = oct_sum(sum8(gx)), s2 = oct_sum(dot8(gx, z));
           const float sc = rstd * (1.f / FD), neg_eta = -s_eta[tok];
 #pragma unroll
           for (int e = 0; e < 8; e++) gx[e] = (FD * gx[e] - s1 - z[e] * s2) * sc;   // dl/dZ2
-          ln_store_g(bGZ2, vln, j * TILE_BYTES, gx);
+          ln_store_g<ROLE != 0>(bGZ2, vln, j * TILE_BYTES, gx);
 #pragma unroll
           for (int e = 0; e < 8; e++) gx[e] *= neg_eta;                             // G2
           ln_store(s_gz2 + tok * LDX + f0, gx);
@@ -692,12 +728,12 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           // bIMG2: W2, lane = hid, contraction = F;  bIMG1: W1^T, lane = F, contraction = hid
           store_state_rows<LDF>(T2, W1s, c, h);                                 // rows [hid][F]
 #pragma unroll
-          for (int s = 0; s < 4; s++) chunk_store(bIMG2, j * IMG_BYTES, s, t16, piece_state(W2t, 0, s));
+          for (int s = 0; s < 4; s++) image_store<ROLE != 0>(bIMG2, j * IMG_BYTES, s, t16, piece_state(W2t, 0, s));
           WAVE_SYNC();
 #pragma unroll
           for (int fb = 0; fb < 2; fb++)
 #pragma unroll
-            for (int s = 0; s < 2; s++) chunk_store(bIMG1, j * IMG_BYTES, 2 * fb + s, t16, piece_tr<LDF>(T2, fb, s, lane));
+            for (int s = 0; s < 2; s++) image_store<ROLE != 0>(bIMG1, j * IMG_BYTES, 2 * fb + s, t16, piece_tr<LDF>(T2, fb, s, lane));
         }
         // post-update forward on XQ; X2_bar rows [tok][hid] -> T0, gelu'(Z1_bar) packed
         bf16x8 d1b[2][2];
@@ -761,7 +797,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
 #pragma unroll
           for (int e = 0; e < 8; e++) gx[e] = (FD * gx[e] - s1 - z[e] * s2) * sc;
           ln_store(s_a + tok * LDX + f0, gx);            // gZ2_bar
-          ln_store_g(bGZB, vln, j * TILE_BYTES, gx);
+          ln_store_g<ROLE != 0>(bGZB, vln, j * TILE_BYTES, gx);
           if (j + 1 < n_mb) stage3_store(st, s_xq, s_xk, s_e2, s_eta, tid);
         }
         __syncthreads();
@@ -791,8 +827,8 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           // what the reverse walk adds to the running gradients, as ready-made operands (lane = hid, contraction = tok)
 #pragma unroll
           for (int s = 0; s < 4; s++) {
-            chunk_store(bX2B, j * IMG_BYTES, s, t16, piece_tr<LDH>(T0, 0, s, lane));
-            chunk_store(bGZ1B, j * IMG_BYTES, s, t16, piece_tr<LDH>(T1, 0, s, lane));
+            image_store<ROLE != 0>(bX2B, j * IMG_BYTES, s, t16, piece_tr<LDH>(T0, 0, s, lane));
+            image_store<ROLE != 0>(bGZ1B, j * IMG_BYTES, s, t16, piece_tr<LDH>(T1, 0, s, lane));
           }
           WAVE_SYNC();   // every reader of T1 / T2 is done before the pair sum takes their place
           pair_sum(s_own, s_partner, dq, c, h);
@@ -848,8 +884,10 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
       const float eta_i[2] = {bf2f(g_ldh(bETA, 2 * c, mb * (CS * 2) + 64 * tb[0])), bf2f(g_ldh(bETA, 2 * c, mb * (CS * 2) + 64 * tb[1]))};
       {
         LANE_VARS;
-        const u32x4 xq = g_ld16(bXQ, t16, xo), xk = g_ld16(bXK, t16, xo), gz = g_ld16(bGZ2, t16, so);
-        const u32x4 gzb = g_ld16(bGZB, t16, so);
+        constexpr bool ST = ROLE != 0;   // tiles another workgroup left here are read once
+        const u32x4 xq = g_ld16(bXQ, t16, xo), xk = g_ld16(bXK, t16, xo);
+        const u32x4 gz = ST ? g_ld_stream<u32x4>(bGZ2, t16, so) : g_ld16(bGZ2, t16, so);
+        const u32x4 gzb = ST ? g_ld_stream<u32x4>(bGZB, t16, so) : g_ld16(bGZB, t16, so);
         const float eta = bf2f(g_ldh(bETA, 2 * (tid & (CS - 1)), mb * (CS * 2)));
         __syncthreads();   // the previous mini-batch's readers of these tiles are done (the loads are under way)
         lds_put16(s_xq, tid, xq);
@@ -863,16 +901,27 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
       // ---- what the output branch adds to the running gradients.  The replay has taken that branch
       //      backwards already and left gZ2_bar (now in LDS) and X2_bar^T, gZ1_bar^T as operand images.
       bf16x8 w2bf[4];   // W2 before this step (lane = hid, contraction = F): fetched now, needed by the next stage
+      bf16x8 gq[2][2], aq[2][2], bq[2][2];
       {
         LANE_VARS;
         bf16x8 x2b[4], g1b[4];   // lane = hid, contraction = tok
 #pragma unroll
         for (int s = 0; s < 4; s++) {
-          x2b[s] = chunk_load(bX2B, ho, s, t16);
-          g1b[s] = chunk_load(bGZ1B, ho, s, t16);
+          x2b[s] = image_load<ROLE != 0>(bX2B, ho, s, t16);
+          g1b[s] = image_load<ROLE != 0>(bGZ1B, ho, s, t16);
         }
 #pragma unroll
         for (int s = 0; s < 4; s++) w2bf[s] = w2_before(bIMG2, bCW2, ckW, j, s, hid0, c, h, t16);
+        if constexpr (ROLE == 2) {   // the three GELU images of the next stage, under way during this one
+#pragma unroll
+          for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+              gq[i][t] = image_load<true>(bZ1, ho, 2 * tb[i] + t, t16);
+              aq[i][t] = chunk_load(bDD, j * (2 * IMG_BYTES), 2 * tb[i] + t, t16);   // read again two stages on
+              bq[i][t] = image_load<true>(bDD, j * (2 * IMG_BYTES) + IMG_BYTES, 2 * tb[i] + t, t16);
+            }
+        }
         mma_jit<4>(gW2s, [&](int, int s) { return x2b[s]; },                                   // X2_bar^T: lane = hid
                    [&](int fb, int s) { return piece_tr<LDX>(s_a, fb, s, lane); });            // gZ2_bar: lane = F
         if (v < 2) lds_rowsum_add_jit(s_gb2 + 32 * v, [&](int s) { return piece_tr<LDX>(s_a, v, s, lane); }, ones, c, h);
@@ -908,27 +957,46 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           mma_jit<4>(S, [&](int, int s) { return piece_rows<LDF>(T2, 0, s, c, h); },
                      [&](int, int s) { return piece_rows<LDX>(s_xk, tb[i], s, c, h); });
           bf16x8 x2c[2], uc[2];
-          const bf16x8 zc[2] = {chunk_load(bZ1, ho, 2 * tb[i], t16), chunk_load(bZ1, ho, 2 * tb[i] + 1, t16)};
+          // gelu(Z1), gelu'(Z1), gelu''(Z1), each rounded to bf16: computed here from the image of Z1, or
+          // fetched as three images that a replaying workgroup computed the same way
+          bf16x8 ac[2], bc[2];
+          if constexpr (ROLE == 0) {
+            const bf16x8 zc[2] = {chunk_load(bZ1, ho, 2 * tb[i], t16), chunk_load(bZ1, ho, 2 * tb[i] + 1, t16)};
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+              for (int jj = 0; jj < 8; jj++) {
+                float g, a, b;
+                gelu_fdd((float)zc[t][jj], g, a, b);
+                x2c[t][jj] = (bf16)g;
+                ac[t][jj] = (bf16)a;
+                bc[t][jj] = (bf16)b;
+              }
+          } else {
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+              x2c[t] = gq[i][t];
+              ac[t] = aq[i][t];
+              bc[t] = bq[i][t];
+            }
+          }
 #pragma unroll
           for (int t = 0; t < 2; t++) {
-            bf16x8 d1c, t2c, g1c;
+            bf16x8 t2c, g1c;
 #pragma unroll
             for (int jj = 0; jj < 8; jj++) {
-              float g, a, b;
-              gelu_fdd((float)zc[t][jj], g, a, b);
+              const float a = (float)ac[t][jj], b = (float)bc[t][jj];
               const float r0 = R.b[0][0][8 * t + jj], sv = S.b[0][0][8 * t + jj];
               const float gz1 = r0 * a;                                   // dl/dZ1
               de[i] = __builtin_fmaf(gz1, sv, de[i]);
-              x2c[t][jj] = (bf16)g;
               uc[t][jj] = (bf16)(sv * a);
               g1c[jj] = (bf16)(-eta_i[i] * gz1);
-              d1c[jj] = (bf16)a;
               t2c[jj] = (bf16)(-eta_i[i] * r0 * sv * b);
             }
-            // nothing stays in registers across the LayerNorm stage: d1, g1 and t2 go to their parks at
-            // once (L2-resident, rewritten every mini-batch; 1 KiB per wave instruction)
-            chunk_store(bPW1, PARK_D1, 2 * tb[i] + t, t16, d1c);
-            chunk_store(bPW1, PARK_T2, 2 * tb[i] + t, t16, t2c);
+            // nothing stays in registers across the LayerNorm stage: g1 and t2 (and, without the images,
+            // gelu'(Z1)) go to their parks at once (L2-resident, rewritten every mini-batch)
+            if constexpr (ROLE == 0) chunk_store(bPW1, PARK_D1, 2 * tb[i] + t, t16, ac[t]);
+            chunk_store(bPW2, PARK_T2, 2 * tb[i] + t, t16, t2c);
             chunk_store(bPW2, PARK_G1, 2 * tb[i] + t, t16, g1c);
             store_piece_rows<LDH>(T0, tb[i], t, c, h, x2c[t]);             // X2 rows [tok][hid]
           }
@@ -965,7 +1033,8 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         float gg[8], xh[8], go[8], gz[8], gam[8], gb[8];
         dxv_old = g_ld8h(bDXV, vln, xo);
         deta_old = g_ldh(bDETA, 2 * tok, mb * (CS * 2));
-        const bf16x8 xhf = g_ld8h(bXHF, vln, so), gof = g_ld8h(bGOF, vln, so);
+        const bf16x8 xhf = ROLE != 0 ? g_ld_stream<bf16x8>(bXHF, vln, so) : g_ld8h(bXHF, vln, so);
+        const bf16x8 gof = ROLE != 0 ? g_ld_stream<bf16x8>(bGOF, vln, so) : g_ld8h(bGOF, vln, so);
         const float sdf = g_ldf(bSDF, vtok, j * (CS * 4));
         ln_gather(gg, s_lnrow);
         ln_load_f32(gb, s_gb2 + f0);
@@ -1053,8 +1122,15 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
                      [&](int, int s) { return piece_rows<LDX>(s_a, tb[i], s, c, h); });
           // dk[:, i] = gW1 G1^T  (gW1: lane = F, contraction = hid)
           const bf16x8 g1c[2] = {chunk_load(bPW2, PARK_G1, 2 * tb[i], t16), chunk_load(bPW2, PARK_G1, 2 * tb[i] + 1, t16)};
-          const bf16x8 d1c[2] = {chunk_load(bPW1, PARK_D1, 2 * tb[i], t16), chunk_load(bPW1, PARK_D1, 2 * tb[i] + 1, t16)};
-          const bf16x8 t2c[2] = {chunk_load(bPW1, PARK_T2, 2 * tb[i], t16), chunk_load(bPW1, PARK_T2, 2 * tb[i] + 1, t16)};
+          bf16x8 d1c[2];
+          if constexpr (ROLE == 0) {
+            d1c[0] = chunk_load(bPW1, PARK_D1, 2 * tb[i], t16);
+            d1c[1] = chunk_load(bPW1, PARK_D1, 2 * tb[i] + 1, t16);
+          } else {
+            d1c[0] = chunk_load(bDD, j * (2 * IMG_BYTES), 2 * tb[i], t16);
+            d1c[1] = chunk_load(bDD, j * (2 * IMG_BYTES), 2 * tb[i] + 1, t16);
+          }
+          const bf16x8 t2c[2] = {chunk_load(bPW2, PARK_T2, 2 * tb[i], t16), chunk_load(bPW2, PARK_T2, 2 * tb[i] + 1, t16)};
 #pragma unroll
           for (int t = 0; t < 2; t++)
 #pragma unroll
@@ -1155,6 +1231,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
 #undef bGOF
 #undef bGZ2
 #undef bSDF
+#undef bDD
 #undef bPW1
 #undef bPW2
 #undef bCW1

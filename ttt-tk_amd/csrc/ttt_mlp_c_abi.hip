@@ -145,23 +145,25 @@ LaunchPlan plan_launches(long long BH, bool after_full_rounds, bool three_way) {
 // alternate sets of the ten per-group tensors that carry a replayed group to the reverse walk; each part
 // 256-byte aligned.
 struct BwdWorkspace {
-  static constexpr int PARTS = 3 + 10 * 3;
+  static constexpr int PER_SET = 11;
+  static constexpr int PARTS = 3 + PER_SET * 3;
   size_t off[PARTS];
   size_t total;
   BwdWorkspace(long long n, long long cgs, int alt_sets) {
     const size_t slot = (size_t)n * (size_t)cgs;
     const size_t tile = TTT_MLP_CS * TTT_MLP_F * 2, img = TTT_MLP_CS * TTT_MLP_HID * 2, vec = TTT_MLP_CS * 4;
     const size_t norm = (size_t)n * 8 * 2 * TTT_MLP_F * sizeof(float);
-    // per set: X2, Z1, Z1_bar, X2_bar (images), gZ2 (tile), gZ1 (image), x_hat_fused, g_x_hat_fused, g_out_fused (tiles), std_fused
-    const size_t per_set[10] = {slot * img, slot * img, slot * img, slot * img, slot * tile, slot * img,
-                                slot * tile, slot * tile, slot * tile, slot * vec};
+    // per set: X2, Z1, Z1_bar, X2_bar (images), gZ2 (tile), gZ1 (image), x_hat_fused, g_x_hat_fused, g_out_fused
+    // (tiles), std_fused, W1_init (two images per slot)
+    const size_t per_set[PER_SET] = {slot * img, slot * img, slot * img, slot * img, slot * tile, slot * img,
+                                     slot * tile, slot * tile, slot * tile, slot * vec, slot * 2 * img};
     size_t o = 0;
     auto put = [&](int i, size_t bytes) { off[i] = o; o += (bytes + 255) & ~(size_t)255; };
     put(0, ttt::bwd_sync_ints(n) * sizeof(int));
     put(1, 2 * norm);
     put(2, norm);
     for (int s = 0; s < 3; s++)
-      for (int t = 0; t < 10; t++) put(3 + 10 * s + t, s < alt_sets ? per_set[t] : 0);
+      for (int t = 0; t < PER_SET; t++) put(3 + PER_SET * s + t, s < alt_sets ? per_set[t] : 0);
     total = o;
   }
 };
@@ -231,7 +233,7 @@ extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* wo
   p.norm_partial = reinterpret_cast<float*>(base + w.off[1]) - b0 * 2 * norm;
   p.norm_park = reinterpret_cast<float*>(base + w.off[2]) - b0 * norm;
   for (int s = 0; s < alt_sets; s++) {
-    const size_t* o = w.off + 3 + 10 * s;
+    const size_t* o = w.off + 3 + BwdWorkspace::PER_SET * s;
     p.alt_X2_group[s] = reinterpret_cast<__bf16*>(base + o[0]) - b0 * img;
     p.alt_Z1_group[s] = reinterpret_cast<__bf16*>(base + o[1]) - b0 * img;
     p.alt_Z1_bar_group[s] = reinterpret_cast<__bf16*>(base + o[2]) - b0 * img;
@@ -242,6 +244,7 @@ extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* wo
     p.alt_grad_x_hat_fused_group[s] = reinterpret_cast<__bf16*>(base + o[7]) - b0 * tile;
     p.alt_grad_output_fused_group[s] = reinterpret_cast<__bf16*>(base + o[8]) - b0 * tile;
     p.alt_std_fused_group[s] = reinterpret_cast<float*>(base + o[9]) - b0 * vec;
+    p.alt_W1_init_group[s] = reinterpret_cast<float*>(base + o[10]) - b0 * img;   // [cgs][64][256] floats = 2 images per slot
   }
   return static_cast<int>(ttt_mlp_bwd_enqueue(p, static_cast<hipStream_t>(stream)));
 }

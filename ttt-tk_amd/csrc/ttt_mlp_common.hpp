@@ -304,6 +304,22 @@ TTT_DEV void g_st(gptr_t b, unsigned voff, unsigned soff, T v) {
   asm("" : "+s"(q), "+v"(voff));
   *(ptr_t)(q + static_cast<uint64_t>(voff)) = v;
 }
+// Streaming variants (`nt`): data written once and read once much later, by this or another workgroup,
+// should not push re-used lines out of the L2.
+template <class T>
+TTT_DEV void g_st_stream(gptr_t b, unsigned voff, unsigned soff, T v) {
+  typedef __attribute__((address_space(1))) T* ptr_t;
+  gptr_t q = b + static_cast<uint64_t>(uni(soff));
+  asm("" : "+s"(q), "+v"(voff));
+  __builtin_nontemporal_store(v, (ptr_t)(q + static_cast<uint64_t>(voff)));
+}
+template <class T>
+TTT_DEV T g_ld_stream(gptr_t b, unsigned voff, unsigned soff) {
+  typedef const __attribute__((address_space(1))) T* ptr_t;
+  gptr_t q = b + static_cast<uint64_t>(uni(soff));
+  asm("" : "+s"(q), "+v"(voff));
+  return __builtin_nontemporal_load((ptr_t)(q + static_cast<uint64_t>(voff)));
+}
 TTT_DEV u32x4 g_ld16(gptr_t b, unsigned voff, unsigned soff) { return g_ld<u32x4>(b, voff, soff); }
 TTT_DEV void g_st16(gptr_t b, unsigned voff, unsigned soff, u32x4 v) { g_st<u32x4>(b, voff, soff, v); }
 TTT_DEV bf16x8 g_ld8h(gptr_t b, unsigned voff, unsigned soff) { return g_ld<bf16x8>(b, voff, soff); }

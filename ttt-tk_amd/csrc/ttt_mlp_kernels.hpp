@@ -52,6 +52,7 @@ struct BwdParams {
   __bf16 *alt_grad_l_wrt_Z2_group[3], *alt_grad_l_wrt_Z1_group[3];
   __bf16 *alt_x_hat_fused_group[3], *alt_grad_x_hat_fused_group[3], *alt_grad_output_fused_group[3];
   float* alt_std_fused_group[3];
+  float* alt_W1_init_group[3];
   float* norm_partial;   // [B*NH][2][8 waves][2][64]: the replay's share of the norm-weight / norm-bias gradients, by group parity
   float* norm_park;      // [B*NH][8 waves][2][64]: n_replay = 1: the share of the parity that is not being added to
   int n_replay;
