@@ -428,11 +428,11 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
       const OpdT<1, 4> w1A = cvt_chain(W1s);
       const OpdT<2, 2> w2A = cvt_chain(W2s);
 #pragma unroll
-      for (int s = 0; s < 4; s++) g_st8h(gImg, 16 * tid, s * 8192, w1A.v[0][s]);
+      for (int s = 0; s < 4; s++) g_st_stream<bf16x8>(gImg, 16 * tid, s * 8192, w1A.v[0][s]);   // read once, by another CU
 #pragma unroll
       for (int fb = 0; fb < 2; fb++)
 #pragma unroll
-        for (int s = 0; s < 2; s++) g_st8h(gImg, 16 * tid, (4 + 2 * fb + s) * 8192, w2A.v[fb][s]);
+        for (int s = 0; s < 2; s++) g_st_stream<bf16x8>(gImg, 16 * tid, (4 + 2 * fb + s) * 8192, w2A.v[fb][s]);
       if (h == 0) gB[hid0 + c] = b1L;
       if (mb % FWD_RING == FWD_RING - 1 || mb == p.NC - 1) publish(w_given, grp + 1);
       // No barrier ends a mini-batch here: every LDS buffer written from now on was last read before a
@@ -538,11 +538,11 @@ TTT_DEV void fwd_output_branch(const FwdParams& p, unsigned char* smem, const in
       OpdT<1, 4> w1A;
       OpdT<2, 2> w2A;
 #pragma unroll
-      for (int s = 0; s < 4; s++) w1A.v[0][s] = g_ld8h(gImg, 16 * tid, s * 8192);
+      for (int s = 0; s < 4; s++) w1A.v[0][s] = g_ld_stream<bf16x8>(gImg, 16 * tid, s * 8192);
 #pragma unroll
       for (int fb = 0; fb < 2; fb++)
 #pragma unroll
-        for (int s = 0; s < 2; s++) w2A.v[fb][s] = g_ld8h(gImg, 16 * tid, (4 + 2 * fb + s) * 8192);
+        for (int s = 0; s < 2; s++) w2A.v[fb][s] = g_ld_stream<bf16x8>(gImg, 16 * tid, (4 + 2 * fb + s) * 8192);
       const OpdT<2, 4> xqB = lds_rows_kappa<2, 4>(s_xq, FLD, c, h);
       AccT<1, 2> z1b;
 #pragma unroll
