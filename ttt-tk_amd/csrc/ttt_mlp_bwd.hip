@@ -782,7 +782,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
 #pragma unroll
             for (int e = 0; e < 8; e++) z[e] += b2v[e];
           }
-          ln_cvt8(gO, g_ld8h(bGO, vln, mb * TILE_BYTES));
+          ln_cvt8(gO, g_ld_stream<bf16x8>(bGO, vln, mb * TILE_BYTES));
           float sd;
           ln_normalize(z, &sd);   // z = x_hat
           ln_load_f32(gam, s_gam + f0);
@@ -837,10 +837,10 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           LANE_VARS;
           float z[8];
           ln_gather(z, s_lnrow);
-          bf16x8 dxq_old = g_ld8h(bDXQ, vln, mb * TILE_BYTES);
+          bf16x8 dxq_old = g_ld_stream<bf16x8>(bDXQ, vln, mb * TILE_BYTES);
 #pragma unroll
           for (int e = 0; e < 8; e++) dxq_old[e] = (bf16)((float)dxq_old[e] + (z[e] + gO[e]));
-          g_st8h(bDXQ, vln, mb * TILE_BYTES, dxq_old);
+          g_st_stream<bf16x8>(bDXQ, vln, mb * TILE_BYTES, dxq_old);
         }
       }
       if constexpr (ROLE == 1) {
@@ -1031,7 +1031,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         LANE_VARS;
         float gy[8];
         float gg[8], xh[8], go[8], gz[8], gam[8], gb[8];
-        dxv_old = g_ld8h(bDXV, vln, xo);
+        dxv_old = g_ld_stream<bf16x8>(bDXV, vln, xo);
         deta_old = g_ldh(bDETA, 2 * tok, mb * (CS * 2));
         const bf16x8 xhf = ROLE != 0 ? g_ld_stream<bf16x8>(bXHF, vln, so) : g_ld8h(bXHF, vln, so);
         const bf16x8 gof = ROLE != 0 ? g_ld_stream<bf16x8>(bGOF, vln, so) : g_ld8h(bGOF, vln, so);
@@ -1088,7 +1088,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           *reinterpret_cast<f32x4*>(s_gy + 4) = hi;
         }
         ln_store(s_a + tok * LDX + f0, gx);
-        g_st8h(bDXV, vln, xo, dxv_old);
+        g_st_stream<bf16x8>(bDXV, vln, xo, dxv_old);
       }
       __syncthreads();  // dZ2 tile complete; regions (T1 / T2) free again
 
@@ -1178,10 +1178,10 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         float z[8], gyv[8];
         ln_gather(z, s_lnrow);
         ln_load_f32(gyv, s_gy);
-        dxk_old = g_ld8h(bDXK, vln, xo);
+        dxk_old = g_ld_stream<bf16x8>(bDXK, vln, xo);
 #pragma unroll
         for (int e = 0; e < 8; e++) dxk_old[e] = (bf16)((float)dxk_old[e] + (z[e] + gyv[e]));
-        g_st8h(bDXK, vln, xo, dxk_old);
+        g_st_stream<bf16x8>(bDXK, vln, xo, dxk_old);
       }
     }
     if constexpr (ROLE == 2) publish(w_walked, done + 1);
