@@ -495,6 +495,9 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
   // Several workgroups per (batch, head): slot j of W1_init_group (of the set) carries gelu'(Z1) and gelu''(Z1)
   // of mini-batch j as two register images, and Z1_group carries gelu(Z1) instead of Z1.
 #define bDD gbuf(GRP(W1_init_group) + opk)
+  // the walk's fourth parked image (-eta * (XK gW1 + gb1) * gelu'(Z1)): second half of slot 0 of W1_init_group,
+  // or - where that tensor carries GELU images - the workspace
+#define bPUH (ROLE == 0 ? gbuf(ka->W1_init_group + opk) + IMG_BYTES : gbuf(ka->walk_park + (size_t)bh * (CS * HID)))
 #define bPW1 gbuf(ka->W1_init_group + opk)
 #define bPW2 gbuf(ka->W2_init_group + opk)
   constexpr unsigned PARK_D1 = 0, PARK_T2 = IMG_BYTES, PARK_G1 = 0;   // d1 in bPW1 (one workgroup only); g1, t2 in bPW2
@@ -982,7 +985,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           }
 #pragma unroll
           for (int t = 0; t < 2; t++) {
-            bf16x8 t2c, g1c;
+            bf16x8 t2c, g1c, uhc;
 #pragma unroll
             for (int jj = 0; jj < 8; jj++) {
               const float a = (float)ac[t][jj], b = (float)bc[t][jj];
@@ -990,9 +993,11 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
               const float gz1 = r0 * a;                                   // dl/dZ1
               de[i] = __builtin_fmaf(gz1, sv, de[i]);
               uc[t][jj] = (bf16)(sv * a);
+              uhc[jj] = (bf16)(-eta_i[i] * sv * a);
               g1c[jj] = (bf16)(-eta_i[i] * gz1);
               t2c[jj] = (bf16)(-eta_i[i] * r0 * sv * b);
             }
+            chunk_store(bPUH, 0, 2 * tb[i] + t, t16, uhc);
             // nothing stays in registers across the LayerNorm stage: g1 and t2 (and, without the images,
             // gelu'(Z1)) go to their parks at once (L2-resident, rewritten every mini-batch)
             if constexpr (ROLE == 0) chunk_store(bPW1, PARK_D1, 2 * tb[i] + t, t16, ac[t]);
@@ -1099,8 +1104,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         bf16x8 w2b[4];   // W2 before the step: lane = hid, contraction = F
 #pragma unroll
         for (int s = 0; s < 4; s++) w2b[s] = w2_before(bIMG2, bCW2, ckW, j, s, hid0, c, h, t16);
-        // T2 = gW1 rows [hid][F] (for S again and for gW1 G1^T), T1 = gW2 rows [F][hid] (transposed
-        // read gives lane = hid)
+        // T2 = gW1 rows [hid][F] (for gW1 G1^T), T1 = gW2 rows [F][hid] (transposed read gives lane = hid)
         store_state_rows<LDF>(T2, gW1s, c, h);
         store_state_rows<LDH>(T1, gW2s, c, h);
         WAVE_SYNC();
@@ -1109,11 +1113,8 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         bf16x8 dzp[2][2], uhp[2][2];
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-          AccT<1, 1> S, dx2;
-          acc_init_rows_lds(S, s_gb1w, h);
+          AccT<1, 1> dx2;
           acc_zero(dx2);
-          mma_jit<4>(S, [&](int, int s) { return piece_rows<LDF>(T2, 0, s, c, h); },
-                     [&](int, int s) { return piece_rows<LDX>(s_xk, tb[i], s, c, h); });
           mma_jit<4>(dx2, [&](int, int s) { return piece_tr<LDH>(T1, 0, s, lane); },           // gW2: lane = hid, contraction = F
                      [&](int, int s) { return piece_rows<LDX>(s_gz2, tb[i], s, c, h); });      // P2 = gZ2 gW2^T
 #pragma unroll
@@ -1142,8 +1143,9 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
             for (int jj = 0; jj < 8; jj++) {
               const float d1v = (float)d1c[t][jj];
               dzp[i][t][jj] = (bf16)__builtin_fmaf(dx2.b[0][0][8 * t + jj], d1v, (float)t2c[t][jj]);
-              uhp[i][t][jj] = (bf16)(-eta_i[i] * S.b[0][0][8 * t + jj] * d1v);
             }
+          uhp[i][0] = chunk_load(bPUH, 0, 2 * tb[i], t16);       // -eta * S * gelu', formed with S two stages back
+          uhp[i][1] = chunk_load(bPUH, 0, 2 * tb[i] + 1, t16);
         }
         bf16x8 w1bf[2][2];   // W1^T before the step (lane = F, contraction = hid), for the product after the next fence
 #pragma unroll
@@ -1232,6 +1234,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
 #undef bGZ2
 #undef bSDF
 #undef bDD
+#undef bPUH
 #undef bPW1
 #undef bPW2
 #undef bCW1

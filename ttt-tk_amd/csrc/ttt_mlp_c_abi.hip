@@ -146,7 +146,7 @@ LaunchPlan plan_launches(long long BH, bool after_full_rounds, bool three_way) {
 // 256-byte aligned.
 struct BwdWorkspace {
   static constexpr int PER_SET = 11;
-  static constexpr int PARTS = 3 + PER_SET * 3;
+  static constexpr int PARTS = 4 + PER_SET * 3;
   size_t off[PARTS];
   size_t total;
   BwdWorkspace(long long n, long long cgs, int alt_sets) {
@@ -162,8 +162,9 @@ struct BwdWorkspace {
     put(0, ttt::bwd_sync_ints(n) * sizeof(int));
     put(1, 2 * norm);
     put(2, norm);
+    put(3, (size_t)n * img);
     for (int s = 0; s < 3; s++)
-      for (int t = 0; t < PER_SET; t++) put(3 + PER_SET * s + t, s < alt_sets ? per_set[t] : 0);
+      for (int t = 0; t < PER_SET; t++) put(4 + PER_SET * s + t, s < alt_sets ? per_set[t] : 0);
     total = o;
   }
 };
@@ -232,8 +233,9 @@ extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* wo
   p.sync = words - b0 * ttt::BWD_SYNC_STRIDE;
   p.norm_partial = reinterpret_cast<float*>(base + w.off[1]) - b0 * 2 * norm;
   p.norm_park = reinterpret_cast<float*>(base + w.off[2]) - b0 * norm;
+  p.walk_park = reinterpret_cast<__bf16*>(base + w.off[3]) - b0 * (TTT_MLP_CS * TTT_MLP_HID);
   for (int s = 0; s < alt_sets; s++) {
-    const size_t* o = w.off + 3 + BwdWorkspace::PER_SET * s;
+    const size_t* o = w.off + 4 + BwdWorkspace::PER_SET * s;
     p.alt_X2_group[s] = reinterpret_cast<__bf16*>(base + o[0]) - b0 * img;
     p.alt_Z1_group[s] = reinterpret_cast<__bf16*>(base + o[1]) - b0 * img;
     p.alt_Z1_bar_group[s] = reinterpret_cast<__bf16*>(base + o[2]) - b0 * img;

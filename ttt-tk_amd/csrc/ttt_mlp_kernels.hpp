@@ -55,6 +55,7 @@ struct BwdParams {
   float* alt_W1_init_group[3];
   float* norm_partial;   // [B*NH][2][8 waves][2][64]: the replay's share of the norm-weight / norm-bias gradients, by group parity
   float* norm_park;      // [B*NH][8 waves][2][64]: n_replay = 1: the share of the parity that is not being added to
+  __bf16* walk_park;     // [B*NH][64][256]: one register image the walking workgroup parks across its LayerNorm stage
   int n_replay;
   int* sync;
   int* status;    // the status word behind the synchronisation words
