@@ -771,6 +771,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         // ---- the output branch, backwards: it needs the state after this step, which is in registers
         //      right now, and nothing of the running gradients.  Output LayerNorm forward and backward:
         float gO[8];
+        bf16x8 dxq_old;
         {
           LANE_VARS;
           // Every reader of this mini-batch's XQ / XK / XV tiles is past the barriers of the pair sum: the
@@ -834,13 +835,16 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
             image_store<ROLE != 0>(bGZ1B, j * IMG_BYTES, s, t16, piece_tr<LDH>(T1, 0, s, lane));
           }
           WAVE_SYNC();   // every reader of T1 / T2 is done before the pair sum takes their place
+          {
+            LANE_VARS;
+            dxq_old = g_ld_stream<bf16x8>(bDXQ, vln, mb * TILE_BYTES);   // under way during the pair sum
+          }
           pair_sum(s_own, s_partner, dq, c, h);
         }
         {
           LANE_VARS;
           float z[8];
           ln_gather(z, s_lnrow);
-          bf16x8 dxq_old = g_ld_stream<bf16x8>(bDXQ, vln, mb * TILE_BYTES);
 #pragma unroll
           for (int e = 0; e < 8; e++) dxq_old[e] = (bf16)((float)dxq_old[e] + (z[e] + gO[e]));
           g_st_stream<bf16x8>(bDXQ, vln, mb * TILE_BYTES, dxq_old);
@@ -939,6 +943,8 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
       //      t2 = -eta * (gZ2 W2^T) * (XK gW1 + gb1) * gelu''(Z1).
       bf16x8 dxv_old;            // LayerNorm lanes: the two outputs the stage accumulates into
       bf16 deta_old;
+      bf16x8 xhf_n, gof_n;       // and the saved x_hat, grad_output, std of the fused LayerNorm
+      float sdf_n;
       {
         LANE_VARS;
         // T1 = W2 before the step, rows [hid][F]; T2 = gW1, rows [hid][F]
@@ -1027,6 +1033,14 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           if (h == 0) s_deta[v * CS + 32 * tb[i] + c] = a;
         }
         WAVE_SYNC();   // this wave's readers of T1 / T2 are done
+        {   // what the LayerNorm stage reads from HBM is under way during the pair sum
+          LANE_VARS;
+          dxv_old = g_ld_stream<bf16x8>(bDXV, vln, xo);
+          deta_old = g_ldh(bDETA, 2 * tok, mb * (CS * 2));
+          xhf_n = ROLE != 0 ? g_ld_stream<bf16x8>(bXHF, vln, so) : g_ld8h(bXHF, vln, so);
+          gof_n = ROLE != 0 ? g_ld_stream<bf16x8>(bGOF, vln, so) : g_ld8h(bGOF, vln, so);
+          sdf_n = g_ldf(bSDF, vtok, j * (CS * 4));
+        }
         pair_sum(s_own, s_partner, pz, c, h);
       }
       // all pair sums of ggZ2 and the dEta partial sums are in LDS
@@ -1036,11 +1050,8 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         LANE_VARS;
         float gy[8];
         float gg[8], xh[8], go[8], gz[8], gam[8], gb[8];
-        dxv_old = g_ld_stream<bf16x8>(bDXV, vln, xo);
-        deta_old = g_ldh(bDETA, 2 * tok, mb * (CS * 2));
-        const bf16x8 xhf = ROLE != 0 ? g_ld_stream<bf16x8>(bXHF, vln, so) : g_ld8h(bXHF, vln, so);
-        const bf16x8 gof = ROLE != 0 ? g_ld_stream<bf16x8>(bGOF, vln, so) : g_ld8h(bGOF, vln, so);
-        const float sdf = g_ldf(bSDF, vtok, j * (CS * 4));
+        const bf16x8 xhf = xhf_n, gof = gof_n;
+        const float sdf = sdf_n;
         ln_gather(gg, s_lnrow);
         ln_load_f32(gb, s_gb2 + f0);
         const float neg_eta = -s_eta[tok];
@@ -1172,6 +1183,10 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
                    [&](int, int s) { return piece_tr<LDH>(T1, 0, s, lane); });                 // dZ1: lane = hid
         lds_rowsum_add_jit(s_gb1w, [&](int s) { return piece_tr<LDH>(T1, 0, s, lane); }, ones, c, h);
         WAVE_SYNC();   // this wave's readers of T1 / T2 are done
+        {
+          LANE_VARS;
+          dxk_old = g_ld_stream<bf16x8>(bDXK, vln, xo);   // under way during the pair sum
+        }
         pair_sum(s_own, s_partner, dk, c, h);
       }
       // pair sums of dXK complete
@@ -1180,7 +1195,6 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         float z[8], gyv[8];
         ln_gather(z, s_lnrow);
         ln_load_f32(gyv, s_gy);
-        dxk_old = g_ld_stream<bf16x8>(bDXK, vln, xo);
 #pragma unroll
         for (int e = 0; e < 8; e++) dxk_old[e] = (bf16)((float)dxk_old[e] + (z[e] + gyv[e]));
         g_st_stream<bf16x8>(bDXK, vln, xo, dxk_old);
