@@ -807,6 +807,11 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         __syncthreads();
         {
           LANE_VARS;
+          bf16x8 w1a[2][2];   // W1 after the step (lane = F, contraction = hid): the image stored above, fetched ahead of its use
+#pragma unroll
+          for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+            for (int s = 0; s < 2; s++) w1a[rb][s] = chunk_load(bIMG1, j * IMG_BYTES, 2 * rb + s, t16);
           {
             LANE_VARS;
             AccT<1, 2> gz1b;   // (gZ2_bar W2^T) * gelu'(Z1_bar): rows hid, lane = tok
@@ -826,7 +831,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           WAVE_SYNC();
           AccT<2, 2> dq;
           acc_zero(dq);
-          mma_jit<2>(dq, [&](int rb, int s) { return chunk_load(bIMG1, j * IMG_BYTES, 2 * rb + s, t16); },   // W1 after: lane = F
+          mma_jit<2>(dq, [&](int rb, int s) { return w1a[rb][s]; },                                // W1 after: lane = F
                      [&](int i, int s) { return piece_rows<LDH>(T1, tb[i], s, c, h); });                   // gZ1_bar: lane = tok
           // what the reverse walk adds to the running gradients, as ready-made operands (lane = hid, contraction = tok)
 #pragma unroll
@@ -903,20 +908,23 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         lds_put16(s_a, tid, gzb);
         if (tid < CS) s_eta[tid] = eta;
       }
-      __syncthreads();
-
       // ---- what the output branch adds to the running gradients.  The replay has taken that branch
       //      backwards already and left gZ2_bar (now in LDS) and X2_bar^T, gZ1_bar^T as operand images.
-      bf16x8 w2bf[4];   // W2 before this step (lane = hid, contraction = F): fetched now, needed by the next stage
-      bf16x8 gq[2][2], aq[2][2], bq[2][2];
+      bf16x8 x2b[4], g1b[4];   // lane = hid, contraction = tok; under way across the barrier
       {
         LANE_VARS;
-        bf16x8 x2b[4], g1b[4];   // lane = hid, contraction = tok
 #pragma unroll
         for (int s = 0; s < 4; s++) {
           x2b[s] = image_load<ROLE != 0>(bX2B, ho, s, t16);
           g1b[s] = image_load<ROLE != 0>(bGZ1B, ho, s, t16);
         }
+      }
+      __syncthreads();
+
+      bf16x8 w2bf[4];   // W2 before this step (lane = hid, contraction = F): fetched now, needed by the next stage
+      bf16x8 gq[2][2], aq[2][2], bq[2][2];
+      {
+        LANE_VARS;
 #pragma unroll
         for (int s = 0; s < 4; s++) w2bf[s] = w2_before(bIMG2, bCW2, ckW, j, s, hid0, c, h, t16);
         if constexpr (ROLE == 2) {   // the three GELU images of the next stage, under way during this one
