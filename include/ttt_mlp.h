@@ -130,22 +130,23 @@ int ttt_mlp_fwd_launch(const ttt_mlp_fwd_args* args, void* stream);
 /* Same for the remat backward. */
 int ttt_mlp_bwd_launch(const ttt_mlp_bwd_args* args, void* stream);
 
-/* The same backward (bit-identical results) with two workgroups per (batch, head)
- * where the device has CUs to spare: one recomputes checkpoint group after
- * checkpoint group, the other walks each recomputed group backwards, so
- * recomputation leaves the critical path.  The reference launcher
+/* The same backward (bit-identical results) with two or three workgroups per
+ * (batch, head) where the device has CUs to spare: one or two recompute checkpoint
+ * group after checkpoint group, the last one walks each recomputed group
+ * backwards, so recomputation leaves the critical path.  The reference launcher
  * (kernels/ttt_backward/ttt.cu:1451-1917) has no counterpart: it spreads one
  * (batch, head) over a cluster of four thread blocks instead.
- * Two workgroups that wait for each other must be resident together (one per CU),
+ * Workgroups that wait for each other must be resident together (one per CU),
  * so the pairs are covered by up to two launches in a row: the largest multiple
  * of the CU count with one workgroup per pair, then the remaining n pairs with
- * two each - provided 2*n fits the CUs.  ttt_mlp_bwd_workspace_bytes() returns 0
- * when it does not (n = 0 or 2*n > CUs of the current device); the launcher then
- * returns TTT_MLP_ERR_NO_ROOM and the caller uses ttt_mlp_bwd_launch.
+ * three each if 3*n fits the CUs, else two each if 2*n fits.
+ * ttt_mlp_bwd_workspace_bytes() returns 0 when neither does (n = 0 or 2*n > CUs of
+ * the current device); the launcher then returns TTT_MLP_ERR_NO_ROOM and the caller
+ * uses ttt_mlp_bwd_launch.
  * The caller owns the device workspace (256-byte aligned, contents unspecified
  * before and after; calls that overlap in time need separate workspaces).  The int
  * at index n*32 of the workspace is a status word: once the stream has drained
- * it reads non-zero only if a workgroup waited 20 s for the other and gave up, in
+ * it reads non-zero only if a workgroup waited 20 s for another and gave up, in
  * which case the outputs are invalid. */
 size_t ttt_mlp_bwd_workspace_bytes(int32_t B, int32_t NH, int32_t checkpoint_group_size);
 
