@@ -149,6 +149,8 @@ int ttt_mlp_bwd_launch(const ttt_mlp_bwd_args* args, void* stream);
  * it reads non-zero only if a workgroup waited 20 s for another and gave up, in
  * which case the outputs are invalid. */
 size_t ttt_mlp_bwd_workspace_bytes(int32_t B, int32_t NH, int32_t checkpoint_group_size);
+/* Byte offset of that status word (an int) inside the workspace; 0 when the mode does not apply. */
+size_t ttt_mlp_bwd_status_offset(int32_t B, int32_t NH);
 
 /* The forward with two workgroups per (batch, head), under the same conditions and with the same
  * conventions (launches, workspace, status word at int index n*32, TTT_MLP_ERR_NO_ROOM, bit-identical
@@ -158,6 +160,7 @@ size_t ttt_mlp_bwd_workspace_bytes(int32_t B, int32_t NH, int32_t checkpoint_gro
  * forward gains nothing from it.
  * No counterpart in the reference launcher (kernels/ttt/ttt.cu:594-721). */
 size_t ttt_mlp_fwd_workspace_bytes(int32_t B, int32_t NH);
+size_t ttt_mlp_fwd_status_offset(int32_t B, int32_t NH);
 int ttt_mlp_fwd_launch_overlapped(const ttt_mlp_fwd_args* args, void* workspace, size_t workspace_bytes, void* stream);
 int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* args, void* workspace, size_t workspace_bytes, void* stream);
 

@@ -63,7 +63,10 @@ def test_overlapped_launchers_through_ctypes(B, NH, NC, cgs):
                 assert launch(ctypes.byref(a), None, ctypes.c_size_t(nbytes), stream) == 1001
                 assert launch(ctypes.byref(a), ctypes.c_void_p(base), ctypes.c_size_t(nbytes), stream) == 0
                 torch.cuda.synchronize()
-                status = ws[base - ws.data_ptr():].view(torch.int32)[B * NH * 32].item()
+                off_fn = getattr(lib, f"ttt_mlp_{which}_status_offset")
+                off_fn.restype = ctypes.c_size_t
+                assert off_fn(B, NH) == B * NH * 32 * 4
+                status = ws[base - ws.data_ptr():].view(torch.int32)[off_fn(B, NH) // 4].item()
                 assert status == 0, "a workgroup gave up waiting for the other"
         torch.cuda.synchronize()
         results.append({k: t[k].float().cpu() for k in ("Out", "W1_checkpoints", "b2_checkpoints") + host.GRAD_NAMES})

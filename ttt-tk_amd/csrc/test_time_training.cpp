@@ -40,11 +40,20 @@ void check_eta(const torch::Tensor& t, const char* name, int64_t B, int64_t NH, 
 const uint16_t* bfp(const torch::Tensor& t) { return reinterpret_cast<const uint16_t*>(t.data_ptr<at::BFloat16>()); }
 uint16_t* bfp_mut(const torch::Tensor& t) { return reinterpret_cast<uint16_t*>(t.data_ptr<at::BFloat16>()); }
 
-void finish(int rc, hipStream_t stream, const char* what) {
+// `status` (may be null): device address of the status word of a launch with several workgroups per
+// (batch, head); it can only be looked at when the host waits for the stream anyway.
+void finish(int rc, hipStream_t stream, const char* what, const void* status = nullptr) {
   TORCH_CHECK(rc == TTT_MLP_OK, what, " launch failed: ", ttt_mlp_error_string(rc));
   if (g_synchronize) {
     hipError_t e = hipStreamSynchronize(stream);
     TORCH_CHECK(e == hipSuccess, what, " execution failed: ", hipGetErrorString(e));
+    if (status != nullptr) {
+      int word = 0;
+      e = hipMemcpy(&word, status, sizeof(int), hipMemcpyDeviceToHost);
+      TORCH_CHECK(e == hipSuccess, what, " execution failed: ", hipGetErrorString(e));
+      TORCH_CHECK(word == 0, what, ": a workgroup waited 20 s for its partner and gave up (were all compute units "
+                  "available to this launch?); the outputs are invalid - set_overlap(False) avoids the mode");
+    }
   }
 }
 
@@ -97,7 +106,8 @@ torch::Tensor ttt_forward(const torch::Tensor XQ, const torch::Tensor XK, const 
   if (ws_bytes > 0) {
     torch::Tensor ws = torch::empty({(int64_t)ws_bytes}, torch::TensorOptions().dtype(torch::kUInt8).device(XQ.device()));
     g_last_forward_mode = 1;
-    finish(ttt_mlp_fwd_launch_overlapped(&a, ws.data_ptr(), ws_bytes, stream), stream, "ttt_forward");
+    const char* status = static_cast<const char*>(ws.data_ptr()) + ttt_mlp_fwd_status_offset((int32_t)B, (int32_t)NH);
+    finish(ttt_mlp_fwd_launch_overlapped(&a, ws.data_ptr(), ws_bytes, stream), stream, "ttt_forward", status);
   } else {
     g_last_forward_mode = 0;
     finish(ttt_mlp_fwd_launch(&a, stream), stream, "ttt_forward");
@@ -208,7 +218,8 @@ torch::Tensor ttt_backward(
   if (ws_bytes > 0) {
     torch::Tensor ws = torch::empty({(int64_t)ws_bytes}, torch::TensorOptions().dtype(torch::kUInt8).device(XQ.device()));
     g_last_backward_mode = 1;
-    finish(ttt_mlp_bwd_launch_overlapped(&a, ws.data_ptr(), ws_bytes, stream), stream, "ttt_backward");
+    const char* status = static_cast<const char*>(ws.data_ptr()) + ttt_mlp_bwd_status_offset((int32_t)B, (int32_t)NH);
+    finish(ttt_mlp_bwd_launch_overlapped(&a, ws.data_ptr(), ws_bytes, stream), stream, "ttt_backward", status);
   } else {
     g_last_backward_mode = 0;
     finish(ttt_mlp_bwd_launch(&a, stream), stream, "ttt_backward");

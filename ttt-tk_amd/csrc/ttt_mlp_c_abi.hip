@@ -206,6 +206,12 @@ extern "C" size_t ttt_mlp_bwd_workspace_bytes(int B, int NH, int checkpoint_grou
   return pl.rest_split ? BwdWorkspace(pl.n_rest, checkpoint_group_size, 2 * (pl.per_pair - 1) - 1).total : 0;
 }
 
+extern "C" size_t ttt_mlp_bwd_status_offset(int B, int NH) {
+  if (B <= 0 || NH <= 0) return 0;
+  const LaunchPlan pl = plan_launches((long long)B * NH, true, true);
+  return pl.rest_split ? (size_t)pl.n_rest * ttt::BWD_SYNC_STRIDE * sizeof(int) : 0;
+}
+
 extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* workspace, size_t workspace_bytes, void* stream) {
   ttt::BwdParams p;
   if (int rc = make_bwd_params(a, p)) return rc;
@@ -263,6 +269,12 @@ extern "C" size_t ttt_mlp_fwd_workspace_bytes(int B, int NH) {
   if (B <= 0 || NH <= 0) return 0;
   const LaunchPlan pl = plan_launches((long long)B * NH, false, false);
   return pl.rest_split ? FwdWorkspace(pl.n_rest).total : 0;
+}
+
+extern "C" size_t ttt_mlp_fwd_status_offset(int B, int NH) {
+  if (B <= 0 || NH <= 0) return 0;
+  const LaunchPlan pl = plan_launches((long long)B * NH, false, false);
+  return pl.rest_split ? (size_t)pl.n_rest * ttt::BWD_SYNC_STRIDE * sizeof(int) : 0;
 }
 
 extern "C" int ttt_mlp_fwd_launch_overlapped(const ttt_mlp_fwd_args* a, void* workspace, size_t workspace_bytes, void* stream) {
