@@ -400,8 +400,11 @@ TTT_DEV bf16x8 w1_before(gptr_t img, gptr_t ck, unsigned ck_off, int j, int rb, 
 // 100 MHz clock raises the status word and both workgroups leave, so every wave always exits.
 // ROLE 0: replay and reverse walk of every group in one workgroup; 1: replays only - every n_replay-th group,
 // starting with group number `turn` (counted from the end of the sequence); 2: the reverse walks only.
-template <int ROLE>
+// IMG (with two replaying workgroups): the replay has time to spare and evaluates gelu, gelu', gelu'' of the
+// rounded Z1 for the walk, which gets them as three images instead of the image of Z1.  Same values either way.
+template <int ROLE, bool IMG>
 TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, const int turn) {
+  static_assert(!(ROLE == 0 && IMG), "one workgroup per (batch, head) evaluates the GELU family in the walk");
   bf16* s_xq = reinterpret_cast<bf16*>(smem + SB_XQ);
   bf16* s_xk = reinterpret_cast<bf16*>(smem + SB_XK);
   bf16* s_gz2 = reinterpret_cast<bf16*>(smem + SB_GZ2);
@@ -620,7 +623,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
 #pragma unroll
             for (int t = 0; t < 2; t++) {
               const bf16x8 zr = pack8(x2.b[0][i], t);
-              if constexpr (ROLE == 0) {
+              if constexpr (!IMG) {
                 image_store<ROLE != 0>(bZ1, j * IMG_BYTES, 2 * tb[i] + t, t16, zr);
               } else {
                 // The walk needs gelu, gelu' and gelu'' of the ROUNDED Z1 (what it would compute from the image
@@ -928,7 +931,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         LANE_VARS;
 #pragma unroll
         for (int s = 0; s < 4; s++) w2bf[s] = w2_before(bIMG2, bCW2, ckW, j, s, hid0, c, h, t16);
-        if constexpr (ROLE == 2) {   // the three GELU images of the next stage, under way during this one
+        if constexpr (IMG) {   // the three GELU images of the next stage, under way during this one
 #pragma unroll
           for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -978,8 +981,8 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           // gelu(Z1), gelu'(Z1), gelu''(Z1), each rounded to bf16: computed here from the image of Z1, or
           // fetched as three images that a replaying workgroup computed the same way
           bf16x8 ac[2], bc[2];
-          if constexpr (ROLE == 0) {
-            const bf16x8 zc[2] = {chunk_load(bZ1, ho, 2 * tb[i], t16), chunk_load(bZ1, ho, 2 * tb[i] + 1, t16)};
+          if constexpr (!IMG) {
+            const bf16x8 zc[2] = {image_load<ROLE != 0>(bZ1, ho, 2 * tb[i], t16), image_load<ROLE != 0>(bZ1, ho, 2 * tb[i] + 1, t16)};
 #pragma unroll
             for (int t = 0; t < 2; t++)
 #pragma unroll
@@ -1015,7 +1018,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
             chunk_store(bPUH, 0, 2 * tb[i] + t, t16, uhc);
             // nothing stays in registers across the LayerNorm stage: g1 and t2 (and, without the images,
             // gelu'(Z1)) go to their parks at once (L2-resident, rewritten every mini-batch)
-            if constexpr (ROLE == 0) chunk_store(bPW1, PARK_D1, 2 * tb[i] + t, t16, ac[t]);
+            if constexpr (!IMG) chunk_store(bPW1, PARK_D1, 2 * tb[i] + t, t16, ac[t]);
             chunk_store(bPW2, PARK_T2, 2 * tb[i] + t, t16, t2c);
             chunk_store(bPW2, PARK_G1, 2 * tb[i] + t, t16, g1c);
             store_piece_rows<LDH>(T0, tb[i], t, c, h, x2c[t]);             // X2 rows [tok][hid]
@@ -1144,7 +1147,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           // dk[:, i] = gW1 G1^T  (gW1: lane = F, contraction = hid)
           const bf16x8 g1c[2] = {chunk_load(bPW2, PARK_G1, 2 * tb[i], t16), chunk_load(bPW2, PARK_G1, 2 * tb[i] + 1, t16)};
           bf16x8 d1c[2];
-          if constexpr (ROLE == 0) {
+          if constexpr (!IMG) {
             d1c[0] = chunk_load(bPW1, PARK_D1, 2 * tb[i], t16);
             d1c[1] = chunk_load(bPW1, PARK_D1, 2 * tb[i] + 1, t16);
           } else {
@@ -1269,7 +1272,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
 
 __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  bwd_body<0>(p, smem, p.bh0 + blockIdx.x, 0);
+  bwd_body<0, false>(p, smem, p.bh0 + blockIdx.x, 0);
 }
 
 // n_replay + 1 workgroups per (batch, head).  Workgroups are dealt to the 8 XCDs in turn, so with a multiple
@@ -1286,8 +1289,13 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_split_kernel(const Bwd
     role = b % per;
   }
   bh += p.bh0;
-  if (role < p.n_replay) bwd_body<1>(p, smem, bh, role);
-  else bwd_body<2>(p, smem, bh, 0);
+  if (p.n_replay == 2) {
+    if (role < 2) bwd_body<1, true>(p, smem, bh, role);
+    else bwd_body<2, true>(p, smem, bh, 0);
+  } else {
+    if (role < 1) bwd_body<1, false>(p, smem, bh, 0);
+    else bwd_body<2, false>(p, smem, bh, 0);
+  }
 }
 
 __global__ void ttt_mlp_zero_words(int* w, int n) {
