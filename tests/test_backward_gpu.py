@@ -152,8 +152,9 @@ def test_bit_reproducible_and_independent_of_workspace_contents(B, NH, NC, cgs):
     (1, 8, 24, 8),       # multiple of 8: the two workgroups of a pair are placed on one XCD
     (2, 8, 10, 5),       # two groups only
     (1, 4, 33, 2),       # seventeen groups
-    (2, 130, 5, 2),      # more pairs than CUs: 256 with one workgroup each, then the last 4 with three
-    (1, 96, 5, 2),       # too many pairs for three workgroups each: one replays all groups, one walks
+    (2, 130, 5, 2),      # more pairs than CUs: 256 with one workgroup each, then the last 4 with four
+    (1, 72, 5, 2),       # too many pairs for four workgroups each: two replay, one walks (and forms grad_L_XK itself)
+    (1, 96, 5, 2),       # too many pairs for three: one replays all groups, one walks
 ])
 def test_overlapped_backward_is_bit_identical(B, NH, NC, cgs):
     """Recomputing the groups on a second workgroup changes the schedule, not one bit of the results."""

@@ -402,9 +402,12 @@ TTT_DEV bf16x8 w1_before(gptr_t img, gptr_t ck, unsigned ck_off, int j, int rb, 
 // starting with group number `turn` (counted from the end of the sequence); 2: the reverse walks only.
 // IMG (with two replaying workgroups): the replay has time to spare and evaluates gelu, gelu', gelu'' of the
 // rounded Z1 for the walk, which gets them as three images instead of the image of Z1.  Same values either way.
-template <int ROLE, bool IMG>
+// FIN: grad_L_XK is a leaf of the walk - it needs the running gradients, but nothing needs it.  With a
+// fourth workgroup the walk hands over the operands of its two products (gW1, G1, dZ1 as register images)
+// and g_y, and that workgroup (bwd_finish_dxk) forms the products, their pair sum and the final sum.
+template <int ROLE, bool IMG, bool FIN>
 TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, const int turn) {
-  static_assert(!(ROLE == 0 && IMG), "one workgroup per (batch, head) evaluates the GELU family in the walk");
+  static_assert(!(ROLE == 0 && (IMG || FIN)), "one workgroup per (batch, head) does everything itself");
   bf16* s_xq = reinterpret_cast<bf16*>(smem + SB_XQ);
   bf16* s_xk = reinterpret_cast<bf16*>(smem + SB_XK);
   bf16* s_gz2 = reinterpret_cast<bf16*>(smem + SB_GZ2);
@@ -535,6 +538,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
   }
   int* const w_sync = p.sync + (size_t)bh * BWD_SYNC_STRIDE;   // + 0, + 8: groups replayed by workgroup 0 / 1
   int* const w_walked = w_sync + 16;
+  int* const w_finished = w_sync + 24;
   const int n_replay = ROLE == 0 ? 1 : p.n_replay, n_sets = 2 * n_replay;
   int* const w_status = p.status;
   int* const s_flag = reinterpret_cast<int*>(smem + SB_FLAG);
@@ -579,6 +583,9 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
     if constexpr (ROLE != 2) {
       if constexpr (ROLE == 1) {   // the set is free once the reverse walk is done with the group that used it last
         if (done >= n_sets && !wait_at_least(w_walked, done - n_sets + 1, w_status, s_flag)) return;
+        if constexpr (FIN) {   // ... and so is the workgroup that reads the before-state images for grad_L_XK
+          if (done >= n_sets && !wait_at_least(w_finished, done - n_sets + 1, w_status, s_flag)) return;
+        }
         // a single replaying workgroup adds to the sum of this group's parity: the groups alternate, so from
         // the second group on the live sum and the parked one change places
         if (n_replay == 1 && done > 0) norm_swap(0);
@@ -887,7 +894,16 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
     // than it gains (measured).
     if constexpr (ROLE == 2) {
       if (!wait_at_least(w_replayed, done / n_replay + 1, w_status, s_flag)) return;
+      if constexpr (FIN) {   // the hand-over set of this group's parity is free once the group before last is finished
+        if (done >= 2 && !wait_at_least(w_finished, done - 1, w_status, s_flag)) return;
+      }
     }
+    // hand-over buffers of this group for the grad_L_XK workgroup (set = parity of the group)
+    const size_t ofin = uni64(((size_t)bh * 2 + (done & 1)) * cgs);
+#define bFGW gbuf(ka->fin_gw1 + ofin * (CS * HID))
+#define bFG1 gbuf(ka->fin_g1 + ofin * (CS * HID))
+#define bFDZ gbuf(ka->fin_dz + ofin * (CS * HID))
+#define bFGY gbuf(ka->fin_gy + ofin * (CS * FD))
     if constexpr (ROLE != 1)
     for (int j = n_mb - 1; j >= 0; j--) {
       const int mb = k * cgs + j;
@@ -1020,7 +1036,8 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
             // gelu'(Z1)) go to their parks at once (L2-resident, rewritten every mini-batch)
             if constexpr (!IMG) chunk_store(bPW1, PARK_D1, 2 * tb[i] + t, t16, ac[t]);
             chunk_store(bPW2, PARK_T2, 2 * tb[i] + t, t16, t2c);
-            chunk_store(bPW2, PARK_G1, 2 * tb[i] + t, t16, g1c);
+            if constexpr (FIN) image_store<true>(bFG1, ho, 2 * tb[i] + t, t16, g1c);   // only grad_L_XK needs G1
+            else chunk_store(bPW2, PARK_G1, 2 * tb[i] + t, t16, g1c);
             store_piece_rows<LDH>(T0, tb[i], t, c, h, x2c[t]);             // X2 rows [tok][hid]
           }
           // pz[:, i] = gW2^T X2^T ; dEta partial ; + W2^T u^T
@@ -1108,12 +1125,17 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           gx[e] = gx[e] * rsd + (sg * xh[e] - sx * rsd) * (1.f / FD);   // dZ2
           dxv_old[e] = (bf16)((float)dxv_old[e] - gy[e]);                // dXV accumulates -g_y
         }
-        // g_y is needed again for dXK: park it (the XQ / E2 tiles are dead by now)
+        // g_y is needed again for dXK: park it (the XQ / E2 tiles are dead by now), or hand it over
         {
           LANE_VARS;
           f32x4 lo = {gy[0], gy[1], gy[2], gy[3]}, hi = {gy[4], gy[5], gy[6], gy[7]};
-          *reinterpret_cast<f32x4*>(s_gy) = lo;
-          *reinterpret_cast<f32x4*>(s_gy + 4) = hi;
+          if constexpr (FIN) {
+            g_st_stream<f32x4>(bFGY, 2 * vln, 2 * so, lo);
+            g_st_stream<f32x4>(bFGY, 2 * vln + 16, 2 * so, hi);
+          } else {
+            *reinterpret_cast<f32x4*>(s_gy) = lo;
+            *reinterpret_cast<f32x4*>(s_gy + 4) = hi;
+          }
         }
         ln_store(s_a + tok * LDX + f0, gx);
         g_st_stream<bf16x8>(bDXV, vln, xo, dxv_old);
@@ -1145,7 +1167,11 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           mma_jit<4>(dx2, [&](int, int s) { return w2b[s]; },                                  // + dZ2 W2^T
                      [&](int, int s) { return piece_rows<LDX>(s_a, tb[i], s, c, h); });
           // dk[:, i] = gW1 G1^T  (gW1: lane = F, contraction = hid)
-          const bf16x8 g1c[2] = {chunk_load(bPW2, PARK_G1, 2 * tb[i], t16), chunk_load(bPW2, PARK_G1, 2 * tb[i] + 1, t16)};
+          bf16x8 g1c[2];
+          if constexpr (!FIN) {
+            g1c[0] = chunk_load(bPW2, PARK_G1, 2 * tb[i], t16);
+            g1c[1] = chunk_load(bPW2, PARK_G1, 2 * tb[i] + 1, t16);
+          }
           bf16x8 d1c[2];
           if constexpr (!IMG) {
             d1c[0] = chunk_load(bPW1, PARK_D1, 2 * tb[i], t16);
@@ -1155,10 +1181,12 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
             d1c[1] = chunk_load(bDD, j * (2 * IMG_BYTES), 2 * tb[i] + 1, t16);
           }
           const bf16x8 t2c[2] = {chunk_load(bPW2, PARK_T2, 2 * tb[i], t16), chunk_load(bPW2, PARK_T2, 2 * tb[i] + 1, t16)};
+          if constexpr (!FIN) {
 #pragma unroll
-          for (int t = 0; t < 2; t++)
+            for (int t = 0; t < 2; t++)
 #pragma unroll
-            for (int rb = 0; rb < 2; rb++) dk.b[rb][i] = MFMA(piece_tr<LDF>(T2, rb, t, lane), g1c[t], dk.b[rb][i]);
+              for (int rb = 0; rb < 2; rb++) dk.b[rb][i] = MFMA(piece_tr<LDF>(T2, rb, t, lane), g1c[t], dk.b[rb][i]);
+          }
           // dZ1 = dX2*gelu' + t2 ;  -eta * S * gelu'   (kept as pieces until T1 / T2 may be overwritten)
 #pragma unroll
           for (int t = 0; t < 2; t++)
@@ -1171,10 +1199,21 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           uhp[i][1] = chunk_load(bPUH, 0, 2 * tb[i] + 1, t16);
         }
         bf16x8 w1bf[2][2];   // W1^T before the step (lane = F, contraction = hid), for the product after the next fence
+        if constexpr (!FIN) {
 #pragma unroll
-        for (int rb = 0; rb < 2; rb++)
+          for (int rb = 0; rb < 2; rb++)
 #pragma unroll
-          for (int s = 0; s < 2; s++) w1bf[rb][s] = w1_before(bIMG1, bCW1, ckW, j, rb, s, hid0, c, h, t16);
+            for (int s = 0; s < 2; s++) w1bf[rb][s] = w1_before(bIMG1, bCW1, ckW, j, rb, s, hid0, c, h, t16);
+        } else {   // gW1 as the operand of gW1 G1^T (lane = F, contraction = hid) and dZ1 leave for the other workgroup
+#pragma unroll
+          for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+            for (int t = 0; t < 2; t++) image_store<true>(bFGW, ho, 2 * rb + t, t16, piece_tr<LDF>(T2, rb, t, lane));
+#pragma unroll
+          for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int t = 0; t < 2; t++) image_store<true>(bFDZ, ho, 2 * tb[i] + t, t16, dzp[i][t]);
+        }
         WAVE_SYNC();   // S, P2 and gW1 G1^T have consumed T2 / T1
 #pragma unroll
         for (int i = 0; i < 2; i++)
@@ -1184,8 +1223,9 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
             store_piece_rows<LDH>(T2, tb[i], t, c, h, uhp[i][t]);   // -eta u rows [tok][hid]
           }
         WAVE_SYNC();
-        mma_jit<2>(dk, [&](int rb, int s) { return w1bf[rb][s]; },                             // + W1 dZ1^T, W1 before the step
-                   [&](int i, int s) { return dzp[i][s]; });
+        if constexpr (!FIN)
+          mma_jit<2>(dk, [&](int rb, int s) { return w1bf[rb][s]; },                           // + W1 dZ1^T, W1 before the step
+                     [&](int i, int s) { return dzp[i][s]; });
         mma_jit<4>(gW2s, [&](int, int s) { return piece_tr<LDH>(T2, 0, s, lane); },            // (-eta u)^T: lane = hid
                    [&](int fb, int s) { return piece_tr<LDX>(s_gz2, fb, s, lane); });          // gZ2: lane = F
         mma_jit<4>(gW2s, [&](int, int s) { return piece_tr<LDH>(T0, 0, s, lane); },            // X2^T: lane = hid
@@ -1195,14 +1235,16 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
                    [&](int, int s) { return piece_tr<LDH>(T1, 0, s, lane); });                 // dZ1: lane = hid
         lds_rowsum_add_jit(s_gb1w, [&](int s) { return piece_tr<LDH>(T1, 0, s, lane); }, ones, c, h);
         WAVE_SYNC();   // this wave's readers of T1 / T2 are done
-        {
-          LANE_VARS;
-          dxk_old = g_ld_stream<bf16x8>(bDXK, vln, xo);   // under way during the pair sum
+        if constexpr (!FIN) {
+          {
+            LANE_VARS;
+            dxk_old = g_ld_stream<bf16x8>(bDXK, vln, xo);   // under way during the pair sum
+          }
+          pair_sum(s_own, s_partner, dk, c, h);
         }
-        pair_sum(s_own, s_partner, dk, c, h);
       }
       // pair sums of dXK complete
-      {
+      if constexpr (!FIN) {
         LANE_VARS;
         float z[8], gyv[8];
         ln_gather(z, s_lnrow);
@@ -1213,6 +1255,10 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
       }
     }
     if constexpr (ROLE == 2) publish(w_walked, done + 1);
+#undef bFGW
+#undef bFG1
+#undef bFDZ
+#undef bFGY
   }
   if constexpr (ROLE == 1) return;
 
@@ -1272,14 +1318,83 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
 
 __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  bwd_body<0, false>(p, smem, p.bh0 + blockIdx.x, 0);
+  bwd_body<0, false, false>(p, smem, p.bh0 + blockIdx.x, 0);
 }
 
-// n_replay + 1 workgroups per (batch, head).  Workgroups are dealt to the 8 XCDs in turn, so with a multiple
-// of 8 (batch, head) pairs the workgroups of a pair are placed 8 apart: same XCD, same L2.
+// grad_L_XK on a workgroup of its own: for every mini-batch of every group, as soon as the walk is done with the
+// group, dk = gW1 G1^T + W1 dZ1^T (W1 before the step: from the replay's image, or the checkpoint), its sum over
+// the hidden dimension, + g_y, accumulated into grad_L_XK.  Same wave / lane roles and the same order of every
+// sum as in the walk, so the result is the same to the bit.
+TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int bh) {
+  float* s_P = reinterpret_cast<float*>(smem + SB_P);
+  const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5, c = lane & 31;
+  const int v = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int pp = v & 3, r = v >> 2;
+  const int tb[2] = {r, 1 - r};
+  const int q8 = lane >> 3, tok = 8 * v + q8, f0 = 8 * (lane & 7);
+  const int hid0 = BW_NS * v;
+  float* s_own = s_P + (pp * 2 + r) * (32 * LDR);
+  float* s_partner = s_P + (pp * 2 + (1 - r)) * (32 * LDR);
+  const float* s_lnrow = s_P + (1 - r) * (32 * LDR) + (tok & 31) * LDR + f0;
+  const int cgs = p.cgs, n_sets = 2 * p.n_replay;
+  const unsigned t16 = 16 * tid, vln = (tok * FD + f0) * 2;
+  int* const w_sync = p.sync + (size_t)bh * BWD_SYNC_STRIDE;
+  int* const w_walked = w_sync + 16;
+  int* const w_finished = w_sync + 24;
+  int* const s_flag = reinterpret_cast<int*>(smem + SB_FLAG);
+  const gptr_t gDXK = gbuf(p.grad_L_XK + uni64((size_t)bh * p.NC * (CS * FD)));
+  const gptr_t gCW1 = gbuf(p.W1_ck + uni64((size_t)bh * p.K * (FD * HID)));
+  for (int k = p.K - 1; k >= 0; k--) {
+    const int n_mb = min(cgs, p.NC - k * cgs);
+    const int done = p.K - 1 - k, set = done % n_sets;
+    if (!wait_at_least(w_walked, done + 1, p.status, s_flag)) return;
+    const size_t ofin = uni64(((size_t)bh * 2 + (done & 1)) * cgs);
+    const gptr_t gGW = gbuf(p.fin_gw1 + ofin * (CS * HID)), gG1 = gbuf(p.fin_g1 + ofin * (CS * HID));
+    const gptr_t gDZ = gbuf(p.fin_dz + ofin * (CS * HID)), gGY = gbuf(p.fin_gy + ofin * (CS * FD));
+    const gptr_t gIMG1 = gbuf((set ? p.alt_X2_group[set - 1] : p.X2_group) + uni64((size_t)bh * cgs * (CS * HID)));
+    const unsigned ckW = k * (FD * HID * 4);
+    for (int j = n_mb - 1; j >= 0; j--) {
+      const unsigned xo = (k * cgs + j) * TILE_BYTES, so = j * TILE_BYTES, ho = j * IMG_BYTES;
+      const bf16x8 dxk_ld = g_ld_stream<bf16x8>(gDXK, vln, xo);
+      const f32x4 gy_lo = g_ld_stream<f32x4>(gGY, 2 * vln, 2 * so), gy_hi = g_ld_stream<f32x4>(gGY, 2 * vln + 16, 2 * so);
+      bf16x8 gw[2][2], g1[2][2], dz[2][2], w1b[2][2];
+#pragma unroll
+      for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+          gw[a][t] = image_load<true>(gGW, ho, 2 * a + t, t16);
+          g1[a][t] = image_load<true>(gG1, ho, 2 * tb[a] + t, t16);
+          dz[a][t] = image_load<true>(gDZ, ho, 2 * tb[a] + t, t16);
+          w1b[a][t] = w1_before(gIMG1, gCW1, ckW, j, a, t, hid0, c, h, t16);
+        }
+      AccT<2, 2> dk;
+      acc_zero(dk);
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+          for (int rb = 0; rb < 2; rb++) dk.b[rb][i] = MFMA(gw[rb][t], g1[i][t], dk.b[rb][i]);
+      mma_jit<2>(dk, [&](int rb, int s) { return w1b[rb][s]; }, [&](int i, int s) { return dz[i][s]; });
+      pair_sum(s_own, s_partner, dk, c, h);
+      float z[8];
+      ln_gather(z, s_lnrow);
+      const float gyv[8] = {gy_lo[0], gy_lo[1], gy_lo[2], gy_lo[3], gy_hi[0], gy_hi[1], gy_hi[2], gy_hi[3]};
+      bf16x8 dxk_new;
+#pragma unroll
+      for (int e = 0; e < 8; e++) dxk_new[e] = (bf16)((float)dxk_ld[e] + (z[e] + gyv[e]));
+      g_st_stream<bf16x8>(gDXK, vln, xo, dxk_new);
+      __syncthreads();   // the readers of the pair sums are done before the next mini-batch's take their place
+    }
+    publish(w_finished, done + 1);
+  }
+}
+
+// n_replay + 1 (+ 1) workgroups per (batch, head).  Workgroups are dealt to the 8 XCDs in turn, so with a
+// multiple of 8 (batch, head) pairs the workgroups of a pair are placed 8 apart: same XCD, same L2.
 __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_split_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int b = blockIdx.x, per = p.n_replay + 1;
+  const int b = blockIdx.x, per = p.n_replay + 1 + p.n_finish;
   int bh, role;
   if (p.nbh % 8 == 0) {
     bh = (b / (8 * per)) * 8 + (b & 7);
@@ -1289,12 +1404,16 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_split_kernel(const Bwd
     role = b % per;
   }
   bh += p.bh0;
-  if (p.n_replay == 2) {
-    if (role < 2) bwd_body<1, true>(p, smem, bh, role);
-    else bwd_body<2, true>(p, smem, bh, 0);
+  if (p.n_finish) {   // two replay, one walks, one forms grad_L_XK
+    if (role < 2) bwd_body<1, true, true>(p, smem, bh, role);
+    else if (role == 2) bwd_body<2, true, true>(p, smem, bh, 0);
+    else bwd_finish_dxk(p, smem, bh);
+  } else if (p.n_replay == 2) {
+    if (role < 2) bwd_body<1, true, false>(p, smem, bh, role);
+    else bwd_body<2, true, false>(p, smem, bh, 0);
   } else {
-    if (role < 1) bwd_body<1, false>(p, smem, bh, 0);
-    else bwd_body<2, false>(p, smem, bh, 0);
+    if (role < 1) bwd_body<1, false, false>(p, smem, bh, 0);
+    else bwd_body<2, false, false>(p, smem, bh, 0);
   }
 }
 
@@ -1322,6 +1441,6 @@ hipError_t ttt_mlp_bwd_enqueue(const ttt::BwdParams& p, hipStream_t stream) {
   const int n = static_cast<int>(ttt::bwd_sync_ints(p.nbh));
   int* const words = p.status - (size_t)p.nbh * ttt::BWD_SYNC_STRIDE;   // p.sync itself is moved back by bh0 entries
   hipLaunchKernelGGL(ttt::ttt_mlp_zero_words, dim3((n + 255) / 256), dim3(256), 0, stream, words, n);
-  hipLaunchKernelGGL(ttt::ttt_mlp_bwd_split_kernel, dim3((p.n_replay + 1) * p.nbh), dim3(ttt::BW_THREADS), ttt::SM_BWD_BYTES, stream, p);
+  hipLaunchKernelGGL(ttt::ttt_mlp_bwd_split_kernel, dim3((p.n_replay + 1 + p.n_finish) * p.nbh), dim3(ttt::BW_THREADS), ttt::SM_BWD_BYTES, stream, p);
   return hipGetLastError();
 }

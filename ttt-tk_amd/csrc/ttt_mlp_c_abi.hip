@@ -120,7 +120,7 @@ struct LaunchPlan {
   long long n_single = 0;   // pairs 0 .. n_single-1: one workgroup each
   long long n_rest = 0;     // pairs n_single .. n_single+n_rest-1
   bool rest_split = false;
-  int per_pair = 1;         // workgroups per pair of the rest: 2, or 3 where the kernel can use them and they fit
+  int per_pair = 1;         // workgroups per pair of the rest: 2, or 3 / 4 where the kernel can use them and they fit
 };
 // `after_full_rounds`: whether the rest may be split when full rounds precede it.  That pays for the
 // backward; the forward's gain from splitting is smaller than what a full device costs it (measured).
@@ -136,7 +136,7 @@ LaunchPlan plan_launches(long long BH, bool after_full_rounds, bool three_way) {
   pl.n_rest = BH - pl.n_single;
   pl.rest_split = pl.n_rest > 0 && 2 * pl.n_rest <= cus && (after_full_rounds || pl.n_single == 0);
   if (!pl.rest_split) { pl.n_single = BH; pl.n_rest = 0; }
-  else pl.per_pair = (three_way && 3 * pl.n_rest <= cus) ? 3 : 2;
+  else pl.per_pair = !three_way ? 2 : 4 * pl.n_rest <= cus ? 4 : 3 * pl.n_rest <= cus ? 3 : 2;
   return pl;
 }
 
@@ -146,10 +146,10 @@ LaunchPlan plan_launches(long long BH, bool after_full_rounds, bool three_way) {
 // 256-byte aligned.
 struct BwdWorkspace {
   static constexpr int PER_SET = 11;
-  static constexpr int PARTS = 4 + PER_SET * 3;
+  static constexpr int PARTS = 8 + PER_SET * 3;
   size_t off[PARTS];
   size_t total;
-  BwdWorkspace(long long n, long long cgs, int alt_sets) {
+  BwdWorkspace(long long n, long long cgs, int alt_sets, bool finish) {
     const size_t slot = (size_t)n * (size_t)cgs;
     const size_t tile = TTT_MLP_CS * TTT_MLP_F * 2, img = TTT_MLP_CS * TTT_MLP_HID * 2, vec = TTT_MLP_CS * 4;
     const size_t norm = (size_t)n * 8 * 2 * TTT_MLP_F * sizeof(float);
@@ -163,8 +163,11 @@ struct BwdWorkspace {
     put(1, 2 * norm);
     put(2, norm);
     put(3, (size_t)n * img);
+    // hand-over to the grad_L_XK workgroup: three images and g_y (fp32) per slot, two sets
+    for (int t = 0; t < 3; t++) put(4 + t, finish ? 2 * slot * img : 0);
+    put(7, finish ? 2 * slot * 2 * tile : 0);
     for (int s = 0; s < 3; s++)
-      for (int t = 0; t < PER_SET; t++) put(4 + PER_SET * s + t, s < alt_sets ? per_set[t] : 0);
+      for (int t = 0; t < PER_SET; t++) put(8 + PER_SET * s + t, s < alt_sets ? per_set[t] : 0);
     total = o;
   }
 };
@@ -203,7 +206,9 @@ extern "C" int ttt_mlp_bwd_launch(const ttt_mlp_bwd_args* a, void* stream) {
 extern "C" size_t ttt_mlp_bwd_workspace_bytes(int B, int NH, int checkpoint_group_size) {
   if (B <= 0 || NH <= 0 || checkpoint_group_size <= 0 || checkpoint_group_size > (1 << 16)) return 0;
   const LaunchPlan pl = plan_launches((long long)B * NH, true, true);
-  return pl.rest_split ? BwdWorkspace(pl.n_rest, checkpoint_group_size, 2 * (pl.per_pair - 1) - 1).total : 0;
+  if (!pl.rest_split) return 0;
+  const int n_replay = pl.per_pair >= 3 ? 2 : 1;
+  return BwdWorkspace(pl.n_rest, checkpoint_group_size, 2 * n_replay - 1, pl.per_pair == 4).total;
 }
 
 extern "C" size_t ttt_mlp_bwd_status_offset(int B, int NH) {
@@ -218,8 +223,9 @@ extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* wo
   if (int rc = check_workspace(workspace)) return rc;
   const LaunchPlan pl = plan_launches((long long)p.B * p.NH, true, true);
   if (!pl.rest_split) return TTT_MLP_ERR_NO_ROOM;
-  const int n_replay = pl.per_pair - 1, alt_sets = 2 * n_replay - 1;
-  const BwdWorkspace w(pl.n_rest, p.cgs, alt_sets);
+  const int n_replay = pl.per_pair >= 3 ? 2 : 1, alt_sets = 2 * n_replay - 1;
+  const bool finish = pl.per_pair == 4;
+  const BwdWorkspace w(pl.n_rest, p.cgs, alt_sets, finish);
   if (workspace_bytes < w.total) return TTT_MLP_ERR_WORKSPACE;
   if (pl.n_single > 0) {
     p.bh0 = 0;
@@ -234,6 +240,13 @@ extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* wo
   p.bh0 = static_cast<int>(pl.n_single);
   p.nbh = static_cast<int>(pl.n_rest);
   p.n_replay = n_replay;
+  p.n_finish = finish ? 1 : 0;
+  if (finish) {
+    p.fin_gw1 = reinterpret_cast<__bf16*>(base + w.off[4]) - b0 * 2 * img;
+    p.fin_g1 = reinterpret_cast<__bf16*>(base + w.off[5]) - b0 * 2 * img;
+    p.fin_dz = reinterpret_cast<__bf16*>(base + w.off[6]) - b0 * 2 * img;
+    p.fin_gy = reinterpret_cast<float*>(base + w.off[7]) - b0 * 2 * tile;
+  }
   int* words = reinterpret_cast<int*>(base + w.off[0]);
   p.status = words + (size_t)pl.n_rest * ttt::BWD_SYNC_STRIDE;
   p.sync = words - b0 * ttt::BWD_SYNC_STRIDE;
@@ -241,7 +254,7 @@ extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* wo
   p.norm_park = reinterpret_cast<float*>(base + w.off[2]) - b0 * norm;
   p.walk_park = reinterpret_cast<__bf16*>(base + w.off[3]) - b0 * (TTT_MLP_CS * TTT_MLP_HID);
   for (int s = 0; s < alt_sets; s++) {
-    const size_t* o = w.off + 4 + BwdWorkspace::PER_SET * s;
+    const size_t* o = w.off + 8 + BwdWorkspace::PER_SET * s;
     p.alt_X2_group[s] = reinterpret_cast<__bf16*>(base + o[0]) - b0 * img;
     p.alt_Z1_group[s] = reinterpret_cast<__bf16*>(base + o[1]) - b0 * img;
     p.alt_Z1_bar_group[s] = reinterpret_cast<__bf16*>(base + o[2]) - b0 * img;

@@ -57,6 +57,12 @@ struct BwdParams {
   float* norm_park;      // [B*NH][8 waves][2][64]: n_replay = 1: the share of the parity that is not being added to
   __bf16* walk_park;     // [B*NH][64][256]: one register image the walking workgroup parks across its LayerNorm stage
   int n_replay;
+  // n_finish = 1: a further workgroup forms grad_L_XK from what the walk hands it per mini-batch - three
+  // register images (gW1 as operand, G1, dZ1: [B*NH][2 sets][cgs][64][256] bf16 each) and g_y
+  // ([B*NH][2][cgs][64][64] fp32); the two sets alternate by group.
+  __bf16 *fin_gw1, *fin_g1, *fin_dz;
+  float* fin_gy;
+  int n_finish;
   int* sync;
   int* status;    // the status word behind the synchronisation words
   int bh0, nbh;   // this launch covers (batch, head) pairs bh0 .. bh0 + nbh - 1 (workspace pointers moved back by bh0 entries)
@@ -64,7 +70,8 @@ struct BwdParams {
 
 // Layout of `sync` (ints): 32 per (batch, head) - words 0 and 8 count the groups replayed by the first /
 // second replaying workgroup (norm_partial is written before the last count), word 16 the groups the
-// reverse walk has finished - then one status word (non-zero: a wait gave up).
+// reverse walk has finished, word 24 the groups the grad_L_XK workgroup has finished - then one status
+// word (non-zero: a wait gave up).
 constexpr int BWD_SYNC_STRIDE = 32;
 inline size_t bwd_sync_ints(long long BH) { return (size_t)BH * BWD_SYNC_STRIDE + 32; }
 
