@@ -130,16 +130,17 @@ int ttt_mlp_fwd_launch(const ttt_mlp_fwd_args* args, void* stream);
 /* Same for the remat backward. */
 int ttt_mlp_bwd_launch(const ttt_mlp_bwd_args* args, void* stream);
 
-/* The same backward (bit-identical results) with two or three workgroups per
+/* The same backward (bit-identical results) with two to four workgroups per
  * (batch, head) where the device has CUs to spare: one or two recompute checkpoint
- * group after checkpoint group, the last one walks each recomputed group
- * backwards, so recomputation leaves the critical path.  The reference launcher
+ * group after checkpoint group, one walks each recomputed group backwards, and a
+ * fourth forms grad_L_XK from what the walk hands it, so that only the chain
+ * through the running gradients stays on the critical path.  The reference launcher
  * (kernels/ttt_backward/ttt.cu:1451-1917) has no counterpart: it spreads one
  * (batch, head) over a cluster of four thread blocks instead.
  * Workgroups that wait for each other must be resident together (one per CU),
  * so the pairs are covered by up to two launches in a row: the largest multiple
  * of the CU count with one workgroup per pair, then the remaining n pairs with
- * three each if 3*n fits the CUs, else two each if 2*n fits.
+ * four each if 4*n fits the CUs, else three if 3*n fits, else two if 2*n fits.
  * ttt_mlp_bwd_workspace_bytes() returns 0 when neither does (n = 0 or 2*n > CUs of
  * the current device); the launcher then returns TTT_MLP_ERR_NO_ROOM and the caller
  * uses ttt_mlp_bwd_launch.
