@@ -57,6 +57,16 @@ void finish(int rc, hipStream_t stream, const char* what, const void* status = n
   }
 }
 
+// The multi-workgroup launches are an optimisation: not worth failing (or evicting the caller's cached
+// blocks) for.  They are used only if their workspace fits comfortably into what the device has free
+// (memory held by torch's caching allocator counts as free for torch, so this is conservative).
+bool workspace_is_affordable(size_t bytes) {
+  if (bytes == 0) return false;
+  size_t free_b = 0, total_b = 0;
+  if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) return false;
+  return bytes <= free_b / 2;
+}
+
 }  // namespace
 
 torch::Tensor ttt_forward(const torch::Tensor XQ, const torch::Tensor XK, const torch::Tensor XV,
@@ -103,7 +113,7 @@ torch::Tensor ttt_forward(const torch::Tensor XQ, const torch::Tensor XK, const 
   // the state recurrence.  Its workspace comes from torch's caching allocator, which orders its reuse
   // after this launch on the same stream.
   const size_t ws_bytes = (g_overlap && NC >= 2) ? ttt_mlp_fwd_workspace_bytes((int32_t)B, (int32_t)NH) : 0;
-  if (ws_bytes > 0) {
+  if (workspace_is_affordable(ws_bytes)) {
     torch::Tensor ws = torch::empty({(int64_t)ws_bytes}, torch::TensorOptions().dtype(torch::kUInt8).device(XQ.device()));
     g_last_forward_mode = 1;
     const char* status = static_cast<const char*>(ws.data_ptr()) + ttt_mlp_fwd_status_offset((int32_t)B, (int32_t)NH);
@@ -215,7 +225,7 @@ torch::Tensor ttt_backward(
   // checkpoint groups ahead of the reverse walk.  Its workspace (a second set of the per-group tensors)
   // comes from torch's caching allocator, which orders its reuse after this launch on the same stream.
   const size_t ws_bytes = (g_overlap && K >= 2) ? ttt_mlp_bwd_workspace_bytes((int32_t)B, (int32_t)NH, checkpoint_group_size) : 0;
-  if (ws_bytes > 0) {
+  if (workspace_is_affordable(ws_bytes)) {
     torch::Tensor ws = torch::empty({(int64_t)ws_bytes}, torch::TensorOptions().dtype(torch::kUInt8).device(XQ.device()));
     g_last_backward_mode = 1;
     const char* status = static_cast<const char*>(ws.data_ptr()) + ttt_mlp_bwd_status_offset((int32_t)B, (int32_t)NH);
