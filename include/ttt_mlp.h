@@ -165,6 +165,11 @@ size_t ttt_mlp_fwd_status_offset(int32_t B, int32_t NH);
 int ttt_mlp_fwd_launch_overlapped(const ttt_mlp_fwd_args* args, void* workspace, size_t workspace_bytes, void* stream);
 int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* args, void* workspace, size_t workspace_bytes, void* stream);
 
+/* How long a workgroup of an overlapped launch waits for another before it gives up and raises the
+ * status word, in ticks of the GPU's 100 MHz clock (default 2,000,000,000 = 20 s).  Process-wide; meant
+ * for tests of that path (a limit of 1 makes the first wait give up) and for hosts that want a shorter one. */
+void ttt_mlp_set_wait_limit(unsigned long long ticks_100mhz);
+
 /* Human-readable text for a return code of the two launchers. */
 const char* ttt_mlp_error_string(int code);
 

@@ -73,3 +73,34 @@ def test_overlapped_launchers_through_ctypes(B, NH, NC, cgs):
     for k in results[0]:
         assert torch.isfinite(results[1][k]).all(), k
         assert torch.equal(results[0][k], results[1][k]), k
+
+
+def test_a_wait_that_gives_up_is_reported_and_every_wave_exits():
+    """Forced from the host: with a wait limit of one clock tick the first workgroup that has to wait for its
+    partner gives up at once, raises the status word, and all workgroups of the launch leave.  The operator
+    (which synchronises by default) reports it; with the default limit the same call then succeeds."""
+    import ttt_mlp_host as host
+    import test_time_training as ext
+    dev = torch.device("cuda:0")
+    B, NH, NC, cgs = 1, 2, 24, 4
+    d = orc.make_inputs(B, NH, NC, seed=41)
+    t = {k: d[k].to(dev).contiguous() for k in FWD_KEYS + UP_KEYS}
+    t.update(host.alloc_forward_buffers(B, NH, NC, cgs, dev))
+    t.update(host.alloc_backward_buffers(B, NH, NC, cgs, dev))
+    try:
+        ext.set_wait_limit(1)
+        with pytest.raises(RuntimeError, match="gave up"):
+            host.forward(t, cgs)
+        assert ext.last_forward_mode() == 1
+        ext.set_wait_limit(2_000_000_000)
+        host.forward(t, cgs)              # checkpoints for the backward
+        ext.set_wait_limit(1)
+        with pytest.raises(RuntimeError, match="gave up"):
+            host.backward(t, cgs)
+        assert ext.last_backward_mode() == 1
+    finally:
+        ext.set_wait_limit(2_000_000_000)
+    torch.cuda.synchronize()
+    host.zero_accumulating_grads(t)
+    host.backward(t, cgs)                 # the device is fine and the same call goes through
+    assert torch.isfinite(t["grad_L_W1_init"]).all()

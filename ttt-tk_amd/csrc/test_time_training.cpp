@@ -249,6 +249,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("set_overlap", [](bool on) { g_overlap = on; },
         "Use a second workgroup per (batch, head) when the device has room: the forward's output branch, the "
         "backward's recomputation of checkpoint groups (default true).");
+  m.def("set_wait_limit", [](unsigned long long ticks) { ttt_mlp_set_wait_limit(ticks); },
+        "Ticks of the GPU's 100 MHz clock a workgroup waits for its partner before giving up (default 2e9 = 20 s).");
   m.def("last_forward_mode", []() { return g_last_forward_mode; },
         "0: the last ttt_forward used one workgroup per (batch, head); 1: two; -1: none yet.");
   m.def("last_backward_mode", []() { return g_last_backward_mode; },

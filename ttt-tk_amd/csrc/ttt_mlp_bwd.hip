@@ -582,9 +582,9 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
     // ================================================================= replay
     if constexpr (ROLE != 2) {
       if constexpr (ROLE == 1) {   // the set is free once the reverse walk is done with the group that used it last
-        if (done >= n_sets && !wait_at_least(w_walked, done - n_sets + 1, w_status, s_flag)) return;
+        if (done >= n_sets && !wait_at_least(w_walked, done - n_sets + 1, w_status, s_flag, p.wait_limit)) return;
         if constexpr (FIN) {   // ... and so is the workgroup that reads the before-state images for grad_L_XK
-          if (done >= n_sets && !wait_at_least(w_finished, done - n_sets + 1, w_status, s_flag)) return;
+          if (done >= n_sets && !wait_at_least(w_finished, done - n_sets + 1, w_status, s_flag, p.wait_limit)) return;
         }
         // a single replaying workgroup adds to the sum of this group's parity: the groups alternate, so from
         // the second group on the live sum and the parked one change places
@@ -893,9 +893,9 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
     // wave covers the latency, while holding requests in registers across stages costs more in spills
     // than it gains (measured).
     if constexpr (ROLE == 2) {
-      if (!wait_at_least(w_replayed, done / n_replay + 1, w_status, s_flag)) return;
+      if (!wait_at_least(w_replayed, done / n_replay + 1, w_status, s_flag, p.wait_limit)) return;
       if constexpr (FIN) {   // the hand-over set of this group's parity is free once the group before last is finished
-        if (done >= 2 && !wait_at_least(w_finished, done - 1, w_status, s_flag)) return;
+        if (done >= 2 && !wait_at_least(w_finished, done - 1, w_status, s_flag, p.wait_limit)) return;
       }
     }
     // hand-over buffers of this group for the grad_L_XK workgroup (set = parity of the group)
@@ -1347,7 +1347,7 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
   for (int k = p.K - 1; k >= 0; k--) {
     const int n_mb = min(cgs, p.NC - k * cgs);
     const int done = p.K - 1 - k, set = done % n_sets;
-    if (!wait_at_least(w_walked, done + 1, p.status, s_flag)) return;
+    if (!wait_at_least(w_walked, done + 1, p.status, s_flag, p.wait_limit)) return;
     const size_t ofin = uni64(((size_t)bh * 2 + (done & 1)) * cgs);
     const gptr_t gGW = gbuf(p.fin_gw1 + ofin * (CS * HID)), gG1 = gbuf(p.fin_g1 + ofin * (CS * HID));
     const gptr_t gDZ = gbuf(p.fin_dz + ofin * (CS * HID)), gGY = gbuf(p.fin_gy + ofin * (CS * FD));

@@ -22,12 +22,16 @@ int check_sizes(int B, int NH, int NC, int K, int cgs) {
   return TTT_MLP_OK;
 }
 
+unsigned long long g_wait_limit = 2000000000ull;   // 20 s of the 100 MHz clock
+
 inline const __bf16* bf(const uint16_t* p) { return reinterpret_cast<const __bf16*>(p); }
 inline __bf16* bf(uint16_t* p) { return reinterpret_cast<__bf16*>(p); }
 
 }  // namespace
 
 extern "C" int ttt_mlp_abi_version(void) { return TTT_MLP_ABI_VERSION; }
+
+extern "C" void ttt_mlp_set_wait_limit(unsigned long long ticks_100mhz) { g_wait_limit = ticks_100mhz; }
 
 extern "C" const char* ttt_mlp_error_string(int code) {
   switch (code) {
@@ -241,6 +245,7 @@ extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* wo
   p.nbh = static_cast<int>(pl.n_rest);
   p.n_replay = n_replay;
   p.n_finish = finish ? 1 : 0;
+  p.wait_limit = g_wait_limit;
   if (finish) {
     p.fin_gw1 = reinterpret_cast<__bf16*>(base + w.off[4]) - b0 * 2 * img;
     p.fin_g1 = reinterpret_cast<__bf16*>(base + w.off[5]) - b0 * 2 * img;
@@ -310,6 +315,7 @@ extern "C" int ttt_mlp_fwd_launch_overlapped(const ttt_mlp_fwd_args* a, void* wo
   int* words = reinterpret_cast<int*>(base + w.off[0]);
   p.status = words + (size_t)pl.n_rest * ttt::BWD_SYNC_STRIDE;
   p.sync = words - b0 * ttt::BWD_SYNC_STRIDE;
+  p.wait_limit = g_wait_limit;
   p.state_img = reinterpret_cast<__bf16*>(base + w.off[1]) - b0 * 2 * ttt::FWD_RING * (ttt::FWD_IMG_BYTES / 2);
   p.bias_img = reinterpret_cast<float*>(base + w.off[2]) - b0 * 2 * ttt::FWD_RING * ttt::FWD_BIAS_FLOATS;
   return static_cast<int>(ttt_mlp_fwd_enqueue(p, static_cast<hipStream_t>(stream)));

@@ -371,17 +371,16 @@ TTT_DEV void gelu_fdd(float x, float& g, float& d1, float& d2) {
 // ---------------------------------------------------------------------------- workgroups that wait for each other
 // Two workgroups of one (batch, head) hand work over through counters in HBM (agent scope).  Both are
 // resident at once because the launchers use such a mode only when the grid fits the CUs of the device.
-// A wait that sees no progress for SPIN_LIMIT ticks of the 100 MHz clock raises the status word and
-// makes both workgroups leave, so every wave always exits.
-constexpr uint64_t SPIN_LIMIT = 2000000000ull;   // 20 s
-TTT_DEV bool wait_at_least(int* word, int target, int* status, int* s_flag) {
+// A wait that sees no progress for `limit` ticks of the 100 MHz clock (20 s unless the host says otherwise)
+// raises the status word and makes all workgroups of the launch leave, so every wave always exits.
+TTT_DEV bool wait_at_least(int* word, int target, int* status, int* s_flag, uint64_t limit) {
   if (threadIdx.x == 0) {
     int ok = 1;
     const uint64_t t0 = wall_clock64();
     // polled without acquire semantics (an acquire at agent scope invalidates caches on every poll);
     // one acquire fence once the value is there
     while (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
-      if (__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 || wall_clock64() - t0 > SPIN_LIMIT) {
+      if (__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 || wall_clock64() - t0 > limit) {
         __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         ok = 0;
         break;

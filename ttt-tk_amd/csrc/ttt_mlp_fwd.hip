@@ -240,7 +240,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
     float* const gB = p.bias_img + ((size_t)bh * 2 * FWD_RING + slot) * FWD_BIAS_FLOATS;
     if constexpr (ROLE == 1) {
       if (mb % FWD_RING == 0 && grp >= 2) {   // the set is free once the output branch is done with the group before last
-        if (!wait_at_least(w_taken, grp - 1, w_status, s_flag)) return;
+        if (!wait_at_least(w_taken, grp - 1, w_status, s_flag, p.wait_limit)) return;
       }
     }
 
@@ -516,7 +516,7 @@ TTT_DEV void fwd_output_branch(const FwdParams& p, unsigned char* smem, const in
     LANE_VARS;
     const int grp = mb / FWD_RING, slot = (grp & 1) * FWD_RING + mb % FWD_RING;
     if (mb % FWD_RING == 0) {
-      if (!wait_at_least(w_given, grp + 1, w_status, s_flag)) return;
+      if (!wait_at_least(w_given, grp + 1, w_status, s_flag, p.wait_limit)) return;
     }
     bf16* s_xq = reinterpret_cast<bf16*>(smem + SM_XQ + (mb & 1) * SM_TILE);
     const gptr_t gImg = gbuf(p.state_img + ((size_t)bh * 2 * FWD_RING + slot) * (FWD_IMG_BYTES / 2));

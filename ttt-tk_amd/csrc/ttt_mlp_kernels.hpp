@@ -21,6 +21,7 @@ struct FwdParams {
   float* bias_img;
   int* sync;
   int* status;    // the status word behind the synchronisation words
+  unsigned long long wait_limit;   // ticks of the 100 MHz clock a workgroup waits for another before it gives up
   int bh0, nbh;   // this launch covers (batch, head) pairs bh0 .. bh0 + nbh - 1
 };
 constexpr int FWD_RING = 8;                    // mini-batches per hand-over
@@ -65,6 +66,7 @@ struct BwdParams {
   int n_finish;
   int* sync;
   int* status;    // the status word behind the synchronisation words
+  unsigned long long wait_limit;   // ticks of the 100 MHz clock a workgroup waits for another before it gives up
   int bh0, nbh;   // this launch covers (batch, head) pairs bh0 .. bh0 + nbh - 1 (workspace pointers moved back by bh0 entries)
 };
 
