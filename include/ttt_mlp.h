@@ -173,6 +173,13 @@ void ttt_mlp_set_wait_limit(unsigned long long ticks_100mhz);
 /* Human-readable text for a return code of the two launchers. */
 const char* ttt_mlp_error_string(int code);
 
+/* How an overlapped launch of `pairs` = B*NH (batch, head) pairs is laid out on a device with
+ * `compute_units` CUs (no device needed): the first *one_workgroup_pairs pairs run with one workgroup each,
+ * the remaining *other_pairs with *workgroups_per_other_pair each (0 if there are none).  which = 0
+ * forward, 1 backward. */
+int ttt_mlp_launch_plan(int which, long long pairs, int compute_units, long long* one_workgroup_pairs,
+                        long long* other_pairs, int* workgroups_per_other_pair);
+
 /* Static facts about the compiled kernels, for harnesses: LDS bytes per
  * workgroup and threads per workgroup of the forward (which = 0) or backward
  * (which = 1) kernel.  Returns 0 on success. */

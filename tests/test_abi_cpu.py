@@ -35,7 +35,7 @@ def test_header_declares_the_expected_entry_points():
     assert declared_functions() == ["ttt_mlp_abi_version", "ttt_mlp_bwd_launch", "ttt_mlp_bwd_launch_overlapped",
                                     "ttt_mlp_bwd_status_offset", "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_error_string",
                                     "ttt_mlp_fwd_launch", "ttt_mlp_fwd_launch_overlapped", "ttt_mlp_fwd_status_offset",
-                                    "ttt_mlp_fwd_workspace_bytes", "ttt_mlp_kernel_info", "ttt_mlp_set_wait_limit"]
+                                    "ttt_mlp_fwd_workspace_bytes", "ttt_mlp_kernel_info", "ttt_mlp_launch_plan", "ttt_mlp_set_wait_limit"]
 
 
 def test_library_exports_every_declared_symbol(lib):
@@ -170,3 +170,32 @@ def test_host_module_offers_the_autograd_wrapper(lib):
     assert list(inspect.signature(host.ttt_mlp).parameters) == [
         "XQ", "XK", "XV", "last_eta", "ttt_norm_weight", "ttt_norm_bias", "W1", "b1", "W2", "b2", "checkpoint_group_size"]
     assert "grad_last" in inspect.signature(host.ttt_mlp_backward).parameters
+
+
+def test_launch_plan_keeps_waiting_workgroups_within_the_device(lib):
+    """Workgroups that wait for each other must all be resident: whatever the plan, the launch with several
+    workgroups per pair never exceeds the CU count, and full rounds of the device come first."""
+    def plan(which, pairs, cus):
+        a, b, c = ctypes.c_longlong(), ctypes.c_longlong(), ctypes.c_int()
+        assert lib.ttt_mlp_launch_plan(which, ctypes.c_longlong(pairs), cus, ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)) == 0
+        return a.value, b.value, c.value
+    assert plan(1, 48, 256) == (0, 48, 4)          # the metric's configuration: four workgroups per pair
+    assert plan(1, 72, 256) == (0, 72, 3)
+    assert plan(1, 96, 256) == (0, 96, 2)
+    assert plan(1, 200, 256) == (200, 0, 0)        # two per pair would not fit: one each
+    assert plan(1, 384, 256) == (256, 128, 2)      # one full round, the rest with two each
+    assert plan(1, 260, 256) == (256, 4, 4)
+    assert plan(1, 512, 256) == (512, 0, 0)
+    assert plan(0, 48, 256) == (0, 48, 2)          # forward: two, and only if everything fits
+    assert plan(0, 384, 256) == (384, 0, 0)
+    assert plan(1, 48, 0) == (48, 0, 0)            # no device: nothing to overlap
+    for which in (0, 1):
+        for cus in (1, 8, 104, 256, 304):
+            for pairs in list(range(1, 40)) + [cus - 1, cus, cus + 1, 2 * cus, 3 * cus + 5, 10 * cus + cus // 3]:
+                if pairs <= 0:
+                    continue
+                one, rest, per = plan(which, pairs, cus)
+                assert one + rest == pairs and one % cus == 0 or rest == 0
+                assert rest * per <= cus
+                assert per in ((0, 2) if which == 0 else (0, 2, 3, 4))
+    assert lib.ttt_mlp_launch_plan(2, ctypes.c_longlong(1), 1, None, None, None) == 1001

@@ -128,11 +128,9 @@ struct LaunchPlan {
 };
 // `after_full_rounds`: whether the rest may be split when full rounds precede it.  That pays for the
 // backward; the forward's gain from splitting is smaller than what a full device costs it (measured).
-LaunchPlan plan_launches(long long BH, bool after_full_rounds, bool three_way) {
+LaunchPlan plan_for(long long BH, int cus, bool after_full_rounds, bool three_way) {
   LaunchPlan pl;
-  int dev = 0, cus = 0;
-  if (BH <= 0 || hipGetDevice(&dev) != hipSuccess ||
-      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+  if (BH <= 0 || cus <= 0) {
     pl.n_single = BH > 0 ? BH : 0;
     return pl;
   }
@@ -142,6 +140,12 @@ LaunchPlan plan_launches(long long BH, bool after_full_rounds, bool three_way) {
   if (!pl.rest_split) { pl.n_single = BH; pl.n_rest = 0; }
   else pl.per_pair = !three_way ? 2 : 4 * pl.n_rest <= cus ? 4 : 3 * pl.n_rest <= cus ? 3 : 2;
   return pl;
+}
+LaunchPlan plan_launches(long long BH, bool after_full_rounds, bool three_way) {
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+    cus = 0;
+  return plan_for(BH, cus, after_full_rounds, three_way);
 }
 
 // Workspace of the backward with 2 or 3 workgroups per pair, for n (batch, head) pairs: the synchronisation
@@ -319,6 +323,17 @@ extern "C" int ttt_mlp_fwd_launch_overlapped(const ttt_mlp_fwd_args* a, void* wo
   p.state_img = reinterpret_cast<__bf16*>(base + w.off[1]) - b0 * 2 * ttt::FWD_RING * (ttt::FWD_IMG_BYTES / 2);
   p.bias_img = reinterpret_cast<float*>(base + w.off[2]) - b0 * 2 * ttt::FWD_RING * ttt::FWD_BIAS_FLOATS;
   return static_cast<int>(ttt_mlp_fwd_enqueue(p, static_cast<hipStream_t>(stream)));
+}
+
+extern "C" int ttt_mlp_launch_plan(int which, long long pairs, int compute_units, long long* one_workgroup_pairs,
+                                   long long* other_pairs, int* workgroups_per_other_pair) {
+  if (one_workgroup_pairs == nullptr || other_pairs == nullptr || workgroups_per_other_pair == nullptr || (which != 0 && which != 1))
+    return TTT_MLP_ERR_BAD_ARG;
+  const LaunchPlan pl = plan_for(pairs, compute_units, which == 1, which == 1);
+  *one_workgroup_pairs = pl.n_single;
+  *other_pairs = pl.n_rest;
+  *workgroups_per_other_pair = pl.n_rest > 0 ? pl.per_pair : 0;
+  return TTT_MLP_OK;
 }
 
 extern "C" int ttt_mlp_kernel_info(int which, int* lds_bytes, int* threads_per_workgroup) {
