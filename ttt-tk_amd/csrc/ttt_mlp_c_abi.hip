@@ -181,12 +181,12 @@ struct BwdWorkspace {
 };
 
 // Workspace of the forward's two-workgroup mode: synchronisation words, then per (batch, head) a ring of
-// 2 * FWD_RING slots of state images and of bias vectors.
+// 2 * FWD_RING_MAX slots of state images and of bias vectors.
 struct FwdWorkspace {
   size_t off[3];
   size_t total;
   explicit FwdWorkspace(long long n) {
-    const size_t slots = (size_t)n * 2 * ttt::FWD_RING;
+    const size_t slots = (size_t)n * 2 * ttt::FWD_RING_MAX;
     const size_t bytes[3] = {ttt::bwd_sync_ints(n) * sizeof(int), slots * ttt::FWD_IMG_BYTES,
                              slots * ttt::FWD_BIAS_FLOATS * sizeof(float)};
     size_t o = 0;
@@ -320,8 +320,9 @@ extern "C" int ttt_mlp_fwd_launch_overlapped(const ttt_mlp_fwd_args* a, void* wo
   p.status = words + (size_t)pl.n_rest * ttt::BWD_SYNC_STRIDE;
   p.sync = words - b0 * ttt::BWD_SYNC_STRIDE;
   p.wait_limit = g_wait_limit;
-  p.state_img = reinterpret_cast<__bf16*>(base + w.off[1]) - b0 * 2 * ttt::FWD_RING * (ttt::FWD_IMG_BYTES / 2);
-  p.bias_img = reinterpret_cast<float*>(base + w.off[2]) - b0 * 2 * ttt::FWD_RING * ttt::FWD_BIAS_FLOATS;
+  p.ring_log2 = p.NC >= 512 ? 5 : 3;   // 32 or 8 mini-batches per hand-over
+  p.state_img = reinterpret_cast<__bf16*>(base + w.off[1]) - b0 * 2 * ttt::FWD_RING_MAX * (ttt::FWD_IMG_BYTES / 2);
+  p.bias_img = reinterpret_cast<float*>(base + w.off[2]) - b0 * 2 * ttt::FWD_RING_MAX * ttt::FWD_BIAS_FLOATS;
   return static_cast<int>(ttt_mlp_fwd_enqueue(p, static_cast<hipStream_t>(stream)));
 }
 

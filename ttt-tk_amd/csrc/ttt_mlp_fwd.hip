@@ -154,7 +154,8 @@ TTT_DEV void output_layernorm(const float* s_P, const float* s_b2, const float* 
 
 // ROLE 0: the whole scan in one workgroup.  ROLE 1: the state recurrence only - after every mini-batch
 // the new state is left in HBM as ready-made bf16 operands for the workgroup that runs fwd_output_branch.
-template <int ROLE>
+// RING: mini-batches per hand-over (ROLE 1).
+template <int ROLE, int RING>
 TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
   bf16* s_g2 = reinterpret_cast<bf16*>(smem + SM_G2);
   float* s_P = reinterpret_cast<float*>(smem + SM_P);
@@ -235,11 +236,11 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
     const bf16* s_xk = reinterpret_cast<const bf16*>(smem + (alt ? SM_XQ : SM_XK));
     const bf16* s_xv = reinterpret_cast<const bf16*>(smem + (alt ? SM_XQ + SM_TILE : SM_XV));
     const float* s_eta = reinterpret_cast<const float*>(smem + (alt ? SM_B1 : SM_ETA));
-    // ROLE 1: where the state after this mini-batch goes (a ring of 2 * FWD_RING slots)
-    const int grp = mb / FWD_RING, slot = (grp & 1) * FWD_RING + mb % FWD_RING;
-    float* const gB = p.bias_img + ((size_t)bh * 2 * FWD_RING + slot) * FWD_BIAS_FLOATS;
+    // ROLE 1: where the state after this mini-batch goes (a ring of 2 * ring slots)
+    constexpr int ring = RING; const int grp = mb / ring, at = mb % ring, slot = (grp & 1) * ring + at;
+    float* const gB = p.bias_img + ((size_t)bh * 2 * FWD_RING_MAX + slot) * FWD_BIAS_FLOATS;
     if constexpr (ROLE == 1) {
-      if (mb % FWD_RING == 0 && grp >= 2) {   // the set is free once the output branch is done with the group before last
+      if (at == 0 && grp >= 2) {   // the set is free once the output branch is done with the group before last
         if (!wait_at_least(w_taken, grp - 1, w_status, s_flag, p.wait_limit)) return;
       }
     }
@@ -424,7 +425,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
       // ---- hand the state after this mini-batch to the output branch: W1s and W2s exactly as the
       //      post-update forward would convert them, and the two bias vectors
       LANE_VARS;
-      const gptr_t gImg = gbuf(p.state_img + ((size_t)bh * 2 * FWD_RING + slot) * (FWD_IMG_BYTES / 2));
+      const gptr_t gImg = gbuf(p.state_img + ((size_t)bh * 2 * FWD_RING_MAX + slot) * (FWD_IMG_BYTES / 2));
       const OpdT<1, 4> w1A = cvt_chain(W1s);
       const OpdT<2, 2> w2A = cvt_chain(W2s);
 #pragma unroll
@@ -434,7 +435,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
 #pragma unroll
         for (int s = 0; s < 2; s++) g_st_stream<bf16x8>(gImg, 16 * tid, (4 + 2 * fb + s) * 8192, w2A.v[fb][s]);
       if (h == 0) gB[hid0 + c] = b1L;
-      if (mb % FWD_RING == FWD_RING - 1 || mb == p.NC - 1) publish(w_given, grp + 1);
+      if (at == ring - 1 || mb == p.NC - 1) publish(w_given, grp + 1);
       // No barrier ends a mini-batch here: every LDS buffer written from now on was last read before a
       // barrier that its writers have yet to pass (the pair sum's, or the one after the LayerNorm stage).
       continue;
@@ -487,6 +488,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
 // The output branch of the forward on its own workgroup: Out[mb] = XQ + LN(gelu(XQ W1' + b1') W2' + b2')
 // with the state after mini-batch mb, taken from the operand images the recurrence leaves behind.  Nothing
 // is carried from one mini-batch to the next here.
+template <int RING>
 TTT_DEV void fwd_output_branch(const FwdParams& p, unsigned char* smem, const int bh) {
   float* s_P = reinterpret_cast<float*>(smem + SM_P);
   float* s_b1 = reinterpret_cast<float*>(smem + SM_B1);
@@ -514,13 +516,13 @@ TTT_DEV void fwd_output_branch(const FwdParams& p, unsigned char* smem, const in
 
   for (int mb = 0; mb < p.NC; mb++) {
     LANE_VARS;
-    const int grp = mb / FWD_RING, slot = (grp & 1) * FWD_RING + mb % FWD_RING;
-    if (mb % FWD_RING == 0) {
+    constexpr int ring = RING; const int grp = mb / ring, at = mb % ring, slot = (grp & 1) * ring + at;
+    if (at == 0) {
       if (!wait_at_least(w_given, grp + 1, w_status, s_flag, p.wait_limit)) return;
     }
     bf16* s_xq = reinterpret_cast<bf16*>(smem + SM_XQ + (mb & 1) * SM_TILE);
-    const gptr_t gImg = gbuf(p.state_img + ((size_t)bh * 2 * FWD_RING + slot) * (FWD_IMG_BYTES / 2));
-    const float* gB = p.bias_img + ((size_t)bh * 2 * FWD_RING + slot) * FWD_BIAS_FLOATS;
+    const gptr_t gImg = gbuf(p.state_img + ((size_t)bh * 2 * FWD_RING_MAX + slot) * (FWD_IMG_BYTES / 2));
+    const float* gB = p.bias_img + ((size_t)bh * 2 * FWD_RING_MAX + slot) * FWD_BIAS_FLOATS;
     {
       LANE_VARS;
       // XQ and b2 alternate between two LDS buffers: other waves may still be in the previous mini-batch's
@@ -568,17 +570,20 @@ TTT_DEV void fwd_output_branch(const FwdParams& p, unsigned char* smem, const in
       LANE_VARS;
       output_layernorm(s_P, s_b2 + (mb & 1) * FD, s_gam, s_bet, s_xq, gOut, mb, tok, f0);
     }
-    if (mb % FWD_RING == FWD_RING - 1 || mb == p.NC - 1) publish(w_taken, grp + 1);
+    if (at == ring - 1 || mb == p.NC - 1) publish(w_taken, grp + 1);
   }
 #undef LANE_VARS
 }
 
 __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  fwd_body<0>(p, smem, p.bh0 + blockIdx.x);
+  fwd_body<0, 8>(p, smem, p.bh0 + blockIdx.x);
 }
 
 // Two workgroups per (batch, head), placed like those of the backward (same XCD where the count allows).
+// RING = mini-batches per hand-over: each hand-over costs a release (an L2 write-back), and the output branch
+// ends that many mini-batches after the recurrence; 32 pays from a few hundred mini-batches on (measured).
+template <int RING>
 __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_split_kernel(const FwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int b = blockIdx.x;
@@ -591,8 +596,8 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_split_kernel(const Fwd
     role = b & 1;
   }
   bh += p.bh0;
-  if (role == 0) fwd_body<1>(p, smem, bh);
-  else fwd_output_branch(p, smem, bh);
+  if (role == 0) fwd_body<1, RING>(p, smem, bh);
+  else fwd_output_branch<RING>(p, smem, bh);
 }
 
 __global__ void ttt_mlp_fwd_zero_words(int* w, int n) {
@@ -614,12 +619,16 @@ hipError_t ttt_mlp_fwd_enqueue(const ttt::FwdParams& p, hipStream_t stream) {
     hipLaunchKernelGGL(ttt::ttt_mlp_fwd_kernel, dim3(p.nbh), dim3(ttt::FW_THREADS), ttt::SM_FWD_BYTES, stream, p);
     return hipGetLastError();
   }
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(ttt::ttt_mlp_fwd_split_kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, ttt::SM_FWD_BYTES);
+  const void* kernel = p.ring_log2 == 5 ? reinterpret_cast<const void*>(ttt::ttt_mlp_fwd_split_kernel<32>)
+                                        : reinterpret_cast<const void*>(ttt::ttt_mlp_fwd_split_kernel<8>);
+  hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, ttt::SM_FWD_BYTES);
   if (e != hipSuccess) return e;
   const int n = static_cast<int>(ttt::bwd_sync_ints(p.nbh));
   int* const words = p.status - (size_t)p.nbh * ttt::BWD_SYNC_STRIDE;   // p.sync itself is moved back by bh0 entries
   hipLaunchKernelGGL(ttt::ttt_mlp_fwd_zero_words, dim3((n + 255) / 256), dim3(256), 0, stream, words, n);
-  hipLaunchKernelGGL(ttt::ttt_mlp_fwd_split_kernel, dim3(2 * p.nbh), dim3(ttt::FW_THREADS), ttt::SM_FWD_BYTES, stream, p);
+  if (p.ring_log2 == 5)
+    hipLaunchKernelGGL(ttt::ttt_mlp_fwd_split_kernel<32>, dim3(2 * p.nbh), dim3(ttt::FW_THREADS), ttt::SM_FWD_BYTES, stream, p);
+  else
+    hipLaunchKernelGGL(ttt::ttt_mlp_fwd_split_kernel<8>, dim3(2 * p.nbh), dim3(ttt::FW_THREADS), ttt::SM_FWD_BYTES, stream, p);
   return hipGetLastError();
 }

@@ -12,19 +12,21 @@ struct FwdParams {
   float *W1_ck, *b1_ck, *W2_ck, *b2_ck;
   __bf16* Out;
   int B, NH, NC, K, cgs;
-  // Two-workgroup mode only (sync != nullptr): per (batch, head) a ring of 2 * FWD_RING mini-batch slots
+  // Two-workgroup mode only (sync != nullptr): per (batch, head) a ring of 2 * FWD_RING_MAX mini-batch slots
+  // (2 << ring_log2 of them in use: 1 << ring_log2 mini-batches per hand-over, chosen by the launcher from NC)
   // with the bf16 operand images (64 KiB) and the bias vectors (256 + 64 floats) of the state after a
   // mini-batch, and the words the two workgroups signal with (layout as in the backward).
   // The workspace pointers are indexed by the global (batch, head) number like everything else: the
   // launcher passes them moved back by bh0 entries.
   __bf16* state_img;
   float* bias_img;
+  int ring_log2;
   int* sync;
   int* status;    // the status word behind the synchronisation words
   unsigned long long wait_limit;   // ticks of the 100 MHz clock a workgroup waits for another before it gives up
   int bh0, nbh;   // this launch covers (batch, head) pairs bh0 .. bh0 + nbh - 1
 };
-constexpr int FWD_RING = 8;                    // mini-batches per hand-over
+constexpr int FWD_RING_MAX = 32;               // most mini-batches per hand-over (8 or 32 are compiled)
 constexpr int FWD_IMG_BYTES = 64 * 256 * 2 * 2;  // W1 and W2 as bf16 operands
 constexpr int FWD_BIAS_FLOATS = 256 + 64;
 
