@@ -1392,9 +1392,11 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
 
 // n_replay + 1 (+ 1) workgroups per (batch, head).  Workgroups are dealt to the 8 XCDs in turn, so with a
 // multiple of 8 (batch, head) pairs the workgroups of a pair are placed 8 apart: same XCD, same L2.
+// One kernel per combination, so that each holds only the code (and the register allocation) of its own roles.
+template <int NREPLAY, bool FINISH>
 __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_split_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int b = blockIdx.x, per = p.n_replay + 1 + p.n_finish;
+  const int b = blockIdx.x, per = NREPLAY + 1 + (FINISH ? 1 : 0);
   int bh, role;
   if (p.nbh % 8 == 0) {
     bh = (b / (8 * per)) * 8 + (b & 7);
@@ -1404,17 +1406,10 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_split_kernel(const Bwd
     role = b % per;
   }
   bh += p.bh0;
-  if (p.n_finish) {   // two replay, one walks, one forms grad_L_XK
-    if (role < 2) bwd_body<1, true, true>(p, smem, bh, role);
-    else if (role == 2) bwd_body<2, true, true>(p, smem, bh, 0);
-    else bwd_finish_dxk(p, smem, bh);
-  } else if (p.n_replay == 2) {
-    if (role < 2) bwd_body<1, true, false>(p, smem, bh, role);
-    else bwd_body<2, true, false>(p, smem, bh, 0);
-  } else {
-    if (role < 1) bwd_body<1, false, false>(p, smem, bh, 0);
-    else bwd_body<2, false, false>(p, smem, bh, 0);
-  }
+  constexpr bool IMG = NREPLAY == 2;   // two replaying workgroups also evaluate the GELU family for the walk
+  if (role < NREPLAY) bwd_body<1, IMG, FINISH>(p, smem, bh, role);
+  else if (role == NREPLAY) bwd_body<2, IMG, FINISH>(p, smem, bh, 0);
+  else if constexpr (FINISH) bwd_finish_dxk(p, smem, bh);
 }
 
 __global__ void ttt_mlp_zero_words(int* w, int n) {
@@ -1435,12 +1430,17 @@ hipError_t ttt_mlp_bwd_enqueue(const ttt::BwdParams& p, hipStream_t stream) {
     hipLaunchKernelGGL(ttt::ttt_mlp_bwd_kernel, dim3(p.nbh), dim3(ttt::BW_THREADS), ttt::SM_BWD_BYTES, stream, p);
     return hipGetLastError();
   }
-  e = hipFuncSetAttribute(reinterpret_cast<const void*>(ttt::ttt_mlp_bwd_split_kernel),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, ttt::SM_BWD_BYTES);
-  if (e != hipSuccess) return e;
   const int n = static_cast<int>(ttt::bwd_sync_ints(p.nbh));
   int* const words = p.status - (size_t)p.nbh * ttt::BWD_SYNC_STRIDE;   // p.sync itself is moved back by bh0 entries
   hipLaunchKernelGGL(ttt::ttt_mlp_zero_words, dim3((n + 255) / 256), dim3(256), 0, stream, words, n);
-  hipLaunchKernelGGL(ttt::ttt_mlp_bwd_split_kernel, dim3((p.n_replay + 1 + p.n_finish) * p.nbh), dim3(ttt::BW_THREADS), ttt::SM_BWD_BYTES, stream, p);
-  return hipGetLastError();
+  const dim3 grid((p.n_replay + 1 + p.n_finish) * p.nbh), block(ttt::BW_THREADS);
+  auto launch = [&](auto kernel) -> hipError_t {
+    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, ttt::SM_BWD_BYTES);
+    if (err != hipSuccess) return err;
+    hipLaunchKernelGGL(kernel, grid, block, ttt::SM_BWD_BYTES, stream, p);
+    return hipGetLastError();
+  };
+  if (p.n_finish) return launch(ttt::ttt_mlp_bwd_split_kernel<2, true>);
+  if (p.n_replay == 2) return launch(ttt::ttt_mlp_bwd_split_kernel<2, false>);
+  return launch(ttt::ttt_mlp_bwd_split_kernel<1, false>);
 }
