@@ -33,7 +33,7 @@ WORKLOADS = {
     "c5": (8, 48, 512, 32, 2.0, "fwd+bwd B=8 NH=48 32,768 tokens/sequence cgs=32 (fill-the-chip)"),
 }
 # HBM bytes per backward launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/), or None.
-MEASURED_TRAFFIC_BYTES = {"c4": 1.99e11}    # FETCH_SIZE 47,533,500 KiB x 2.0 + WRITE_SIZE 99,104,600 KiB x 1.0
+MEASURED_TRAFFIC_BYTES = {"c4": 1.97e11}    # FETCH_SIZE 47,472,500 KiB x 2.0 + WRITE_SIZE 99,813,800 KiB x 1.0
 
 
 def make_device_inputs(B, NH, NC, eta_std, dev):
@@ -152,7 +152,17 @@ def main():
     bwd_tflops = BWD_G * G_FLOP * mb_steps / (bwd_ms * 1e-3) / 1e12
     fwd_tflops = FWD_G * G_FLOP * mb_steps / (fwd_ms * 1e-3) / 1e12
     all_tflops = (FWD_G + BWD_G) * G_FLOP * mb_steps / (ms_per_step * 1e-3) / 1e12
-    bwd_kernel = "ttt_mlp_bwd_split_kernel" if ext.last_backward_mode() == 1 else "ttt_mlp_bwd_kernel"
+    # one kernel per combination of roles: ttt_mlp_bwd_split_kernel<replaying workgroups, grad_L_XK workgroup>
+    bwd_kernel = "ttt_mlp_bwd_kernel"
+    if ext.last_backward_mode() == 1:
+        import ctypes
+        lib = ctypes.CDLL(os.path.join(os.path.dirname(os.path.abspath(host.__file__)), "libttt_mlp.so"))
+        one, rest, per = ctypes.c_longlong(), ctypes.c_longlong(), ctypes.c_int()
+        cus = torch.cuda.get_device_properties(dev).multi_processor_count
+        lib.ttt_mlp_launch_plan(1, ctypes.c_longlong(B * NH), cus, ctypes.byref(one), ctypes.byref(rest), ctypes.byref(per))
+        bwd_kernel = f"ttt_mlp_bwd_split_kernel<{2 if per.value >= 3 else 1}, {'true' if per.value == 4 else 'false'}>"
+        if one.value:
+            bwd_kernel = "ttt_mlp_bwd_kernel + " + bwd_kernel
     out = {
         "metric": "TTT-MLP fwd+bwd tokens/sec on 1 MI355X (B=1,NH=48,256K tok); % bf16 MFMA peak",
         "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
