@@ -156,7 +156,8 @@ size_t ttt_mlp_bwd_status_offset(int32_t B, int32_t NH);
 /* The forward with two workgroups per (batch, head), under the same conditions and with the same
  * conventions (launches, workspace, status word at int index n*32, TTT_MLP_ERR_NO_ROOM, bit-identical
  * results): one workgroup carries the state through the mini-batches and leaves every new state
- * in the workspace as bf16 operands, the other computes Out from them, eight mini-batches behind.
+ * in the workspace as bf16 operands, the other computes Out from them, 8 mini-batches behind
+ * (32 when NC >= 512).
  * Used only when all pairs fit at two workgroups each (2*B*NH <= CUs): behind full rounds the
  * forward gains nothing from it.
  * No counterpart in the reference launcher (kernels/ttt/ttt.cu:594-721). */
@@ -164,6 +165,20 @@ size_t ttt_mlp_fwd_workspace_bytes(int32_t B, int32_t NH);
 size_t ttt_mlp_fwd_status_offset(int32_t B, int32_t NH);
 int ttt_mlp_fwd_launch_overlapped(const ttt_mlp_fwd_args* args, void* workspace, size_t workspace_bytes, void* stream);
 int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* args, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Optional: fills the sixteen *_group tensors with the values of checkpoint group 0 (the group the
+ * backward processes last) in the layouts of the struct above, as the reference's kernel leaves them
+ * (kernels/ttt_backward/ttt.cu:518-521, 551-552, 607-610, 636-637, 669, 699, 744-745, 798-800; its
+ * harness compares them, kernels/ttt_backward/matching.py:667-690).  Slot i holds, for mini-batch i:
+ * the state before it (W1/b1/W2/b2_init_group), Z1, X2 = gelu(Z1), the LayerNorm-fused loss
+ * gradient's x_hat / std / grad_output / grad_x_hat (*_fused_group), grad_l_wrt_Z2, grad_l_wrt_Z1,
+ * and of the output branch with the state after it Z1_bar, X2_bar and the LayerNorm's x_hat / std
+ * (*_ln_group).  The backward launchers use these tensors as workspace in formats of their own, so
+ * this is a separate, slower kernel (fp32 on the vector units, values rounded only when stored) that
+ * replays group 0 from checkpoint 0: enqueue it behind the backward on the same stream.  Reads XQ,
+ * XK, XV, last_eta, the norm parameters and the checkpoints; slots of mini-batches beyond NC are
+ * left as they are.  Takes the argument struct of ttt_mlp_bwd_launch and validates it the same way. */
+int ttt_mlp_bwd_export_group0(const ttt_mlp_bwd_args* args, void* stream);
 
 /* How long a workgroup of an overlapped launch waits for another before it gives up and raises the
  * status word, in ticks of the GPU's 100 MHz clock (default 2,000,000,000 = 20 s).  Process-wide; meant

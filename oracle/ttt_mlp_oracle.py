@@ -30,6 +30,10 @@ How each function is pinned (none of it by retyping its own formula):
   forward_step         autograd of sum_t eta_t * loss_t wrt (W1,b1,W2,b2) gives the step;
                        eta = 0 collapses to Out = XQ + LN(MLP(XQ))
   ttt_forward          checkpoint invariants + composition of the above
+  replay_group_tensors the values it copies out of forward_step are the ones backward_step consumes
+                       (pinned by the gradients below); slot 0 of the state tensors = the checkpoint,
+                       slot i+1 = slot i after the step; x_hat rows have mean 0 / variance 1,
+                       X2 = gelu(Z1); grad_l_wrt_Z2 = autograd of the loss at that slot's Z2
   backward_step /      torch.autograd straight through ``ttt_forward_differentiable`` in
   ttt_backward         fp64 (all ten gradients), invariance to checkpoint_group_size,
                        linearity in the upstream grads, finite differences at NC = 2
@@ -349,6 +353,41 @@ def ttt_backward(XQ, XK, XV, last_eta, ttt_norm_weight, ttt_norm_bias, ckpt: Sta
     return dict(grad_L_ttt_norm_weight=d_gamma, grad_L_ttt_norm_bias=d_beta,
                 grad_L_W1_init=g.W1, grad_L_b1_init=g.b1, grad_L_W2_init=g.W2, grad_L_b2_init=g.b2,
                 grad_L_last_eta=dEta, grad_L_XQ=dXQ, grad_L_XK=dXK, grad_L_XV=dXV)
+
+
+# ------------------------------------------------- per-group tensors of one checkpoint group
+GROUP_TENSOR_FROM_SAVED = dict(
+    Z1_group="Z1", X2_group="X2", Z1_bar_group="Z1b", X2_bar_group="X2b",
+    grad_l_wrt_Z2_group="gZ2", grad_l_wrt_Z1_group="gZ1",
+    x_hat_fused_group="xhat_f", std_fused_group="std_f", grad_output_fused_group="g_out",
+    grad_x_hat_fused_group="g_xhat", x_hat_ln_group="xhat_l", std_ln_group="std_l")
+
+
+def replay_group_tensors(XQ, XK, XV, last_eta, ttt_norm_weight, ttt_norm_bias, ckpt: State,
+                         checkpoint_group_size: int, group: int = 0, *, dtype=torch.float32):
+    """The sixteen ``*_group`` tensors of ``ttt_backward`` as the upstream harness fills its reference copies
+    for one checkpoint group (kernels/ttt_backward/matching.py:552-590; after the call the kernel's tensors
+    hold group 0, compared at :667-690): slot i = state before mini-batch i of the group and the
+    intermediates of its step.  Slots past the end of the sequence stay zero.  Shapes [B,NH,cgs,..]."""
+    XQ, XK, XV = XQ.to(dtype), XK.to(dtype), XV.to(dtype)
+    eta = _eta5(last_eta).to(dtype)
+    gamma, beta = _norm_params(ttt_norm_weight, ttt_norm_bias, dtype)
+    B, NH, NC, CS, F = XQ.shape
+    cgs = int(checkpoint_group_size)
+    st = State(*[t[:, :, group].to(dtype) for t in ckpt])
+    H = st.W1.shape[-1]
+    out = dict(W1_init_group=torch.zeros(B, NH, cgs, F, H, dtype=dtype), b1_init_group=torch.zeros(B, NH, cgs, 1, H, dtype=dtype),
+               W2_init_group=torch.zeros(B, NH, cgs, H, F, dtype=dtype), b2_init_group=torch.zeros(B, NH, cgs, 1, F, dtype=dtype))
+    for name, key in GROUP_TENSOR_FROM_SAVED.items():
+        last = 1 if key.startswith("std") else (F if key in ("gZ2", "xhat_f", "g_out", "g_xhat", "xhat_l") else H)
+        out[name] = torch.zeros(B, NH, cgs, CS, last, dtype=dtype)
+    for slot, i in enumerate(range(group * cgs, min(NC, (group + 1) * cgs))):
+        for name, t in zip(("W1_init_group", "b1_init_group", "W2_init_group", "b2_init_group"), st):
+            out[name][:, :, slot] = t
+        _, st, sv = forward_step(st, XQ[:, :, i], XK[:, :, i], XV[:, :, i], eta[:, :, i], gamma, beta)
+        for name, key in GROUP_TENSOR_FROM_SAVED.items():
+            out[name][:, :, slot] = sv[key]
+    return out
 
 
 # ----------------------------------------------------------- synthetic workloads

@@ -28,11 +28,11 @@ def lib():
 def declared_functions():
     src = open(HEADER).read()
     src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
-    return sorted(set(re.findall(r"\b(ttt_mlp_[a-z_]+)\s*\(", src)))
+    return sorted(set(re.findall(r"\b(ttt_mlp_[a-z0-9_]+)\s*\(", src)))
 
 
 def test_header_declares_the_expected_entry_points():
-    assert declared_functions() == ["ttt_mlp_abi_version", "ttt_mlp_bwd_launch", "ttt_mlp_bwd_launch_overlapped",
+    assert declared_functions() == ["ttt_mlp_abi_version", "ttt_mlp_bwd_export_group0", "ttt_mlp_bwd_launch", "ttt_mlp_bwd_launch_overlapped",
                                     "ttt_mlp_bwd_status_offset", "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_error_string",
                                     "ttt_mlp_fwd_launch", "ttt_mlp_fwd_launch_overlapped", "ttt_mlp_fwd_status_offset",
                                     "ttt_mlp_fwd_workspace_bytes", "ttt_mlp_kernel_info", "ttt_mlp_launch_plan", "ttt_mlp_set_wait_limit"]
@@ -199,3 +199,7 @@ def test_launch_plan_keeps_waiting_workgroups_within_the_device(lib):
                 assert rest * per <= cus
                 assert per in ((0, 2) if which == 0 else (0, 2, 3, 4))
     assert lib.ttt_mlp_launch_plan(2, ctypes.c_longlong(1), 1, None, None, None) == 1001
+
+
+def test_export_of_group_zero_validates_like_the_backward(lib):
+    assert lib.ttt_mlp_bwd_export_group0(None, None) == 1001

@@ -233,3 +233,55 @@ def test_bf16_operand_variant_stays_close_to_fp32_oracle():
     st = orc.parity_stats(b, a)
     assert st["max_rel"] < 2e-2 and st["cosine"] > 0.9999
     assert orc.parity_stats(ckb.W1, cka.W1)["cosine"] > 0.9999
+
+
+# ------------------------------------------------- per-group tensors (what the kernel leaves for group 0)
+@pytest.mark.parametrize("NC,cgs,group", [(5, 2, 0), (5, 2, 2), (3, 4, 0), (4, 4, 0)])
+def test_group_tensors_match_library_routines_and_autograd(NC, cgs, group):
+    """Every slot of replay_group_tensors, rebuilt from PyTorch's own gelu / layer_norm / autograd and from the
+    per-mini-batch states that ttt_forward's checkpoints give at checkpoint_group_size = 1."""
+    Fn = torch.nn.functional
+    d, _ = _small(NC=NC, seed=7)
+    out, ck, fin = orc.ttt_forward(*[d[k] for k in FWD_KEYS], cgs, dtype=F64)
+    _, ck1, _ = orc.ttt_forward(*[d[k] for k in FWD_KEYS], 1, dtype=F64)       # state before every mini-batch
+    states = [orc.State(*[t[:, :, i] for t in ck1]) for i in range(NC)] + [fin]
+    got = orc.replay_group_tensors(d["XQ"], d["XK"], d["XV"], d["last_eta"], d["ttt_norm_weight"], d["ttt_norm_bias"],
+                                   ck, cgs, group, dtype=F64)
+    gamma, beta = d["ttt_norm_weight"], d["ttt_norm_bias"]
+    Fdim = d["XQ"].shape[-1]
+    n = min(NC, (group + 1) * cgs) - group * cgs
+    for slot in range(cgs):
+        if slot >= n:
+            for name, v in got.items():
+                assert not v[:, :, slot].any(), name
+            continue
+        i = group * cgs + slot
+        st, nxt = states[i], states[i + 1]
+        xq, xk, xv = d["XQ"][:, :, i], d["XK"][:, :, i], d["XV"][:, :, i]
+        for name, ref in zip(("W1_init_group", "b1_init_group", "W2_init_group", "b2_init_group"), st):
+            assert torch.equal(got[name][:, :, slot], ref), name
+        z1 = (xk @ st.W1 + st.b1).requires_grad_(True)
+        x2 = Fn.gelu(z1, approximate="tanh")
+        z2 = (x2 @ st.W2 + st.b2)
+        z2_leaf = z2.detach().requires_grad_(True)
+        xh_leaf = Fn.layer_norm(z2_leaf, (Fdim,), eps=orc.LN_EPS).detach().requires_grad_(True)
+        loss_from_xh = 0.5 * ((gamma * xh_leaf + beta - (xv - xk)) ** 2).sum()
+        g_xhat, = torch.autograd.grad(loss_from_xh, xh_leaf)
+        loss_from_z2 = 0.5 * ((gamma * Fn.layer_norm(z2_leaf, (Fdim,), eps=orc.LN_EPS) + beta - (xv - xk)) ** 2).sum()
+        g_z2, = torch.autograd.grad(loss_from_z2, z2_leaf)
+        loss_from_z1 = 0.5 * ((gamma * Fn.layer_norm(z2, (Fdim,), eps=orc.LN_EPS) + beta - (xv - xk)) ** 2).sum()
+        g_z1_total, = torch.autograd.grad(loss_from_z1, z1)
+        z1b = xq @ nxt.W1 + nxt.b1
+        x2b = Fn.gelu(z1b, approximate="tanh")
+        z2b = x2b @ nxt.W2 + nxt.b2
+        ref = dict(Z1_group=z1.detach(), X2_group=x2.detach(), grad_l_wrt_Z2_group=g_z2, grad_l_wrt_Z1_group=g_z1_total,
+                   x_hat_fused_group=xh_leaf.detach(),
+                   std_fused_group=torch.sqrt(z2.detach().var(dim=-1, unbiased=False, keepdim=True) + orc.LN_EPS),
+                   grad_output_fused_group=(gamma * xh_leaf + beta - (xv - xk)).detach(), grad_x_hat_fused_group=g_xhat,
+                   Z1_bar_group=z1b, X2_bar_group=x2b, x_hat_ln_group=Fn.layer_norm(z2b, (Fdim,), eps=orc.LN_EPS),
+                   std_ln_group=torch.sqrt(z2b.var(dim=-1, unbiased=False, keepdim=True) + orc.LN_EPS))
+        for name, r in ref.items():
+            assert got[name][:, :, slot].shape == r.shape, name
+            assert (got[name][:, :, slot] - r).abs().max() < 1e-8 * (1 + r.abs().max()), (name, slot)
+        # and the output the forward returns is the residual on top of this slot's output LayerNorm
+        assert (xq + gamma * got["x_hat_ln_group"][:, :, slot] + beta - out[:, :, i]).abs().max() < 1e-10

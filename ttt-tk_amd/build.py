@@ -22,7 +22,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libttt_mlp.so")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
-HIP_SOURCES = ["ttt_mlp_fwd.hip", "ttt_mlp_bwd.hip", "ttt_mlp_c_abi.hip"]
+HIP_SOURCES = ["ttt_mlp_fwd.hip", "ttt_mlp_bwd.hip", "ttt_mlp_export.hip", "ttt_mlp_c_abi.hip"]
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
              # packed-fp32 VALU forms are kept out of the generated code on purpose
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

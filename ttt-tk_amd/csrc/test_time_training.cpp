@@ -14,6 +14,7 @@ namespace {
 
 constexpr int64_t F = TTT_MLP_F, CS = TTT_MLP_CS, HID = TTT_MLP_HID;
 bool g_synchronize = true;  // upstream blocks the host until the kernel has finished
+bool g_fill_group_tensors = false;   // leave the values of checkpoint group 0 in the sixteen *_group tensors
 bool g_overlap = true;      // two workgroups per (batch, head) whenever they fit the device
 int g_last_forward_mode = -1;    // 0 = one workgroup per (batch, head), 1 = two
 int g_last_backward_mode = -1;
@@ -229,10 +230,14 @@ torch::Tensor ttt_backward(
     torch::Tensor ws = torch::empty({(int64_t)ws_bytes}, torch::TensorOptions().dtype(torch::kUInt8).device(XQ.device()));
     g_last_backward_mode = 1;
     const char* status = static_cast<const char*>(ws.data_ptr()) + ttt_mlp_bwd_status_offset((int32_t)B, (int32_t)NH);
-    finish(ttt_mlp_bwd_launch_overlapped(&a, ws.data_ptr(), ws_bytes, stream), stream, "ttt_backward", status);
+    int rc = ttt_mlp_bwd_launch_overlapped(&a, ws.data_ptr(), ws_bytes, stream);
+    if (rc == 0 && g_fill_group_tensors) rc = ttt_mlp_bwd_export_group0(&a, stream);
+    finish(rc, stream, "ttt_backward", status);
   } else {
     g_last_backward_mode = 0;
-    finish(ttt_mlp_bwd_launch(&a, stream), stream, "ttt_backward");
+    int rc = ttt_mlp_bwd_launch(&a, stream);
+    if (rc == 0 && g_fill_group_tensors) rc = ttt_mlp_bwd_export_group0(&a, stream);
+    finish(rc, stream, "ttt_backward");
   }
   return Out;
 }
@@ -249,6 +254,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("set_overlap", [](bool on) { g_overlap = on; },
         "Use a second workgroup per (batch, head) when the device has room: the forward's output branch, the "
         "backward's recomputation of checkpoint groups (default true).");
+  m.def("set_fill_group_tensors", [](bool on) { g_fill_group_tensors = on; },
+        "After ttt_backward, leave the values of checkpoint group 0 in the sixteen *_group tensors, row-major, as the "
+        "upstream kernel does (its harness compares them); costs one more, slower kernel (default false: the tensors "
+        "are workspace with unspecified contents).");
   m.def("set_wait_limit", [](unsigned long long ticks) { ttt_mlp_set_wait_limit(ticks); },
         "Ticks of the GPU's 100 MHz clock a workgroup waits for its partner before giving up (default 2e9 = 20 s).");
   m.def("last_forward_mode", []() { return g_last_forward_mode; },

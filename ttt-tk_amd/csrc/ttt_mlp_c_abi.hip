@@ -211,6 +211,14 @@ extern "C" int ttt_mlp_bwd_launch(const ttt_mlp_bwd_args* a, void* stream) {
   return static_cast<int>(ttt_mlp_bwd_enqueue(p, static_cast<hipStream_t>(stream)));
 }
 
+extern "C" int ttt_mlp_bwd_export_group0(const ttt_mlp_bwd_args* a, void* stream) {
+  ttt::BwdParams p;
+  if (int rc = make_bwd_params(a, p)) return rc;
+  p.bh0 = 0;
+  p.nbh = p.B * p.NH;
+  return static_cast<int>(ttt_mlp_export_group0_enqueue(p, static_cast<hipStream_t>(stream)));
+}
+
 extern "C" size_t ttt_mlp_bwd_workspace_bytes(int B, int NH, int checkpoint_group_size) {
   if (B <= 0 || NH <= 0 || checkpoint_group_size <= 0 || checkpoint_group_size > (1 << 16)) return 0;
   const LaunchPlan pl = plan_launches((long long)B * NH, true, true);

@@ -85,6 +85,8 @@ inline size_t bwd_sync_ints(long long BH) { return (size_t)BH * BWD_SYNC_STRIDE 
 hipError_t ttt_mlp_fwd_enqueue(const ttt::FwdParams& p, hipStream_t stream);
 // p.sync == nullptr: one workgroup per (batch, head); otherwise two (replay / reverse walk).
 hipError_t ttt_mlp_bwd_enqueue(const ttt::BwdParams& p, hipStream_t stream);
+// Replays checkpoint group 0 and writes the sixteen per-group tensors row-major (side path, one workgroup per pair).
+hipError_t ttt_mlp_export_group0_enqueue(const ttt::BwdParams& p, hipStream_t stream);
 extern "C" int ttt_mlp_fwd_lds_bytes();
 extern "C" int ttt_mlp_bwd_lds_bytes();
 extern "C" int ttt_mlp_fwd_threads();

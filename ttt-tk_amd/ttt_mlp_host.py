@@ -92,6 +92,18 @@ def set_synchronize(on: bool) -> None:
     _ext.set_synchronize(bool(on))
 
 
+GROUP_TENSORS = ("W1_init_group", "b1_init_group", "W2_init_group", "b2_init_group", "x_hat_ln_group", "std_ln_group",
+                 "X2_group", "Z1_group", "Z1_bar_group", "X2_bar_group", "grad_l_wrt_Z2_group", "grad_l_wrt_Z1_group",
+                 "x_hat_fused_group", "grad_x_hat_fused_group", "grad_output_fused_group", "std_fused_group")
+
+
+def set_fill_group_tensors(on: bool) -> None:
+    """After ``ttt_backward`` leave the values of checkpoint group 0 in the sixteen ``*_group`` tensors, as the
+    upstream kernel does (its harness compares them, kernels/ttt_backward/matching.py:667-690).  Off by default:
+    the kernels use those tensors as workspace in their own formats, filling them costs one more kernel."""
+    _ext.set_fill_group_tensors(bool(on))
+
+
 class TTTMLPFunction(torch.autograd.Function):
     """`Out = ttt_mlp(XQ, XK, XV, last_eta, ttt_norm_weight, ttt_norm_bias, W1, b1, W2, b2)` with the
     remat backward, as the usage block of the upstream README (README.md:22-96) and its test harness
