@@ -90,6 +90,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c4")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--overwrite", action="store_true",
+                    help="let ttt_backward overwrite grad_L_XQ / XK / XV / last_eta instead of adding to them "
+                         "(no zero-fill in the step; not the upstream calling convention, so not the default)")
     ap.add_argument("--no-overlap", action="store_true",
                     help="backward with one workgroup per (batch, head) even where two fit the device")
     ap.add_argument("--cpu-sample-mb", type=int, default=1536, help="mini-batches in the CPU baseline sample")
@@ -113,9 +116,11 @@ def main():
     host.set_synchronize(False)           # time with events; the operator's default host sync is not part of the kernel
     import test_time_training as ext
     ext.set_overlap(not a.no_overlap)
+    ext.set_accumulate(not a.overwrite)
 
     def step(ev=None):
-        host.zero_accumulating_grads(t)
+        if not a.overwrite:
+            host.zero_accumulating_grads(t)    # the operator adds to four of its outputs, as upstream does
         if ev:
             ev[0].record()
         host.forward(t, cgs)

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define TTT_MLP_ABI_VERSION 1
+#define TTT_MLP_ABI_VERSION 2
 
 #define TTT_MLP_CS 64   /* tokens per mini-batch        */
 #define TTT_MLP_F 64    /* head dimension               */
@@ -70,8 +70,8 @@ typedef struct ttt_mlp_fwd_args {
  * (test_time_training.cpp:47-91).  The sixteen *_group tensors are caller-owned
  * scratch of checkpoint_group_size mini-batches; the library uses them as
  * workspace and leaves their contents unspecified.  grad_L_last_eta / grad_L_XQ /
- * grad_L_XK / grad_L_XV are accumulated into (the caller zero-fills them), all
- * other outputs are overwritten.  `Out` is not touched. */
+ * grad_L_XK / grad_L_XV are accumulated into (the caller zero-fills them) unless
+ * `overwrite` is set, all other outputs are overwritten.  `Out` is not touched. */
 typedef struct ttt_mlp_bwd_args {
   const uint16_t* XQ;
   const uint16_t* XK;
@@ -117,6 +117,11 @@ typedef struct ttt_mlp_bwd_args {
   uint16_t* grad_L_XV;
   int32_t checkpoint_group_size;
   int32_t B, NH, NC, K;
+  /* 0: grad_L_last_eta / grad_L_XQ / grad_L_XK / grad_L_XV are added to, as the reference's kernel does with
+   * its four thread blocks per head (the caller zero-fills them, kernels/ttt_backward/matching.py:406-415).
+   * 1: they are overwritten - these kernels write every element exactly once, so the zero-fill and the
+   * read of the old value can both be left out.  Same values either way when the tensors start at zero. */
+  int32_t overwrite;
 } ttt_mlp_bwd_args;
 
 /* Version of this header the library was built against. */

@@ -41,7 +41,7 @@ def test_header_declares_the_expected_entry_points():
 def test_library_exports_every_declared_symbol(lib):
     for name in declared_functions():
         assert hasattr(lib, name), name
-    assert lib.ttt_mlp_abi_version() == 1
+    assert lib.ttt_mlp_abi_version() == 2
 
 
 def test_kernel_info_reports_lds_within_one_cu(lib):

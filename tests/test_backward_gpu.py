@@ -167,3 +167,43 @@ def test_overlapped_backward_is_bit_identical(B, NH, NC, cgs):
     for k in host.GRAD_NAMES:
         assert torch.isfinite(two[k]).all(), k
         assert torch.equal(one[k], two[k]), k
+
+
+@pytest.mark.parametrize("B,NH,NC,cgs,overlap", [(1, 2, 9, 2, True), (1, 2, 9, 2, False), (2, 3, 7, 4, True),
+                                                 (1, 96, 5, 2, True), (1, 72, 5, 2, True)])
+def test_overwrite_policy_matches_accumulation_into_zeros(B, NH, NC, cgs, overlap):
+    """set_accumulate(False): the four outputs the operator normally adds to are overwritten, whatever they held,
+    with exactly the values that adding to zeros gives (every element is written once), in every launch shape;
+    set_accumulate(True) adds to what is there."""
+    import ttt_mlp_host as host
+    import test_time_training as ext
+    print(f"case B={B} NH={NH} NC={NC} cgs={cgs} overlap={overlap}", flush=True)
+    d = orc.make_inputs(B, NH, NC, seed=77)
+    dev = torch.device("cuda:0")
+    names = ("grad_L_last_eta", "grad_L_XQ", "grad_L_XK", "grad_L_XV")
+
+    def run(accumulate, prefill):
+        t = {k: d[k].to(dev).contiguous() for k in FWD_KEYS + UP_KEYS}
+        t.update(host.alloc_forward_buffers(B, NH, NC, cgs, dev))
+        host.forward(t, cgs)
+        t.update(host.alloc_backward_buffers(B, NH, NC, cgs, dev))
+        for k in names:
+            t[k].fill_(prefill)
+        ext.set_overlap(overlap)
+        host.set_accumulate(accumulate)
+        try:
+            host.backward(t, cgs)
+        finally:
+            host.set_accumulate(True)
+            ext.set_overlap(True)
+        assert ext.last_backward_mode() == int(overlap)
+        return {k: t[k].clone() for k in host.GRAD_NAMES}
+
+    base = run(True, 0.0)
+    over = run(False, float("nan"))
+    for k in host.GRAD_NAMES:
+        assert torch.equal(base[k], over[k]), k
+    added = run(True, 0.5)
+    for k in names:
+        # the kernel rounds old + fp32 value once, base + 0.5 rounds twice: equal up to one bf16 step
+        assert torch.allclose(added[k].float(), base[k].float() + 0.5, rtol=2 ** -7, atol=2 ** -7), k

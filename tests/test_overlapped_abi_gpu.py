@@ -26,7 +26,8 @@ def _lib():
 
 def _args(order, t, cgs, B, NH, NC, K):
     class Args(ctypes.Structure):
-        _fields_ = [(n, ctypes.c_void_p) for n in order] + [(n, ctypes.c_int32) for n in SIZES]
+        _fields_ = [(n, ctypes.c_void_p) for n in order] + [(n, ctypes.c_int32) for n in SIZES] + \
+                   ([("overwrite", ctypes.c_int32)] if len(order) == 42 else [])    # the backward's struct ends with its policy flag
     return Args(*[t[k].data_ptr() for k in order], cgs, B, NH, NC, K)
 
 

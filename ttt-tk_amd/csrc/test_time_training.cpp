@@ -15,6 +15,7 @@ namespace {
 constexpr int64_t F = TTT_MLP_F, CS = TTT_MLP_CS, HID = TTT_MLP_HID;
 bool g_synchronize = true;  // upstream blocks the host until the kernel has finished
 bool g_fill_group_tensors = false;   // leave the values of checkpoint group 0 in the sixteen *_group tensors
+bool g_accumulate = true;            // grad_L_XQ / XK / XV / last_eta are added to (upstream behaviour) rather than overwritten
 bool g_overlap = true;      // two workgroups per (batch, head) whenever they fit the device
 int g_last_forward_mode = -1;    // 0 = one workgroup per (batch, head), 1 = two
 int g_last_backward_mode = -1;
@@ -220,6 +221,7 @@ torch::Tensor ttt_backward(
   a.grad_L_XQ = bfp_mut(grad_L_XQ); a.grad_L_XK = bfp_mut(grad_L_XK); a.grad_L_XV = bfp_mut(grad_L_XV);
   a.checkpoint_group_size = checkpoint_group_size;
   a.B = (int32_t)B; a.NH = (int32_t)NH; a.NC = (int32_t)NC; a.K = (int32_t)K;
+  a.overwrite = g_accumulate ? 0 : 1;
   const c10::DeviceGuard guard(XQ.device());
   hipStream_t stream = c10::hip::getCurrentHIPStream(XQ.device().index()).stream();
   // With few (batch, head) pairs most CUs would idle: then a second workgroup per pair recomputes the
@@ -258,6 +260,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "After ttt_backward, leave the values of checkpoint group 0 in the sixteen *_group tensors, row-major, as the "
         "upstream kernel does (its harness compares them); costs one more, slower kernel (default false: the tensors "
         "are workspace with unspecified contents).");
+  m.def("set_accumulate", [](bool on) { g_accumulate = on; },
+        "True (default, the upstream behaviour): ttt_backward adds to grad_L_last_eta / grad_L_XQ / grad_L_XK / "
+        "grad_L_XV, which the caller zero-fills.  False: it overwrites them - no zero-fill needed, and the kernels "
+        "skip the read of the old values.");
+  m.def("get_accumulate", []() { return g_accumulate; });
   m.def("set_wait_limit", [](unsigned long long ticks) { ttt_mlp_set_wait_limit(ticks); },
         "Ticks of the GPU's 100 MHz clock a workgroup waits for its partner before giving up (default 2e9 = 20 s).");
   m.def("last_forward_mode", []() { return g_last_forward_mode; },

@@ -40,6 +40,10 @@
 
 namespace ttt {
 
+// Zeros standing in for the old contents of an output tile (8 KiB) when the outputs are overwritten rather
+// than added to: the load stays where it is in the instruction stream and is served by the L2.
+__device__ __attribute__((aligned(256))) const uint4 zero_tile[512] = {};
+
 constexpr int BW_NWAVE = 8;
 constexpr int BW_THREADS = 64 * BW_NWAVE;
 constexpr int BW_NS = HID / BW_NWAVE;     // hidden columns per wave: 32
@@ -514,6 +518,8 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
 #define bDXK gbuf(ka->grad_L_XK + ox)
 #define bDXV gbuf(ka->grad_L_XV + ox)
 #define bDETA gbuf(ka->grad_L_last_eta + oe)
+// what an accumulating output held before: the tile itself, or zeros when the outputs are overwritten
+#define OLD_VALUE(buf, off) (ka->overwrite ? gbuf(zero_tile) : (buf)), vln, (ka->overwrite ? 0u : (off))
   const unsigned t16 = 16 * tid, vln = (tok * FD + f0) * 2, vtok = 4 * tok;
   // Everything derived from the lane index is cheap to recompute and expensive to keep: a value
   // computed once before the loops is held in a register (or spilled and reloaded) for the whole
@@ -853,7 +859,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           WAVE_SYNC();   // every reader of T1 / T2 is done before the pair sum takes their place
           {
             LANE_VARS;
-            dxq_old = g_ld_stream<bf16x8>(bDXQ, vln, mb * TILE_BYTES);   // under way during the pair sum
+            dxq_old = g_ld_stream<bf16x8>(OLD_VALUE(bDXQ, mb * TILE_BYTES));   // under way during the pair sum
           }
           pair_sum(s_own, s_partner, dq, c, h);
         }
@@ -1064,8 +1070,8 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         WAVE_SYNC();   // this wave's readers of T1 / T2 are done
         {   // what the LayerNorm stage reads from HBM is under way during the pair sum
           LANE_VARS;
-          dxv_old = g_ld_stream<bf16x8>(bDXV, vln, xo);
-          deta_old = g_ldh(bDETA, 2 * tok, mb * (CS * 2));
+          dxv_old = g_ld_stream<bf16x8>(OLD_VALUE(bDXV, xo));
+          deta_old = g_ldh(ka->overwrite ? gbuf(zero_tile) : bDETA, 2 * tok, ka->overwrite ? 0u : mb * (CS * 2));
           xhf_n = ROLE != 0 ? g_ld_stream<bf16x8>(bXHF, vln, so) : g_ld8h(bXHF, vln, so);
           gof_n = ROLE != 0 ? g_ld_stream<bf16x8>(bGOF, vln, so) : g_ld8h(bGOF, vln, so);
           sdf_n = g_ldf(bSDF, vtok, j * (CS * 4));
@@ -1238,7 +1244,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         if constexpr (!FIN) {
           {
             LANE_VARS;
-            dxk_old = g_ld_stream<bf16x8>(bDXK, vln, xo);   // under way during the pair sum
+            dxk_old = g_ld_stream<bf16x8>(OLD_VALUE(bDXK, xo));   // under way during the pair sum
           }
           pair_sum(s_own, s_partner, dk, c, h);
         }
@@ -1355,7 +1361,7 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
     const unsigned ckW = k * (FD * HID * 4);
     for (int j = n_mb - 1; j >= 0; j--) {
       const unsigned xo = (k * cgs + j) * TILE_BYTES, so = j * TILE_BYTES, ho = j * IMG_BYTES;
-      const bf16x8 dxk_ld = g_ld_stream<bf16x8>(gDXK, vln, xo);
+      const bf16x8 dxk_ld = g_ld_stream<bf16x8>(p.overwrite ? gbuf(zero_tile) : gDXK, vln, p.overwrite ? 0u : xo);
       const f32x4 gy_lo = g_ld_stream<f32x4>(gGY, 2 * vln, 2 * so), gy_hi = g_ld_stream<f32x4>(gGY, 2 * vln + 16, 2 * so);
       bf16x8 gw[2][2], g1[2][2], dz[2][2], w1b[2][2];
 #pragma unroll

@@ -112,6 +112,7 @@ int make_bwd_params(const ttt_mlp_bwd_args* a, ttt::BwdParams& p) {
   p.grad_L_last_eta = bf(a->grad_L_last_eta);
   p.grad_L_XQ = bf(a->grad_L_XQ); p.grad_L_XK = bf(a->grad_L_XK); p.grad_L_XV = bf(a->grad_L_XV);
   p.B = a->B; p.NH = a->NH; p.NC = a->NC; p.K = a->K; p.cgs = a->checkpoint_group_size;
+  p.overwrite = a->overwrite != 0;
   return TTT_MLP_OK;
 }
 

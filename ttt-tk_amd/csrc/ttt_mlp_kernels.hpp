@@ -69,6 +69,7 @@ struct BwdParams {
   int* sync;
   int* status;    // the status word behind the synchronisation words
   unsigned long long wait_limit;   // ticks of the 100 MHz clock a workgroup waits for another before it gives up
+  int overwrite;  // non-zero: grad_L_XQ / XK / XV / last_eta are stored, not added to (every element is written exactly once)
   int bh0, nbh;   // this launch covers (batch, head) pairs bh0 .. bh0 + nbh - 1 (workspace pointers moved back by bh0 entries)
 };
 

@@ -53,8 +53,10 @@ def alloc_forward_buffers(B: int, NH: int, NC: int, cgs: int, device) -> Dict[st
                 Out=torch.empty(B, NH, NC, CS, F, dtype=torch.bfloat16, device=device))
 
 
-def alloc_backward_buffers(B: int, NH: int, NC: int, cgs: int, device) -> Dict[str, torch.Tensor]:
-    """The sixteen remat scratch tensors, and the ten output gradients (accumulating ones zeroed)."""
+def alloc_backward_buffers(B: int, NH: int, NC: int, cgs: int, device, zero_fill: bool = True) -> Dict[str, torch.Tensor]:
+    """The sixteen remat scratch tensors, and the ten output gradients.  The four that `ttt_backward` adds to are
+    zero-filled unless ``zero_fill`` is False (for the operator's overwrite policy, `set_accumulate(False)`)."""
+    acc = torch.zeros if zero_fill else torch.empty
     f32 = dict(dtype=torch.float32, device=device)
     bf = dict(dtype=torch.bfloat16, device=device)
     G = cgs
@@ -70,8 +72,8 @@ def alloc_backward_buffers(B: int, NH: int, NC: int, cgs: int, device) -> Dict[s
         grad_L_ttt_norm_weight=torch.empty(B, NH, 1, F, **f32), grad_L_ttt_norm_bias=torch.empty(B, NH, 1, F, **f32),
         grad_L_W1_init=torch.empty(B, NH, F, HID, **f32), grad_L_b1_init=torch.empty(B, NH, 1, HID, **f32),
         grad_L_W2_init=torch.empty(B, NH, HID, F, **f32), grad_L_b2_init=torch.empty(B, NH, 1, F, **f32),
-        grad_L_last_eta=torch.zeros(B, NH, NC, CS, 1, **bf), grad_L_XQ=torch.zeros(B, NH, NC, CS, F, **bf),
-        grad_L_XK=torch.zeros(B, NH, NC, CS, F, **bf), grad_L_XV=torch.zeros(B, NH, NC, CS, F, **bf))
+        grad_L_last_eta=acc(B, NH, NC, CS, 1, **bf), grad_L_XQ=acc(B, NH, NC, CS, F, **bf),
+        grad_L_XK=acc(B, NH, NC, CS, F, **bf), grad_L_XV=acc(B, NH, NC, CS, F, **bf))
     return d
 
 
@@ -95,6 +97,13 @@ def set_synchronize(on: bool) -> None:
 GROUP_TENSORS = ("W1_init_group", "b1_init_group", "W2_init_group", "b2_init_group", "x_hat_ln_group", "std_ln_group",
                  "X2_group", "Z1_group", "Z1_bar_group", "X2_bar_group", "grad_l_wrt_Z2_group", "grad_l_wrt_Z1_group",
                  "x_hat_fused_group", "grad_x_hat_fused_group", "grad_output_fused_group", "std_fused_group")
+
+
+def set_accumulate(on: bool) -> None:
+    """True (default, upstream behaviour, kernels/ttt_backward/matching.py:406-415): `ttt_backward` adds to
+    grad_L_last_eta / grad_L_XQ / grad_L_XK / grad_L_XV and the caller zero-fills them.  False: it overwrites
+    them; `ttt_mlp` / `ttt_mlp_backward` then allocate them without the fill."""
+    _ext.set_accumulate(bool(on))
 
 
 def set_fill_group_tensors(on: bool) -> None:
@@ -158,7 +167,7 @@ def ttt_mlp_backward(XQ, XK, XV, last_eta, ttt_norm_weight, ttt_norm_bias, check
     for name, gl in zip(("grad_L_W1_last", "grad_L_b1_last", "grad_L_W2_last", "grad_L_b2_last"), grad_last):
         t[name] = gl.to(torch.float32).contiguous()
     t["Out"] = torch.empty(B, NH, NC, CS, F, dtype=torch.bfloat16, device=dev)   # unused by the operator, must exist
-    t.update(alloc_backward_buffers(B, NH, NC, cgs, dev))
+    t.update(alloc_backward_buffers(B, NH, NC, cgs, dev, zero_fill=_ext.get_accumulate()))
     backward(t, cgs)
     return {k: t[k] for k in GRAD_NAMES}
 
