@@ -1,4 +1,4 @@
-"""BASELINE's configurations at their full sizes on the GPU.
+"""The benchmark configurations (C2 - C5) at their full sizes on the GPU.
 
 C2/C3 (16,384 tokens, 48 heads) are checked against the CPU oracle for every head.  C4 (262,144 tokens)
 and C5 (8 x 48 recurrences) run in full on the GPU; the oracle, which needs minutes for them, checks a
