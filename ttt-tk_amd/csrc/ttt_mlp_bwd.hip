@@ -909,7 +909,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
 #define bFGW gbuf(ka->fin_gw1 + ofin * (CS * HID))
 #define bFG1 gbuf(ka->fin_g1 + ofin * (CS * HID))
 #define bFDZ gbuf(ka->fin_dz + ofin * (CS * HID))
-#define bFGY gbuf(ka->fin_gy + ofin * (CS * FD))
+#define bFGY gbuf(ka->fin_gy + ofin * (2 * CS * FD))
     if constexpr (ROLE != 1)
     for (int j = n_mb - 1; j >= 0; j--) {
       const int mb = k * cgs + j;
@@ -1070,7 +1070,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         WAVE_SYNC();   // this wave's readers of T1 / T2 are done
         {   // what the LayerNorm stage reads from HBM is under way during the pair sum
           LANE_VARS;
-          dxv_old = g_ld_stream<bf16x8>(OLD_VALUE(bDXV, xo));
+          if constexpr (!FIN) dxv_old = g_ld_stream<bf16x8>(OLD_VALUE(bDXV, xo));
           deta_old = g_ldh(ka->overwrite ? gbuf(zero_tile) : bDETA, 2 * tok, ka->overwrite ? 0u : mb * (CS * 2));
           xhf_n = ROLE != 0 ? g_ld_stream<bf16x8>(bXHF, vln, so) : g_ld8h(bXHF, vln, so);
           gof_n = ROLE != 0 ? g_ld_stream<bf16x8>(bGOF, vln, so) : g_ld8h(bGOF, vln, so);
@@ -1124,27 +1124,32 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         }
         sg = oct_sum(sg);
         sx = oct_sum(sx);
-        ln_token_sum_add(s_dgw, dg, q8, f0);
-        ln_token_sum_add(s_dbw, gy, q8, f0);
+        if constexpr (!FIN) {   // with a grad_L_XK workgroup these token sums and grad_L_XV are formed there, from g_y and dg
+          ln_token_sum_add(s_dgw, dg, q8, f0);
+          ln_token_sum_add(s_dbw, gy, q8, f0);
+        }
 #pragma unroll
         for (int e = 0; e < 8; e++) {
           gx[e] = gx[e] * rsd + (sg * xh[e] - sx * rsd) * (1.f / FD);   // dZ2
-          dxv_old[e] = (bf16)((float)dxv_old[e] - gy[e]);                // dXV accumulates -g_y
+          if constexpr (!FIN) dxv_old[e] = (bf16)((float)dxv_old[e] - gy[e]);   // dXV accumulates -g_y
         }
         // g_y is needed again for dXK: park it (the XQ / E2 tiles are dead by now), or hand it over
         {
           LANE_VARS;
           f32x4 lo = {gy[0], gy[1], gy[2], gy[3]}, hi = {gy[4], gy[5], gy[6], gy[7]};
           if constexpr (FIN) {
-            g_st_stream<f32x4>(bFGY, 2 * vln, 2 * so, lo);
-            g_st_stream<f32x4>(bFGY, 2 * vln + 16, 2 * so, hi);
+            g_st_stream<f32x4>(bFGY, 2 * vln, 4 * so, lo);
+            g_st_stream<f32x4>(bFGY, 2 * vln + 16, 4 * so, hi);
+            f32x4 dlo = {dg[0], dg[1], dg[2], dg[3]}, dhi = {dg[4], dg[5], dg[6], dg[7]};
+            g_st_stream<f32x4>(bFGY, 2 * vln, 4 * so + 2 * TILE_BYTES, dlo);
+            g_st_stream<f32x4>(bFGY, 2 * vln + 16, 4 * so + 2 * TILE_BYTES, dhi);
           } else {
             *reinterpret_cast<f32x4*>(s_gy) = lo;
             *reinterpret_cast<f32x4*>(s_gy + 4) = hi;
           }
         }
         ln_store(s_a + tok * LDX + f0, gx);
-        g_st_stream<bf16x8>(bDXV, vln, xo, dxv_old);
+        if constexpr (!FIN) g_st_stream<bf16x8>(bDXV, vln, xo, dxv_old);
       }
       __syncthreads();  // dZ2 tile complete; regions (T1 / T2) free again
 
@@ -1278,6 +1283,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
   // The replay's two sums: parked in HBM by this workgroup, or handed over by the replaying workgroups, whose
   // last counts this workgroup has acquired (a second replaying workgroup has nothing to hand over if there is
   // one group only).
+  if constexpr (FIN) return;   // with a grad_L_XK workgroup the walk holds no share of these sums: they are written there
   if (tid < 2 * FD) {
     const int which = tid / FD, f = tid % FD;
     const float* rp = ROLE == 0 ? reinterpret_cast<const float*>(p.x_hat_ln_group + (size_t)bh * cgs * (CS * FD))
@@ -1349,20 +1355,29 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
   int* const w_finished = w_sync + 24;
   int* const s_flag = reinterpret_cast<int*>(smem + SB_FLAG);
   const gptr_t gDXK = gbuf(p.grad_L_XK + uni64((size_t)bh * p.NC * (CS * FD)));
+  const gptr_t gDXV = gbuf(p.grad_L_XV + uni64((size_t)bh * p.NC * (CS * FD)));
   const gptr_t gCW1 = gbuf(p.W1_ck + uni64((size_t)bh * p.K * (FD * HID)));
+  // the walk's share of the norm-weight / norm-bias gradients: per wave, summed in the walk's order
+  float* s_red = reinterpret_cast<float*>(smem + SB_RED);
+  float* s_dgw = s_red + (v * 2 + 0) * FD;
+  float* s_dbw = s_red + (v * 2 + 1) * FD;
+  if (lane < FD) { s_dgw[lane] = 0.f; s_dbw[lane] = 0.f; }
   for (int k = p.K - 1; k >= 0; k--) {
     const int n_mb = min(cgs, p.NC - k * cgs);
     const int done = p.K - 1 - k, set = done % n_sets;
     if (!wait_at_least(w_walked, done + 1, p.status, s_flag, p.wait_limit)) return;
     const size_t ofin = uni64(((size_t)bh * 2 + (done & 1)) * cgs);
     const gptr_t gGW = gbuf(p.fin_gw1 + ofin * (CS * HID)), gG1 = gbuf(p.fin_g1 + ofin * (CS * HID));
-    const gptr_t gDZ = gbuf(p.fin_dz + ofin * (CS * HID)), gGY = gbuf(p.fin_gy + ofin * (CS * FD));
+    const gptr_t gDZ = gbuf(p.fin_dz + ofin * (CS * HID)), gGY = gbuf(p.fin_gy + ofin * (2 * CS * FD));
     const gptr_t gIMG1 = gbuf((set ? p.alt_X2_group[set - 1] : p.X2_group) + uni64((size_t)bh * cgs * (CS * HID)));
     const unsigned ckW = k * (FD * HID * 4);
     for (int j = n_mb - 1; j >= 0; j--) {
       const unsigned xo = (k * cgs + j) * TILE_BYTES, so = j * TILE_BYTES, ho = j * IMG_BYTES;
       const bf16x8 dxk_ld = g_ld_stream<bf16x8>(p.overwrite ? gbuf(zero_tile) : gDXK, vln, p.overwrite ? 0u : xo);
-      const f32x4 gy_lo = g_ld_stream<f32x4>(gGY, 2 * vln, 2 * so), gy_hi = g_ld_stream<f32x4>(gGY, 2 * vln + 16, 2 * so);
+      const bf16x8 dxv_ld = g_ld_stream<bf16x8>(p.overwrite ? gbuf(zero_tile) : gDXV, vln, p.overwrite ? 0u : xo);
+      const f32x4 gy_lo = g_ld_stream<f32x4>(gGY, 2 * vln, 4 * so), gy_hi = g_ld_stream<f32x4>(gGY, 2 * vln + 16, 4 * so);
+      const f32x4 dg_lo = g_ld_stream<f32x4>(gGY, 2 * vln, 4 * so + 2 * TILE_BYTES);
+      const f32x4 dg_hi = g_ld_stream<f32x4>(gGY, 2 * vln + 16, 4 * so + 2 * TILE_BYTES);
       bf16x8 gw[2][2], g1[2][2], dz[2][2], w1b[2][2];
 #pragma unroll
       for (int a = 0; a < 2; a++)
@@ -1386,13 +1401,36 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
       float z[8];
       ln_gather(z, s_lnrow);
       const float gyv[8] = {gy_lo[0], gy_lo[1], gy_lo[2], gy_lo[3], gy_hi[0], gy_hi[1], gy_hi[2], gy_hi[3]};
-      bf16x8 dxk_new;
+      const float dgv[8] = {dg_lo[0], dg_lo[1], dg_lo[2], dg_lo[3], dg_hi[0], dg_hi[1], dg_hi[2], dg_hi[3]};
+      bf16x8 dxk_new, dxv_new;
 #pragma unroll
-      for (int e = 0; e < 8; e++) dxk_new[e] = (bf16)((float)dxk_ld[e] + (z[e] + gyv[e]));
+      for (int e = 0; e < 8; e++) {
+        dxk_new[e] = (bf16)((float)dxk_ld[e] + (z[e] + gyv[e]));
+        dxv_new[e] = (bf16)((float)dxv_ld[e] - gyv[e]);                 // dXV accumulates -g_y
+      }
       g_st_stream<bf16x8>(gDXK, vln, xo, dxk_new);
+      g_st_stream<bf16x8>(gDXV, vln, xo, dxv_new);
+      ln_token_sum_add(s_dgw, dgv, q8, f0);
+      ln_token_sum_add(s_dbw, gyv, q8, f0);
       __syncthreads();   // the readers of the pair sums are done before the next mini-batch's take their place
     }
     publish(w_finished, done + 1);
+  }
+  // norm-weight / norm-bias gradients: the replaying workgroups' two sums (handed over before their last counts,
+  // which the walk had acquired before its own last count) + the walk's, in the order of the other launch shapes
+  __syncthreads();
+  if (tid < 2 * FD) {
+    const int which = tid / FD, f = tid % FD;
+    const float* rp = p.norm_partial + (size_t)bh * 2 * (BW_NWAVE * 2 * FD);
+    const bool have_odd = p.K > 1 || p.n_replay == 1;
+    float s = 0.f, sr0 = 0.f, sr1 = 0.f;
+#pragma unroll
+    for (int u = 0; u < BW_NWAVE; u++) {
+      s += s_red[(u * 2 + which) * FD + f];
+      sr0 += rp[(u * 2 + which) * FD + f];
+      if (have_odd) sr1 += rp[BW_NWAVE * 2 * FD + (u * 2 + which) * FD + f];
+    }
+    (which == 0 ? p.grad_L_ttt_norm_weight : p.grad_L_ttt_norm_bias)[(size_t)bh * FD + f] = (sr0 + sr1) + s;
   }
 }
 
