@@ -906,7 +906,6 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
     }
     // hand-over buffers of this group for the grad_L_XK workgroup (set = parity of the group)
     const size_t ofin = uni64(((size_t)bh * 2 + (done & 1)) * cgs);
-#define bFGW gbuf(ka->fin_gw1 + ofin * (CS * HID))
 #define bFG1 gbuf(ka->fin_g1 + ofin * (CS * HID))
 #define bFDZ gbuf(ka->fin_dz + ofin * (CS * HID))
 #define bFGY gbuf(ka->fin_gy + ofin * (2 * CS * FD))
@@ -1161,7 +1160,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
 #pragma unroll
         for (int s = 0; s < 4; s++) w2b[s] = w2_before(bIMG2, bCW2, ckW, j, s, hid0, c, h, t16);
         // T2 = gW1 rows [hid][F] (for gW1 G1^T), T1 = gW2 rows [F][hid] (transposed read gives lane = hid)
-        store_state_rows<LDF>(T2, gW1s, c, h);
+        if constexpr (!FIN) store_state_rows<LDF>(T2, gW1s, c, h);
         store_state_rows<LDH>(T1, gW2s, c, h);
         WAVE_SYNC();
         AccT<2, 2> dk;
@@ -1215,11 +1214,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           for (int rb = 0; rb < 2; rb++)
 #pragma unroll
             for (int s = 0; s < 2; s++) w1bf[rb][s] = w1_before(bIMG1, bCW1, ckW, j, rb, s, hid0, c, h, t16);
-        } else {   // gW1 as the operand of gW1 G1^T (lane = F, contraction = hid) and dZ1 leave for the other workgroup
-#pragma unroll
-          for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-            for (int t = 0; t < 2; t++) image_store<true>(bFGW, ho, 2 * rb + t, t16, piece_tr<LDF>(T2, rb, t, lane));
+        } else {   // dZ1 leaves for the other workgroup (which keeps its own copy of gW1: it sees every term added to it)
 #pragma unroll
           for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -1266,7 +1261,6 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
       }
     }
     if constexpr (ROLE == 2) publish(w_walked, done + 1);
-#undef bFGW
 #undef bFG1
 #undef bFDZ
 #undef bFGY
@@ -1357,6 +1351,15 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
   const gptr_t gDXK = gbuf(p.grad_L_XK + uni64((size_t)bh * p.NC * (CS * FD)));
   const gptr_t gDXV = gbuf(p.grad_L_XV + uni64((size_t)bh * p.NC * (CS * FD)));
   const gptr_t gCW1 = gbuf(p.W1_ck + uni64((size_t)bh * p.K * (FD * HID)));
+  const gptr_t gXQ = gbuf(p.XQ + uni64((size_t)bh * p.NC * (CS * FD))), gXK = gbuf(p.XK + uni64((size_t)bh * p.NC * (CS * FD)));
+  bf16* const s_xq = reinterpret_cast<bf16*>(smem + SB_XQ);
+  bf16* const s_xk = reinterpret_cast<bf16*>(smem + SB_XK);
+  bf16* const T1 = reinterpret_cast<bf16*>(s_own);   // wave-private tiles in this wave's pair-sum region, as in the walk
+  bf16* const T2 = T1 + 64 * LDH;
+  // This workgroup keeps its own copy of the running gradient wrt W1: both terms the walk adds to it per
+  // mini-batch (XQ^T gZ1_bar and XK^T dZ1) are formed from data that reaches this workgroup anyway, in the walk's order.
+  AccT<2, 1> gW1s;
+  acc_load_rows(gW1s, gbuf(p.grad_L_W1_last + (size_t)bh * FD * HID), 0, HID, 0, hid0, c, h);
   // the walk's share of the norm-weight / norm-bias gradients: per wave, summed in the walk's order
   float* s_red = reinterpret_cast<float*>(smem + SB_RED);
   float* s_dgw = s_red + (v * 2 + 0) * FD;
@@ -1367,7 +1370,8 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
     const int done = p.K - 1 - k, set = done % n_sets;
     if (!wait_at_least(w_walked, done + 1, p.status, s_flag, p.wait_limit)) return;
     const size_t ofin = uni64(((size_t)bh * 2 + (done & 1)) * cgs);
-    const gptr_t gGW = gbuf(p.fin_gw1 + ofin * (CS * HID)), gG1 = gbuf(p.fin_g1 + ofin * (CS * HID));
+    const gptr_t gG1 = gbuf(p.fin_g1 + ofin * (CS * HID));
+    const gptr_t gGZ1B = gbuf((set ? p.alt_Z1_bar_group[set - 1] : p.Z1_bar_group) + uni64((size_t)bh * cgs * (CS * HID)));
     const gptr_t gDZ = gbuf(p.fin_dz + ofin * (CS * HID)), gGY = gbuf(p.fin_gy + ofin * (2 * CS * FD));
     const gptr_t gIMG1 = gbuf((set ? p.alt_X2_group[set - 1] : p.X2_group) + uni64((size_t)bh * cgs * (CS * HID)));
     const unsigned ckW = k * (FD * HID * 4);
@@ -1378,16 +1382,30 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
       const f32x4 gy_lo = g_ld_stream<f32x4>(gGY, 2 * vln, 4 * so), gy_hi = g_ld_stream<f32x4>(gGY, 2 * vln + 16, 4 * so);
       const f32x4 dg_lo = g_ld_stream<f32x4>(gGY, 2 * vln, 4 * so + 2 * TILE_BYTES);
       const f32x4 dg_hi = g_ld_stream<f32x4>(gGY, 2 * vln + 16, 4 * so + 2 * TILE_BYTES);
-      bf16x8 gw[2][2], g1[2][2], dz[2][2], w1b[2][2];
+      const u32x4 xq = g_ld16(gXQ, t16, xo), xk = g_ld16(gXK, t16, xo);
+      bf16x8 g1b[4];   // gZ1_bar^T of the output branch: lane = hid, contraction = tok
+#pragma unroll
+      for (int s = 0; s < 4; s++) g1b[s] = image_load<true>(gGZ1B, ho, s, t16);
+      bf16x8 g1[2][2], dz[2][2], w1b[2][2];
 #pragma unroll
       for (int a = 0; a < 2; a++)
 #pragma unroll
         for (int t = 0; t < 2; t++) {
-          gw[a][t] = image_load<true>(gGW, ho, 2 * a + t, t16);
           g1[a][t] = image_load<true>(gG1, ho, 2 * tb[a] + t, t16);
           dz[a][t] = image_load<true>(gDZ, ho, 2 * tb[a] + t, t16);
           w1b[a][t] = w1_before(gIMG1, gCW1, ckW, j, a, t, hid0, c, h, t16);
         }
+      lds_put16(s_xq, tid, xq);
+      lds_put16(s_xk, tid, xk);
+      __syncthreads();
+      mma_jit<4>(gW1s, [&](int fb, int s) { return piece_tr<LDX>(s_xq, fb, s, lane); },      // + XQ^T gZ1_bar
+                 [&](int, int s) { return g1b[s]; });
+      store_state_rows<LDF>(T2, gW1s, c, h);                                                  // gW1 rows [hid][F]
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int t = 0; t < 2; t++) store_piece_rows<LDH>(T1, tb[i], t, c, h, dz[i][t]);     // dZ1 rows [tok][hid]
+      WAVE_SYNC();
       AccT<2, 2> dk;
       acc_zero(dk);
 #pragma unroll
@@ -1395,8 +1413,11 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
 #pragma unroll
         for (int t = 0; t < 2; t++)
 #pragma unroll
-          for (int rb = 0; rb < 2; rb++) dk.b[rb][i] = MFMA(gw[rb][t], g1[i][t], dk.b[rb][i]);
+          for (int rb = 0; rb < 2; rb++) dk.b[rb][i] = MFMA(piece_tr<LDF>(T2, rb, t, lane), g1[i][t], dk.b[rb][i]);
       mma_jit<2>(dk, [&](int rb, int s) { return w1b[rb][s]; }, [&](int i, int s) { return dz[i][s]; });
+      mma_jit<4>(gW1s, [&](int fb, int s) { return piece_tr<LDX>(s_xk, fb, s, lane); },      // + XK^T dZ1
+                 [&](int, int s) { return piece_tr<LDH>(T1, 0, s, lane); });
+      WAVE_SYNC();   // this wave's readers of T1 / T2 are done
       pair_sum(s_own, s_partner, dk, c, h);
       float z[8];
       ln_gather(z, s_lnrow);

@@ -60,10 +60,11 @@ struct BwdParams {
   float* norm_park;      // [B*NH][8 waves][2][64]: n_replay = 1: the share of the parity that is not being added to
   __bf16* walk_park;     // [B*NH][64][256]: one register image the walking workgroup parks across its LayerNorm stage
   int n_replay;
-  // n_finish = 1: a further workgroup forms grad_L_XK from what the walk hands it per mini-batch - three
-  // register images (gW1 as operand, G1, dZ1: [B*NH][2 sets][cgs][64][256] bf16 each) and g_y
-  // ([B*NH][2][cgs][64][64] fp32); the two sets alternate by group.
-  __bf16 *fin_gw1, *fin_g1, *fin_dz;
+  // n_finish = 1: a further workgroup forms grad_L_XK, grad_L_XV and the walk's share of the norm gradients from
+  // what the walk hands it per mini-batch - two register images (G1, dZ1: [B*NH][2 sets][cgs][64][256] bf16
+  // each) and two fp32 tiles (g_y and the norm-weight gradient terms: [B*NH][2][cgs][2][64][64]); the two sets
+  // alternate by group.  It keeps its own copy of the running gradient wrt W1.
+  __bf16 *fin_g1, *fin_dz;
   float* fin_gy;
   int n_finish;
   int* sync;
