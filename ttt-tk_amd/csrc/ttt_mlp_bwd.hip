@@ -906,7 +906,6 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
     }
     // hand-over buffers of this group for the grad_L_XK workgroup (set = parity of the group)
     const size_t ofin = uni64(((size_t)bh * 2 + (done & 1)) * cgs);
-#define bFG1 gbuf(ka->fin_g1 + ofin * (CS * HID))
 #define bFDZ gbuf(ka->fin_dz + ofin * (CS * HID))
 #define bFGY gbuf(ka->fin_gy + ofin * (2 * CS * FD))
     if constexpr (ROLE != 1)
@@ -1041,8 +1040,8 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
             // gelu'(Z1)) go to their parks at once (L2-resident, rewritten every mini-batch)
             if constexpr (!IMG) chunk_store(bPW1, PARK_D1, 2 * tb[i] + t, t16, ac[t]);
             chunk_store(bPW2, PARK_T2, 2 * tb[i] + t, t16, t2c);
-            if constexpr (FIN) image_store<true>(bFG1, ho, 2 * tb[i] + t, t16, g1c);   // only grad_L_XK needs G1
-            else chunk_store(bPW2, PARK_G1, 2 * tb[i] + t, t16, g1c);
+            // only grad_L_XK needs G1: its workgroup, where there is one, forms G1 itself
+            if constexpr (!FIN) chunk_store(bPW2, PARK_G1, 2 * tb[i] + t, t16, g1c);
             store_piece_rows<LDH>(T0, tb[i], t, c, h, x2c[t]);             // X2 rows [tok][hid]
           }
           // pz[:, i] = gW2^T X2^T ; dEta partial ; + W2^T u^T
@@ -1261,7 +1260,6 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
       }
     }
     if constexpr (ROLE == 2) publish(w_walked, done + 1);
-#undef bFG1
 #undef bFDZ
 #undef bFGY
   }
@@ -1354,6 +1352,9 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
   const gptr_t gXQ = gbuf(p.XQ + uni64((size_t)bh * p.NC * (CS * FD))), gXK = gbuf(p.XK + uni64((size_t)bh * p.NC * (CS * FD)));
   bf16* const s_xq = reinterpret_cast<bf16*>(smem + SB_XQ);
   bf16* const s_xk = reinterpret_cast<bf16*>(smem + SB_XK);
+  bf16* const s_gz2 = reinterpret_cast<bf16*>(smem + SB_GZ2);
+  const gptr_t gETA = gbuf(p.last_eta + uni64((size_t)bh * p.NC * CS));
+  const gptr_t gCW2 = gbuf(p.W2_ck + uni64((size_t)bh * p.K * (FD * HID)));
   bf16* const T1 = reinterpret_cast<bf16*>(s_own);   // wave-private tiles in this wave's pair-sum region, as in the walk
   bf16* const T2 = T1 + 64 * LDH;
   // This workgroup keeps its own copy of the running gradient wrt W1: both terms the walk adds to it per
@@ -1370,7 +1371,10 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
     const int done = p.K - 1 - k, set = done % n_sets;
     if (!wait_at_least(w_walked, done + 1, p.status, s_flag, p.wait_limit)) return;
     const size_t ofin = uni64(((size_t)bh * 2 + (done & 1)) * cgs);
-    const gptr_t gG1 = gbuf(p.fin_g1 + ofin * (CS * HID));
+    const size_t o_img = uni64((size_t)bh * cgs * (CS * HID)), o_tile = uni64((size_t)bh * cgs * (CS * FD));
+    const gptr_t gIMG2 = gbuf((set ? p.alt_grad_l_wrt_Z1_group[set - 1] : p.grad_l_wrt_Z1_group) + o_img);   // W2 after each step
+    const gptr_t gGZ2 = gbuf((set ? p.alt_grad_l_wrt_Z2_group[set - 1] : p.grad_l_wrt_Z2_group) + o_tile);   // dl/dZ2
+    const gptr_t gDD = gbuf((set ? p.alt_W1_init_group[set - 1] : p.W1_init_group) + uni64((size_t)bh * cgs * (FD * HID)));   // gelu'(Z1) images
     const gptr_t gGZ1B = gbuf((set ? p.alt_Z1_bar_group[set - 1] : p.Z1_bar_group) + uni64((size_t)bh * cgs * (CS * HID)));
     const gptr_t gDZ = gbuf(p.fin_dz + ofin * (CS * HID)), gGY = gbuf(p.fin_gy + ofin * (2 * CS * FD));
     const gptr_t gIMG1 = gbuf((set ? p.alt_X2_group[set - 1] : p.X2_group) + uni64((size_t)bh * cgs * (CS * HID)));
@@ -1383,37 +1387,62 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
       const f32x4 dg_lo = g_ld_stream<f32x4>(gGY, 2 * vln, 4 * so + 2 * TILE_BYTES);
       const f32x4 dg_hi = g_ld_stream<f32x4>(gGY, 2 * vln + 16, 4 * so + 2 * TILE_BYTES);
       const u32x4 xq = g_ld16(gXQ, t16, xo), xk = g_ld16(gXK, t16, xo);
+      const u32x4 gz = g_ld_stream<u32x4>(gGZ2, t16, so);
+      const float eta_i[2] = {bf2f(g_ldh(gETA, 2 * c, (k * cgs + j) * (CS * 2) + 64 * tb[0])),
+                              bf2f(g_ldh(gETA, 2 * c, (k * cgs + j) * (CS * 2) + 64 * tb[1]))};
       bf16x8 g1b[4];   // gZ1_bar^T of the output branch: lane = hid, contraction = tok
+      bf16x8 w2bf[4];  // W2 before the step: lane = hid, contraction = F
 #pragma unroll
-      for (int s = 0; s < 4; s++) g1b[s] = image_load<true>(gGZ1B, ho, s, t16);
-      bf16x8 g1[2][2], dz[2][2], w1b[2][2];
+      for (int s = 0; s < 4; s++) {
+        g1b[s] = image_load<true>(gGZ1B, ho, s, t16);
+        w2bf[s] = w2_before(gIMG2, gCW2, ckW, j, s, hid0, c, h, t16);
+      }
+      bf16x8 g1[2][2], dz[2][2], w1b[2][2], d1[2][2];
 #pragma unroll
       for (int a = 0; a < 2; a++)
 #pragma unroll
         for (int t = 0; t < 2; t++) {
-          g1[a][t] = image_load<true>(gG1, ho, 2 * tb[a] + t, t16);
+          d1[a][t] = chunk_load(gDD, j * (2 * IMG_BYTES), 2 * tb[a] + t, t16);   // gelu'(Z1)
           dz[a][t] = image_load<true>(gDZ, ho, 2 * tb[a] + t, t16);
           w1b[a][t] = w1_before(gIMG1, gCW1, ckW, j, a, t, hid0, c, h, t16);
         }
       lds_put16(s_xq, tid, xq);
       lds_put16(s_xk, tid, xk);
+      lds_put16(s_gz2, tid, gz);
       __syncthreads();
       mma_jit<4>(gW1s, [&](int fb, int s) { return piece_tr<LDX>(s_xq, fb, s, lane); },      // + XQ^T gZ1_bar
                  [&](int, int s) { return g1b[s]; });
       store_state_rows<LDF>(T2, gW1s, c, h);                                                  // gW1 rows [hid][F]
 #pragma unroll
-      for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int t = 0; t < 2; t++) store_piece_rows<LDH>(T1, tb[i], t, c, h, dz[i][t]);     // dZ1 rows [tok][hid]
+      for (int s = 0; s < 4; s++) store_piece_rows<LDF>(T1, 0, s, c, h, w2bf[s]);            // W2 before the step, rows [hid][F]
       WAVE_SYNC();
       AccT<2, 2> dk;
       acc_zero(dk);
 #pragma unroll
-      for (int i = 0; i < 2; i++)
+      for (int i = 0; i < 2; i++) {
+        // G1 = -eta * dl/dZ1 with dl/dZ1 = (gZ2 W2^T) * gelu'(Z1), as the walk forms it
+        AccT<1, 1> R;
+        acc_zero(R);
+        mma_jit<4>(R, [&](int, int s) { return piece_rows<LDF>(T1, 0, s, c, h); },
+                   [&](int, int s) { return piece_rows<LDX>(s_gz2, tb[i], s, c, h); });
 #pragma unroll
-        for (int t = 0; t < 2; t++)
+        for (int t = 0; t < 2; t++) {
+#pragma unroll
+          for (int jj = 0; jj < 8; jj++) {
+            const float a = (float)d1[i][t][jj];
+            const float gz1 = R.b[0][0][8 * t + jj] * a;
+            g1[i][t][jj] = (bf16)(-eta_i[i] * gz1);
+          }
 #pragma unroll
           for (int rb = 0; rb < 2; rb++) dk.b[rb][i] = MFMA(piece_tr<LDF>(T2, rb, t, lane), g1[i][t], dk.b[rb][i]);
+        }
+      }
+      WAVE_SYNC();   // the readers of T1 (W2 rows) are done
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int t = 0; t < 2; t++) store_piece_rows<LDH>(T1, tb[i], t, c, h, dz[i][t]);     // dZ1 rows [tok][hid]
+      WAVE_SYNC();
       mma_jit<2>(dk, [&](int rb, int s) { return w1b[rb][s]; }, [&](int i, int s) { return dz[i][s]; });
       mma_jit<4>(gW1s, [&](int fb, int s) { return piece_tr<LDX>(s_xk, fb, s, lane); },      // + XK^T dZ1
                  [&](int, int s) { return piece_tr<LDH>(T1, 0, s, lane); });

@@ -172,9 +172,10 @@ struct BwdWorkspace {
     put(1, 2 * norm);
     put(2, norm);
     put(3, (size_t)n * img);
-    // hand-over to the grad_L_XK workgroup: two images and two fp32 tiles (g_y, norm-weight gradient terms) per slot, two sets
+    // hand-over to the grad_L_XK workgroup: one image (dZ1) and two fp32 tiles (g_y, norm-weight gradient terms) per slot, two sets
     put(4, 0);
-    for (int t = 1; t < 3; t++) put(4 + t, finish ? 2 * slot * img : 0);
+    put(5, 0);
+    put(6, finish ? 2 * slot * img : 0);
     put(7, finish ? 2 * slot * 4 * tile : 0);
     for (int s = 0; s < 3; s++)
       for (int t = 0; t < PER_SET; t++) put(8 + PER_SET * s + t, s < alt_sets ? per_set[t] : 0);
@@ -261,7 +262,6 @@ extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* wo
   p.n_finish = finish ? 1 : 0;
   p.wait_limit = g_wait_limit;
   if (finish) {
-    p.fin_g1 = reinterpret_cast<__bf16*>(base + w.off[5]) - b0 * 2 * img;
     p.fin_dz = reinterpret_cast<__bf16*>(base + w.off[6]) - b0 * 2 * img;
     p.fin_gy = reinterpret_cast<float*>(base + w.off[7]) - b0 * 2 * 2 * tile;
   }

@@ -61,10 +61,10 @@ struct BwdParams {
   __bf16* walk_park;     // [B*NH][64][256]: one register image the walking workgroup parks across its LayerNorm stage
   int n_replay;
   // n_finish = 1: a further workgroup forms grad_L_XK, grad_L_XV and the walk's share of the norm gradients from
-  // what the walk hands it per mini-batch - two register images (G1, dZ1: [B*NH][2 sets][cgs][64][256] bf16
-  // each) and two fp32 tiles (g_y and the norm-weight gradient terms: [B*NH][2][cgs][2][64][64]); the two sets
-  // alternate by group.  It keeps its own copy of the running gradient wrt W1.
-  __bf16 *fin_g1, *fin_dz;
+  // what the walk hands it per mini-batch - one register image (dZ1: [B*NH][2 sets][cgs][64][256] bf16) and two
+  // fp32 tiles (g_y and the norm-weight gradient terms: [B*NH][2][cgs][2][64][64]); the two sets alternate by
+  // group.  It keeps its own copy of the running gradient wrt W1 and forms G1 = -eta * dl/dZ1 itself.
+  __bf16* fin_dz;
   float* fin_gy;
   int n_finish;
   int* sync;
