@@ -33,7 +33,7 @@ WORKLOADS = {
     "c5": (8, 48, 512, 32, 2.0, "fwd+bwd B=8 NH=48 32,768 tokens/sequence cgs=32 (fill-the-chip)"),
 }
 # HBM bytes per backward launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/), or None.
-MEASURED_TRAFFIC_BYTES = {"c4": 1.97e11}    # FETCH_SIZE 47,472,500 KiB x 2.0 + WRITE_SIZE 99,813,800 KiB x 1.0
+MEASURED_TRAFFIC_BYTES = {"c4": 2.15e11}    # FETCH_SIZE 56,436,600 KiB x 2.0 + WRITE_SIZE 97,333,000 KiB x 1.0
 
 
 def make_device_inputs(B, NH, NC, eta_std, dev):
