@@ -50,7 +50,9 @@ constexpr int BW_NS = HID / BW_NWAVE;     // hidden columns per wave: 32
 constexpr int LDX = 68;                   // row stride (elements) of the shared [64][64] bf16 tiles
 constexpr int LDH = 36;                   // row stride of wave-private [64][32 hid] bf16 tiles
 constexpr int LDF = 68;                   // row stride of wave-private [32 hid][64 F] bf16 tiles
-constexpr int LDR = 72;                   // row stride (floats) of a pair-sum region [32 tok][64 F]
+constexpr int LDR = 68;                   // row stride (floats) of a pair-sum region [32 tok][64 F]: 16-byte accesses of
+                                          // 16 consecutive rows fall on 64 distinct banks
+constexpr int RGN = 2304;                 // floats per pair-sum region
 
 constexpr int SB_TILE = 64 * LDX * 2;     // 8704
 constexpr int SB_XQ = 0;                  // reverse: XQ until the post-update stage is done, then (with SB_E2)
@@ -60,7 +62,8 @@ constexpr int SB_GZ2 = SB_XK + SB_TILE;   // replay: G2 = -eta*dl/dZ2 ; reverse:
 constexpr int SB_A = SB_GZ2 + SB_TILE;    // reverse: gZ2_bar, later dZ2
 static_assert(2 * SB_TILE >= CS * FD * 4, "g_y park does not fit");
 constexpr int SB_P = SB_A + SB_TILE;      // 8 pair-sum regions (one per wave), fp32 [32][LDR]
-constexpr int SB_REGION = 32 * LDR * 4;   // 9216: also two wave-private bf16 tiles
+constexpr int SB_REGION = RGN * 4;        // 9216: also two wave-private bf16 tiles
+static_assert(32 * LDR <= RGN, "pair-sum rows do not fit their region");
 constexpr int SB_WTILE = 64 * LDH * 2;    // 4608
 static_assert(2 * SB_WTILE <= SB_REGION && 32 * LDF * 2 <= SB_WTILE, "private tiles do not fit a region");
 constexpr int SB_BNC = SB_P + BW_NWAVE * SB_REGION;   // 8 wave-private bounce tiles [64][LDH]
@@ -181,8 +184,8 @@ TTT_DEV void ln_gather(float (&z)[8], const float* row) {
   f32x4 a = *reinterpret_cast<const f32x4*>(row), b = *reinterpret_cast<const f32x4*>(row + 4);
 #pragma unroll
   for (int pp = 1; pp < 4; pp++) {
-    a += *reinterpret_cast<const f32x4*>(row + pp * 2 * (32 * LDR));
-    b += *reinterpret_cast<const f32x4*>(row + pp * 2 * (32 * LDR) + 4);
+    a += *reinterpret_cast<const f32x4*>(row + pp * 2 * RGN);
+    b += *reinterpret_cast<const f32x4*>(row + pp * 2 * RGN + 4);
   }
 #pragma unroll
   for (int e = 0; e < 4; e++) { z[e] = a[e]; z[4 + e] = b[e]; }
@@ -435,10 +438,10 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
   const int q8 = lane >> 3, tok = 8 * v + q8, f0 = 8 * (lane & 7);   // LayerNorm ownership (token block r)
   const int head = bh % p.NH;
   const int hid0 = BW_NS * v;
-  float* s_own = s_P + (pp * 2 + r) * (32 * LDR);
-  float* s_partner = s_P + (pp * 2 + (1 - r)) * (32 * LDR);
+  float* s_own = s_P + (pp * 2 + r) * RGN;
+  float* s_partner = s_P + (pp * 2 + (1 - r)) * RGN;
   // the pair sums of token block r sit in region 1-r of every pair
-  const float* s_lnrow = s_P + (1 - r) * (32 * LDR) + (tok & 31) * LDR + f0;
+  const float* s_lnrow = s_P + (1 - r) * RGN + (tok & 31) * LDR + f0;
   bf16* const T0 = reinterpret_cast<bf16*>(smem + SB_BNC) + v * (64 * LDH);   // wave-private tiles: T0 = the bounce
   bf16* const T1 = reinterpret_cast<bf16*>(s_own);                            // tile; T1, T2 = the two halves of
   bf16* const T2 = T1 + 64 * LDH;                                             // this wave's pair-sum region
@@ -531,7 +534,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
   const int lane = lane_v, h = lane >> 5, c = lane & 31, tid = (v << 6) | lane;                         \
   const int q8 = lane >> 3, tok = 8 * v + q8, f0 = 8 * (lane & 7);                                      \
   const unsigned t16 = 16 * tid, vln = (tok * FD + f0) * 2, vtok = 4 * tok;                             \
-  const float* s_lnrow = s_P + (1 - r) * (32 * LDR) + (tok & 31) * LDR + f0;                            \
+  const float* s_lnrow = s_P + (1 - r) * RGN + (tok & 31) * LDR + f0;                            \
   float* s_gy = reinterpret_cast<float*>(smem + SB_XQ) + tok * FD + f0;                                 \
   (void)h; (void)c; (void)tid; (void)q8; (void)t16; (void)vln; (void)vtok; (void)s_lnrow; (void)s_gy
 
@@ -1337,9 +1340,9 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
   const int tb[2] = {r, 1 - r};
   const int q8 = lane >> 3, tok = 8 * v + q8, f0 = 8 * (lane & 7);
   const int hid0 = BW_NS * v;
-  float* s_own = s_P + (pp * 2 + r) * (32 * LDR);
-  float* s_partner = s_P + (pp * 2 + (1 - r)) * (32 * LDR);
-  const float* s_lnrow = s_P + (1 - r) * (32 * LDR) + (tok & 31) * LDR + f0;
+  float* s_own = s_P + (pp * 2 + r) * RGN;
+  float* s_partner = s_P + (pp * 2 + (1 - r)) * RGN;
+  const float* s_lnrow = s_P + (1 - r) * RGN + (tok & 31) * LDR + f0;
   const int cgs = p.cgs, n_sets = 2 * p.n_replay;
   const unsigned t16 = 16 * tid, vln = (tok * FD + f0) * 2;
   int* const w_sync = p.sync + (size_t)bh * BWD_SYNC_STRIDE;
