@@ -519,7 +519,8 @@ TTT_DEV void fwd_output_branch(const FwdParams& p, unsigned char* smem, const in
   // eta of a mini-batch one LayerNorm stage before it needs them, which does not cover the latency of HBM; this
   // workgroup has time to spare, so it reads those tiles ahead of the recurrence - which is about a hand-over
   // group ahead of this workgroup - and the recurrence finds them in the L2.  The values are not used.
-  constexpr int AHEAD = RING + 4;   // measured: RING + 1 .. RING + 4 alike, RING + 10 and more slower (the tiles leave the L2 again)
+  constexpr int AHEAD = RING + 4;   // measured: RING + 1 .. RING + 4 alike; RING + 10 and more slower (the tiles leave the L2
+                                    // again), RING - 4 slower and RING - 12 no gain at all (the recurrence is that far ahead)
   static_assert(AHEAD > 0, "the tiles read ahead must lie ahead: a negative mini-batch index would address memory before the tensor");
   u32x4 warm_k = {0, 0, 0, 0}, warm_v = {0, 0, 0, 0};
   unsigned warm = 0;
