@@ -139,6 +139,7 @@ def main():
         step(events[i])
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    ext.check_last_status()               # raises if workgroups of an unsynchronised launch gave up waiting for each other
     host.set_synchronize(True)
     if a.calibrate_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)     # 1 GiB read + 1 GiB written

@@ -40,7 +40,7 @@ extern "C" {
 #define TTT_MLP_ERR_BAD_ARG 1001   /* null pointer or non-positive size           */
 #define TTT_MLP_ERR_BAD_CKPT 1002  /* K != ceil(NC / checkpoint_group_size)       */
 #define TTT_MLP_ERR_ALIGN 1003     /* a pointer is not 16-byte aligned            */
-#define TTT_MLP_ERR_TOO_LARGE 1004 /* B*NH > 2^31-1, NC > 2^18 or cgs > 2^16         */
+#define TTT_MLP_ERR_TOO_LARGE 1004 /* B*NH > 2^31-1, NC > 2^18, cgs > 2^16 or K > 2^15 */
 #define TTT_MLP_ERR_NO_ROOM 1005   /* 2*B*NH workgroups exceed the CUs of the device */
 #define TTT_MLP_ERR_WORKSPACE 1006 /* workspace smaller than required              */
 
@@ -171,6 +171,15 @@ size_t ttt_mlp_fwd_workspace_bytes(int32_t B, int32_t NH);
 size_t ttt_mlp_fwd_status_offset(int32_t B, int32_t NH);
 int ttt_mlp_fwd_launch_overlapped(const ttt_mlp_fwd_args* args, void* workspace, size_t workspace_bytes, void* stream);
 int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* args, void* workspace, size_t workspace_bytes, void* stream);
+
+/* For callers that do not wait for the stream after an overlapped launch (and may free or reuse the
+ * workspace before they do): enqueues, behind the launch on the same stream, `if (*status_word != 0)
+ * *sticky_word = 1`.  `status_word` = workspace + ttt_mlp_*_status_offset(); `sticky_word` = a device int
+ * owned by the caller that outlives the workspace (zero it once).  After any later synchronisation a
+ * non-zero sticky word says that some launch since it was last zeroed gave up a wait: the reference's
+ * launchers report execution errors right after their own device synchronisation
+ * (kernels/ttt/ttt.cu:708-718); this is the same report for callers that synchronise later. */
+int ttt_mlp_status_accumulate(const void* status_word, int* sticky_word, void* stream);
 
 /* Optional: fills the sixteen *_group tensors with the values of checkpoint group 0 (the group the
  * backward processes last) in the layouts of the struct above, as the reference's kernel leaves them

@@ -35,7 +35,8 @@ def test_header_declares_the_expected_entry_points():
     assert declared_functions() == ["ttt_mlp_abi_version", "ttt_mlp_bwd_export_group0", "ttt_mlp_bwd_launch", "ttt_mlp_bwd_launch_overlapped",
                                     "ttt_mlp_bwd_status_offset", "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_error_string",
                                     "ttt_mlp_fwd_launch", "ttt_mlp_fwd_launch_overlapped", "ttt_mlp_fwd_status_offset",
-                                    "ttt_mlp_fwd_workspace_bytes", "ttt_mlp_kernel_info", "ttt_mlp_launch_plan", "ttt_mlp_set_wait_limit"]
+                                    "ttt_mlp_fwd_workspace_bytes", "ttt_mlp_kernel_info", "ttt_mlp_launch_plan", "ttt_mlp_set_wait_limit",
+                                    "ttt_mlp_status_accumulate"]
 
 
 def test_library_exports_every_declared_symbol(lib):
@@ -79,6 +80,12 @@ def test_forward_launch_rejects_bad_arguments_before_touching_the_gpu(lib):
     assert lib.ttt_mlp_fwd_launch(ctypes.byref(a), None) == 1004
     a.NC, a.checkpoint_group_size, a.K = 1 << 17, (1 << 16) + 1, 2
     assert lib.ttt_mlp_fwd_launch(ctypes.byref(a), None) == 1004
+    # more checkpoints than 32-bit byte offsets of 64 KiB slots reach: NC = 2^17 with a checkpoint before every mini-batch
+    a.NC, a.checkpoint_group_size, a.K = 1 << 17, 1, 1 << 17
+    assert lib.ttt_mlp_fwd_launch(ctypes.byref(a), None) == 1004
+    a.NC, a.checkpoint_group_size, a.K = (1 << 15) + 1, 1, (1 << 15) + 1
+    assert lib.ttt_mlp_fwd_launch(ctypes.byref(a), None) == 1004
+    assert b"32768 checkpoints" in lib.ttt_mlp_error_string(1004)
     assert lib.ttt_mlp_bwd_launch(None, None) == 1001
 
 

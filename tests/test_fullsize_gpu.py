@@ -2,17 +2,18 @@
 
 C2/C3 (16,384 tokens, 48 heads) are checked against the CPU oracle for every head.  C4 (262,144 tokens)
 and C5 (8 x 48 recurrences) run in full on the GPU; the oracle, which needs minutes for them, checks a
-subset of the independent (batch, head) recurrences, and size-independent properties cover the rest:
-exact linearity in the upstream gradients, zero gradients for zero upstream gradients, independence of
-heads, and agreement between two checkpoint group sizes.
+subset of the independent (batch, head) recurrences (4 heads of C4, 6 pairs of C5), and size-independent
+properties cover the rest: exact linearity in the upstream gradients, zero gradients for zero upstream
+gradients, independence of heads, and agreement between two checkpoint group sizes.
 
-Bar: max|hw - ref| / max|ref| <= 2e-2 and cosine >= 0.9999 per tensor (Out, checkpoints, ten gradients),
-reference = fp32 oracle.  bf16 matrix-product operands with fp32 accumulation cannot hold that bar over
-thousands of recurrent steps whatever the implementation: the oracle itself, run in fp32 with nothing but
-its matrix-product operands rounded to bf16, already leaves it (cosine 0.99985 at 1,024 mini-batches,
-0.9998 at 2,048).  Where the strict bar is missed, a tensor therefore passes if the kernel is no further
-from the fp32 oracle than twice that ideal bf16-operand arithmetic is (1 - cosine and max-rel both), and
-within an absolute floor of cosine >= 0.9995, max-rel <= 6e-2."""
+Bar, on every configuration: max|hw - ref| / max|ref| <= 2e-2 and cosine >= 0.9999 per tensor (Out,
+checkpoints, ten gradients), reference = fp32 oracle on the same bf16-rounded inputs.
+
+Inputs: the benchmark's distributions, except that b1, b2 and the norm weight / bias are not the trivial
+zeros / ones / zeros here (b ~ N(0, 0.02), weight ~ 1 + N(0, 0.1), bias ~ N(0, 0.1)), so that the bias and
+norm-parameter paths carry signal over the whole sequence.
+
+If the environment variable TTT_PARITY_LOG names a file, every per-tensor line is appended to it."""
 import os
 
 import pytest
@@ -39,8 +40,8 @@ def device_inputs(B, NH, NC, eta_std, seed=0):
         for b in range(B):
             t[name][b] = rn(NH, NC, 64, 64).to(torch.bfloat16)
     t["W1"], t["W2"] = rn(B, NH, 64, 256) * 0.02, rn(B, NH, 256, 64) * 0.02
-    t["b1"], t["b2"] = torch.zeros(B, NH, 1, 256, device=dev), torch.zeros(B, NH, 1, 64, device=dev)
-    t["ttt_norm_weight"], t["ttt_norm_bias"] = torch.ones(1, NH, 1, 64, device=dev), torch.zeros(1, NH, 1, 64, device=dev)
+    t["b1"], t["b2"] = rn(B, NH, 1, 256) * 0.02, rn(B, NH, 1, 64) * 0.02
+    t["ttt_norm_weight"], t["ttt_norm_bias"] = 1 + rn(1, NH, 1, 64) * 0.1, rn(1, NH, 1, 64) * 0.1
     t["last_eta"] = (torch.sigmoid(rn(B, NH, NC, 64, 1) * eta_std) / 64).to(torch.bfloat16)
     t["grad_L_W1_last"], t["grad_L_b1_last"] = rn(B, NH, 64, 256) * 1e-3, rn(B, NH, 1, 256) * 1e-3
     t["grad_L_W2_last"], t["grad_L_b2_last"] = rn(B, NH, 256, 64) * 1e-3, rn(B, NH, 1, 64) * 1e-3
@@ -60,62 +61,61 @@ def run(t, cgs, backward=True):
     return r
 
 
-def cpu_slice(t, b, h):
-    """The (b, h) recurrence as B=1, NH=1 CPU tensors."""
+def cpu_pairs(t, pairs):
+    """The (b, h) recurrences of `pairs` as one CPU problem with B = 1 and one head per pair."""
     d = {}
     for k in FWD_KEYS + UP_KEYS:
         v = t[k]
-        d[k] = (v[:, h:h + 1] if v.shape[0] == 1 and k.startswith("ttt_norm") else v[b:b + 1, h:h + 1]).cpu()
+        if k.startswith("ttt_norm"):
+            d[k] = torch.cat([v[:, h:h + 1] for _, h in pairs], dim=1).cpu()
+        else:
+            d[k] = torch.cat([v[b:b + 1, h:h + 1] for b, h in pairs], dim=1).cpu()
     return d
 
 
-def oracle(d, cgs, backward=True, emulate=False):
-    out, ck, _ = orc.ttt_forward(*[d[k] for k in FWD_KEYS], cgs, emulate_bf16_operands=emulate)
+def oracle(d, cgs, backward=True):
+    out, ck, _ = orc.ttt_forward(*[d[k] for k in FWD_KEYS], cgs)
     ref = {"Out": out, "W1_checkpoints": ck.W1, "b1_checkpoints": ck.b1, "W2_checkpoints": ck.W2, "b2_checkpoints": ck.b2}
     if backward:
         ref.update(orc.ttt_backward(d["XQ"], d["XK"], d["XV"], d["last_eta"], d["ttt_norm_weight"], d["ttt_norm_bias"], ck,
                                     orc.State(d["grad_L_W1_last"], d["grad_L_b1_last"], d["grad_L_W2_last"],
-                                              d["grad_L_b2_last"]), d["grad_L_XQW_mini_batch"], cgs,
-                                    emulate_bf16_operands=emulate))
+                                              d["grad_L_b2_last"]), d["grad_L_XQW_mini_batch"], cgs))
     return ref
 
 
-def compare(tag, hw, ref, failures, ideal=None):
-    """ideal: the oracle with bf16-rounded matrix-product operands (None = strict bar only)."""
+def report(line):
+    print(line, flush=True)
+    path = os.environ.get("TTT_PARITY_LOG")
+    if path:
+        with open(path, "a") as f:
+            f.write(line + "\n")
+
+
+def compare(tag, hw, ref, failures, bar=True):
+    """One line per tensor; with `bar` a tensor outside max-rel 2e-2 / cosine 0.9999 is a failure."""
     for name, r in ref.items():
         if r.abs().max() == 0:
             assert hw[name].abs().max() == 0, name
             continue
         st = orc.parity_stats(hw[name], r)
-        ok = st["max_rel"] <= MAX_REL and st["cosine"] >= MIN_COS
-        note = ""
-        if not ok and ideal is not None:
-            si = orc.parity_stats(ideal[name], r)
-            ok = (1 - st["cosine"] <= 2 * (1 - si["cosine"]) + 1e-5 and st["max_rel"] <= 2 * si["max_rel"] + 5e-3
-                  and st["cosine"] >= 0.9995 and st["max_rel"] <= 6e-2)
-            note = f"  [ideal bf16-operand arithmetic: max_rel={si['max_rel']:.3e} cos={si['cosine']:.6f}]"
-        print(f"{tag} {name:24s} max_rel={st['max_rel']:.3e} cos={st['cosine']:.6f}{note}{'' if ok else '  <-- FAIL'}",
-              flush=True)
+        ok = not bar or (st["max_rel"] <= MAX_REL and st["cosine"] >= MIN_COS)
+        report(f"{tag} {name:24s} max_rel={st['max_rel']:.3e} cos={st['cosine']:.6f}{'' if ok else '  <-- FAIL'}")
         if not ok:
             failures.append((tag, name, st["max_rel"], st["cosine"]))
 
 
-def check_subset(t, r, cgs, pairs, backward=True):
+def check_subset(case, t, r, cgs, pairs, backward=True):
     torch.set_num_threads(min(16, os.cpu_count() or 1))
     failures = []
-    for b, h in pairs:
-        d = cpu_slice(t, b, h)
-        ref = oracle(d, cgs, backward)
+    ref = oracle(cpu_pairs(t, pairs), cgs, backward)
+    for i, (b, h) in enumerate(pairs):
         hw = {k: r[k][b:b + 1, h:h + 1].float().cpu() for k in ref}
-        strict = all(orc.parity_stats(hw[k], ref[k])["max_rel"] <= MAX_REL and
-                     orc.parity_stats(hw[k], ref[k])["cosine"] >= MIN_COS for k in ref if ref[k].abs().max() > 0)
-        ideal = None if strict else oracle(d, cgs, backward, emulate=True)
-        compare(f"(b={b},h={h})", hw, ref, failures, ideal)
+        compare(f"{case} (b={b},h={h})", hw, {k: v[:, i:i + 1] for k, v in ref.items()}, failures)
     assert not failures, failures
 
 
 def test_c2_forward_16k_tokens_all_heads():
-    print("case C2: forward B=1 NH=48 NC=256 cgs=16", flush=True)
+    report("case C2: forward B=1 NH=48 NC=256 cgs=16")
     t = device_inputs(1, 48, 256, 1.0)
     r = run(t, 16, backward=False)
     d = {k: t[k].cpu() for k in FWD_KEYS}
@@ -126,7 +126,7 @@ def test_c2_forward_16k_tokens_all_heads():
 
 
 def test_c3_forward_backward_16k_tokens_all_heads():
-    print("case C3: forward+backward B=1 NH=48 NC=256 cgs=16", flush=True)
+    report("case C3: forward+backward B=1 NH=48 NC=256 cgs=16")
     t = device_inputs(1, 48, 256, 1.0)
     r = run(t, 16)
     d = {k: t[k].cpu() for k in FWD_KEYS + UP_KEYS}
@@ -138,12 +138,12 @@ def test_c3_forward_backward_16k_tokens_all_heads():
 
 
 def test_c4_long_sequence_262k_tokens():
-    print("case C4: forward+backward B=1 NH=48 NC=4096 cgs=64", flush=True)
+    report("case C4: forward+backward B=1 NH=48 NC=4096 cgs=64")
     t = device_inputs(1, 48, 4096, 1.0)
     r = run(t, 64)
     for k in GRADS + ("Out",):
         assert bool(torch.isfinite(r[k].float()).all()), k
-    check_subset(t, r, 64, [(0, 0), (0, 47)])
+    check_subset("C4", t, r, 64, [(0, 0), (0, 13), (0, 30), (0, 47)])
     # exact linearity: doubling every upstream gradient doubles every output gradient bit for bit
     t2 = dict(t)
     for k in UP_KEYS:
@@ -155,17 +155,17 @@ def test_c4_long_sequence_262k_tokens():
     # another checkpoint group size walks the same recurrence from other restart points
     r3 = run(t, 128)
     failures = []
-    compare("cgs 128 vs 64", {k: r3[k].float().cpu() for k in GRADS}, {k: r[k].float().cpu() for k in GRADS}, failures)
+    compare("C4 cgs 128 vs 64", {k: r3[k].float().cpu() for k in GRADS}, {k: r[k].float().cpu() for k in GRADS}, failures)
     assert not failures, failures
 
 
 def test_c5_fill_the_chip_384_recurrences():
-    print("case C5: forward+backward B=8 NH=48 NC=512 cgs=32, wide eta", flush=True)
+    report("case C5: forward+backward B=8 NH=48 NC=512 cgs=32, wide eta")
     t = device_inputs(8, 48, 512, 2.0)
     r = run(t, 32)
     for k in GRADS + ("Out",):
         assert bool(torch.isfinite(r[k].float()).all()), k
-    check_subset(t, r, 32, [(0, 0), (3, 17), (7, 47)])
+    check_subset("C5", t, r, 32, [(0, 0), (1, 40), (3, 17), (4, 5), (6, 29), (7, 47)])
     # zero upstream gradients give zero gradients everywhere
     tz = dict(t)
     for k in UP_KEYS:

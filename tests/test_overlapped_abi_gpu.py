@@ -105,3 +105,45 @@ def test_a_wait_that_gives_up_is_reported_and_every_wave_exits():
     host.zero_accumulating_grads(t)
     host.backward(t, cgs)                 # the device is fine and the same call goes through
     assert torch.isfinite(t["grad_L_W1_init"]).all()
+
+
+def test_a_wait_that_gives_up_is_reported_to_callers_that_synchronise_later():
+    """With set_synchronize(False) the operator returns before the kernels have run, and its workspace (with the
+    status word) goes back to the allocator: the status is folded into a device word that stays, and
+    check_last_status() raises after the caller's own synchronisation - once; then the word is clear again."""
+    import ttt_mlp_host as host
+    import test_time_training as ext
+    dev = torch.device("cuda:0")
+    B, NH, NC, cgs = 1, 2, 24, 4
+    d = orc.make_inputs(B, NH, NC, seed=43)
+    t = {k: d[k].to(dev).contiguous() for k in FWD_KEYS + UP_KEYS}
+    t.update(host.alloc_forward_buffers(B, NH, NC, cgs, dev))
+    t.update(host.alloc_backward_buffers(B, NH, NC, cgs, dev))
+    try:
+        host.set_synchronize(False)
+        host.forward(t, cgs)
+        host.backward(t, cgs)
+        ext.check_last_status()            # nothing gave up: no error
+        ext.set_wait_limit(1)
+        host.forward(t, cgs)               # gives up on the device; the call itself cannot know
+        assert ext.last_forward_mode() == 1
+        torch.cuda.synchronize()
+        with pytest.raises(RuntimeError, match="gave up"):
+            ext.check_last_status()
+        ext.check_last_status()            # reported once
+        ext.set_wait_limit(2_000_000_000)
+        host.forward(t, cgs)
+        ext.set_wait_limit(1)
+        host.zero_accumulating_grads(t)
+        host.backward(t, cgs)
+        ext.set_wait_limit(2_000_000_000)
+        host.forward(t, cgs)               # a good launch afterwards does not hide the earlier failure
+        with pytest.raises(RuntimeError, match="gave up"):
+            ext.check_last_status()
+    finally:
+        ext.set_wait_limit(2_000_000_000)
+        host.set_synchronize(True)
+    host.zero_accumulating_grads(t)
+    host.forward(t, cgs)
+    host.backward(t, cgs)
+    assert torch.isfinite(t["grad_L_W1_init"]).all()

@@ -17,6 +17,9 @@ bool g_synchronize = true;  // upstream blocks the host until the kernel has fin
 bool g_fill_group_tensors = false;   // leave the values of checkpoint group 0 in the sixteen *_group tensors
 bool g_accumulate = true;            // grad_L_XQ / XK / XV / last_eta are added to (upstream behaviour) rather than overwritten
 bool g_overlap = true;      // two workgroups per (batch, head) whenever they fit the device
+unsigned long long g_wait_ticks = 2000000000ull;   // mirrors the library's limit, for the error text
+torch::Tensor* g_sticky = nullptr;   // a device int, non-zero once a launch that nobody waited for gave up a wait (never freed:
+                                     // a static tensor would be destroyed after the runtime at process exit)
 int g_last_forward_mode = -1;    // 0 = one workgroup per (batch, head), 1 = two
 int g_last_backward_mode = -1;
 
@@ -44,8 +47,25 @@ uint16_t* bfp_mut(const torch::Tensor& t) { return reinterpret_cast<uint16_t*>(t
 
 // `status` (may be null): device address of the status word of a launch with several workgroups per
 // (batch, head); it can only be looked at when the host waits for the stream anyway.
-void finish(int rc, hipStream_t stream, const char* what, const void* status = nullptr) {
+std::string gave_up_text() {
+  return "a workgroup waited " + std::to_string(g_wait_ticks / 100000000.0) + " s for its partner and gave up (were all "
+         "compute units available to this launch?); the outputs are invalid - set_overlap(False) avoids the mode";
+}
+
+// The device int that collects the status words of launches the host did not wait for.
+int* sticky_word(const torch::Device& dev) {
+  if (g_sticky == nullptr || g_sticky->device() != dev)
+    g_sticky = new torch::Tensor(torch::zeros({1}, torch::TensorOptions().dtype(torch::kInt32).device(dev)));
+  return g_sticky->data_ptr<int>();
+}
+
+void finish(int rc, hipStream_t stream, const char* what, const torch::Device& dev, const void* status = nullptr) {
   TORCH_CHECK(rc == TTT_MLP_OK, what, " launch failed: ", ttt_mlp_error_string(rc));
+  if (!g_synchronize && status != nullptr) {
+    // nobody looks at the status word before the workspace goes back to the allocator: fold it into a word that stays
+    rc = ttt_mlp_status_accumulate(status, sticky_word(dev), stream);
+    TORCH_CHECK(rc == TTT_MLP_OK, what, " launch failed: ", ttt_mlp_error_string(rc));
+  }
   if (g_synchronize) {
     hipError_t e = hipStreamSynchronize(stream);
     TORCH_CHECK(e == hipSuccess, what, " execution failed: ", hipGetErrorString(e));
@@ -53,8 +73,7 @@ void finish(int rc, hipStream_t stream, const char* what, const void* status = n
       int word = 0;
       e = hipMemcpy(&word, status, sizeof(int), hipMemcpyDeviceToHost);
       TORCH_CHECK(e == hipSuccess, what, " execution failed: ", hipGetErrorString(e));
-      TORCH_CHECK(word == 0, what, ": a workgroup waited 20 s for its partner and gave up (were all compute units "
-                  "available to this launch?); the outputs are invalid - set_overlap(False) avoids the mode");
+      TORCH_CHECK(word == 0, what, ": ", gave_up_text());
     }
   }
 }
@@ -119,10 +138,10 @@ torch::Tensor ttt_forward(const torch::Tensor XQ, const torch::Tensor XK, const 
     torch::Tensor ws = torch::empty({(int64_t)ws_bytes}, torch::TensorOptions().dtype(torch::kUInt8).device(XQ.device()));
     g_last_forward_mode = 1;
     const char* status = static_cast<const char*>(ws.data_ptr()) + ttt_mlp_fwd_status_offset((int32_t)B, (int32_t)NH);
-    finish(ttt_mlp_fwd_launch_overlapped(&a, ws.data_ptr(), ws_bytes, stream), stream, "ttt_forward", status);
+    finish(ttt_mlp_fwd_launch_overlapped(&a, ws.data_ptr(), ws_bytes, stream), stream, "ttt_forward", XQ.device(), status);
   } else {
     g_last_forward_mode = 0;
-    finish(ttt_mlp_fwd_launch(&a, stream), stream, "ttt_forward");
+    finish(ttt_mlp_fwd_launch(&a, stream), stream, "ttt_forward", XQ.device());
   }
   return Out;
 }
@@ -234,12 +253,12 @@ torch::Tensor ttt_backward(
     const char* status = static_cast<const char*>(ws.data_ptr()) + ttt_mlp_bwd_status_offset((int32_t)B, (int32_t)NH);
     int rc = ttt_mlp_bwd_launch_overlapped(&a, ws.data_ptr(), ws_bytes, stream);
     if (rc == 0 && g_fill_group_tensors) rc = ttt_mlp_bwd_export_group0(&a, stream);
-    finish(rc, stream, "ttt_backward", status);
+    finish(rc, stream, "ttt_backward", XQ.device(), status);
   } else {
     g_last_backward_mode = 0;
     int rc = ttt_mlp_bwd_launch(&a, stream);
     if (rc == 0 && g_fill_group_tensors) rc = ttt_mlp_bwd_export_group0(&a, stream);
-    finish(rc, stream, "ttt_backward");
+    finish(rc, stream, "ttt_backward", XQ.device());
   }
   return Out;
 }
@@ -265,7 +284,25 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "grad_L_XV, which the caller zero-fills.  False: it overwrites them - no zero-fill needed, and the kernels "
         "skip the read of the old values.");
   m.def("get_accumulate", []() { return g_accumulate; });
-  m.def("set_wait_limit", [](unsigned long long ticks) { ttt_mlp_set_wait_limit(ticks); },
+  m.def("check_last_status", []() {
+          if (g_sticky == nullptr) return;
+          const c10::DeviceGuard guard(g_sticky->device());
+          hipStream_t stream = c10::hip::getCurrentHIPStream(g_sticky->device().index()).stream();
+          hipError_t e = hipStreamSynchronize(stream);
+          TORCH_CHECK(e == hipSuccess, "check_last_status: ", hipGetErrorString(e));
+          int word = 0;
+          e = hipMemcpy(&word, g_sticky->data_ptr<int>(), sizeof(int), hipMemcpyDeviceToHost);
+          TORCH_CHECK(e == hipSuccess, "check_last_status: ", hipGetErrorString(e));
+          if (word != 0) {
+            (void)hipMemset(g_sticky->data_ptr<int>(), 0, sizeof(int));
+            TORCH_CHECK(false, "ttt_forward / ttt_backward: ", gave_up_text());
+          }
+        },
+        "With set_synchronize(False) the operators cannot report a multi-workgroup launch whose workgroups gave up "
+        "waiting for each other (the reference reports execution errors after its own synchronisation, "
+        "kernels/ttt/ttt.cu:708-718).  Call this after such launches: it waits for the current stream and raises if "
+        "any launch since the last call gave up (the outputs of that launch are invalid).");
+  m.def("set_wait_limit", [](unsigned long long ticks) { g_wait_ticks = ticks; ttt_mlp_set_wait_limit(ticks); },
         "Ticks of the GPU's 100 MHz clock a workgroup waits for its partner before giving up (default 2e9 = 20 s).");
   m.def("last_forward_mode", []() { return g_last_forward_mode; },
         "0: the last ttt_forward used one workgroup per (batch, head); 1: two; -1: none yet.");

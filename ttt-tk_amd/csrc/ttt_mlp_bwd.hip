@@ -153,6 +153,10 @@ TTT_DEV void ln_load(float (&x)[8], const bf16* p) {      // p 8-byte aligned
 #pragma unroll
   for (int e = 0; e < 4; e++) { x[e] = (float)a[e]; x[4 + e] = (float)b[e]; }
 }
+TTT_DEV void ln_store_h(bf16* p, bf16x8 v) {
+  *reinterpret_cast<bf16x4*>(p) = __builtin_shufflevector(v, v, 0, 1, 2, 3);
+  *reinterpret_cast<bf16x4*>(p + 4) = __builtin_shufflevector(v, v, 4, 5, 6, 7);
+}
 TTT_DEV void ln_store(bf16* p, const float (&x)[8]) {
   bf16x4 a, b;
 #pragma unroll
@@ -242,25 +246,6 @@ TTT_DEV void lds_put16(bf16* s_tile, int tid, u32x4 v) {
 }
 
 // ---------------------------------------------------------------- just-in-time operand pieces
-// One MFMA operand piece = 8 bf16 per lane = (free block blk, k-step s).  Loading pieces right
-// before the MFMA that consumes them keeps whole operands out of the register file.
-template <int LD>
-TTT_DEV bf16x8 piece_rows(const bf16* tile, int blk, int s, int c, int h) {
-  const bf16* q = tile + (32 * blk + c) * LD + 16 * s + 4 * h;
-  return cat(*reinterpret_cast<const bf16x4*>(q), *reinterpret_cast<const bf16x4*>(q + 8));
-}
-template <int LD>
-TTT_DEV bf16x8 piece_tr(const bf16* tile, int blk, int s, int lane) {
-  const int h = lane >> 5, c = lane & 31, i = lane & 15;
-  const bf16* q = tile + (16 * s + 4 * h + (i >> 2)) * LD + 32 * blk + 16 * (c >> 4) + 4 * (i & 3);
-  return cat(lds_tr4(q), lds_tr4(q + 8 * LD));
-}
-template <int LD>
-TTT_DEV void store_piece_rows(bf16* tile, int blk, int s, int c, int h, bf16x8 v) {
-  bf16* q = tile + (32 * blk + c) * LD + 16 * s + 4 * h;
-  *reinterpret_cast<bf16x4*>(q) = __builtin_shufflevector(v, v, 0, 1, 2, 3);
-  *reinterpret_cast<bf16x4*>(q + 8) = __builtin_shufflevector(v, v, 4, 5, 6, 7);
-}
 // Piece (free block fb, k-step s) of the chained operand of an accumulator tile.
 template <int RB, int CB>
 TTT_DEV bf16x8 piece_state(const AccT<RB, CB>& x, int fb, int s) { return pack8(x.b[s >> 1][fb], s & 1); }
@@ -271,22 +256,6 @@ TTT_DEV void store_state_rows(bf16* tile, const AccT<RB, CB>& x, int c, int h) {
   for (int fb = 0; fb < CB; fb++)
 #pragma unroll
     for (int s = 0; s < 2 * RB; s++) store_piece_rows<LD>(tile, fb, s, c, h, piece_state(x, fb, s));
-}
-// d += A * B over KS k-steps, pieces produced by the callables fa(row block, s) and fb(column block, s).
-template <int KS, int RB, int CB, class FA, class FB>
-TTT_DEV void mma_jit(AccT<RB, CB>& d, FA fa, FB fb) {
-#pragma unroll
-  for (int s = 0; s < KS; s++) {
-    bf16x8 a[RB], b[CB];
-#pragma unroll
-    for (int r = 0; r < RB; r++) a[r] = fa(r, s);
-#pragma unroll
-    for (int c = 0; c < CB; c++) b[c] = fb(c, s);
-#pragma unroll
-    for (int r = 0; r < RB; r++)
-#pragma unroll
-      for (int c = 0; c < CB; c++) d.b[r][c] = MFMA(a[r], b[c], d.b[r][c]);
-  }
 }
 // s_vec[row] += sum over the 64-long contraction of the 32-row operand whose pieces fa(s) yields; the
 // sum is formed on the matrix cores, lanes with c == 0 fold it into the LDS vector.
@@ -587,7 +556,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
     int* const w_replayed = w_sync + 8 * (done % n_replay);
     REFRESH_OFFSETS();
     const size_t slot = (size_t)bh * p.K + k;
-    const unsigned ckW = k * (FD * HID * 4);   // byte offset of this group's checkpoint in bCW1 / bCW2
+    const unsigned ckW = static_cast<unsigned>(k) * (FD * HID * 4u);   // byte offset of this group's checkpoint in bCW1 / bCW2
     // ================================================================= replay
     if constexpr (ROLE != 2) {
       if constexpr (ROLE == 1) {   // the set is free once the reverse walk is done with the group that used it last
@@ -626,14 +595,27 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         LANE_VARS;
         __syncthreads();   // the staged inputs (and, for j = 0, the biases) are visible
 
-        // Z1^T = W1s^T XK^T + b1  (rows hid, lane = tok); X2 rows [tok][hid] -> T0, gelu'(Z1) packed
-        bf16x8 d1p[2][2];
+        // Z1^T = W1s^T XK^T + b1  (rows hid, lane = tok); X2 rows [tok][hid] -> T0; gelu'(Z1) (fp32) and the
+        // low-order term of X2 stay in registers.  The products that carry the state to the next mini-batch
+        // take their fp32 operands in two bf16 terms (see split8).
+        float d1f[2][16];
+        bf16x8 x2lo[2][2];
         {
           LANE_VARS;
           AccT<1, 2> x2;
           acc_init_rows_lds(x2, s_b1w, h);
-          mma_jit<4>(x2, [&](int, int s) { return piece_state(W1s, 0, s); },
-                     [&](int i, int s) { return piece_rows<LDX>(s_xk, tb[i], s, c, h); });
+#pragma unroll
+          for (int s = 0; s < 4; s++) {
+            bf16x8 wh, wl, xk[2];
+            split8(W1s.b[s >> 1][0], s & 1, wh, wl);
+#pragma unroll
+            for (int i = 0; i < 2; i++) xk[i] = piece_rows<LDX>(s_xk, tb[i], s, c, h);
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+              x2.b[0][i] = MFMA(wl, xk[i], x2.b[0][i]);
+              x2.b[0][i] = MFMA(wh, xk[i], x2.b[0][i]);
+            }
+          }
 #pragma unroll
           for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -662,8 +644,10 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
               for (int jj = 0; jj < 8; jj++) {
                 float g, d;
                 gelu_fd(x2.b[0][i][8 * t + jj], g, d);
-                xv[jj] = (bf16)g;
-                d1p[i][t][jj] = (bf16)d;
+                const bf16 gh = (bf16)g;
+                xv[jj] = gh;
+                x2lo[i][t][jj] = (bf16)(g - (float)gh);
+                d1f[i][8 * t + jj] = d;
               }
               store_piece_rows<LDH>(T0, tb[i], t, c, h, xv);
             }
@@ -673,8 +657,21 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           LANE_VARS;
           AccT<2, 2> z2;
           acc_zero(z2);
-          mma_jit<2>(z2, [&](int rb, int s) { return piece_state(W2s, rb, s); },                 // lane = F, contraction = hid
-                     [&](int i, int s) { return piece_rows<LDH>(T0, tb[i], s, c, h); });         // X2: lane = tok
+#pragma unroll
+          for (int s = 0; s < 2; s++) {                      // W2s: lane = F, contraction = hid, two terms; X2: lane = tok
+            bf16x8 wh[2], wl[2], xb[2];
+#pragma unroll
+            for (int rb = 0; rb < 2; rb++) split8(W2s.b[0][rb], s, wh[rb], wl[rb]);
+#pragma unroll
+            for (int i = 0; i < 2; i++) xb[i] = piece_rows<LDH>(T0, tb[i], s, c, h);
+#pragma unroll
+            for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+              for (int i = 0; i < 2; i++) {
+                z2.b[rb][i] = MFMA(wl[rb], xb[i], z2.b[rb][i]);
+                z2.b[rb][i] = MFMA(wh[rb], xb[i], z2.b[rb][i]);
+              }
+          }
           pair_sum(s_own, s_partner, z2, c, h);
         }
         // fused LayerNorm + reconstruction-loss gradient; saves for the reverse walk
@@ -711,8 +708,13 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           for (int e = 0; e < 8; e++) gx[e] = (FD * gx[e] - s1 - z[e] * s2) * sc;   // dl/dZ2
           ln_store_g<ROLE != 0>(bGZ2, vln, j * TILE_BYTES, gx);
 #pragma unroll
-          for (int e = 0; e < 8; e++) gx[e] *= neg_eta;                             // G2
-          ln_store(s_gz2 + tok * LDX + f0, gx);
+          for (int e = 0; e < 8; e++) gx[e] *= neg_eta;                             // G2, in two terms (the second in
+          {                                                                          // the tile gZ2_bar takes later)
+            bf16x8 gh, gl;
+            split8(gx, gh, gl);
+            ln_store_h(s_gz2 + tok * LDX + f0, gh);
+            ln_store_h(s_a + tok * LDX + f0, gl);
+          }
           if ((lane & 7) == 0) g_stf(bSDF, vtok, j * (CS * 4), sd);
         }
         __syncthreads();
@@ -721,29 +723,85 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           LANE_VARS;
           AccT<1, 2> g1;
           acc_zero(g1);
-          mma_jit<4>(g1, [&](int, int s) { return piece_state(W2t, 0, s); },                     // lane = hid, contraction = F
-                     [&](int i, int s) { return piece_rows<LDX>(s_gz2, tb[i], s, c, h); });      // G2: lane = tok
+#pragma unroll
+          for (int s = 0; s < 4; s++) {                      // W2t: lane = hid, contraction = F; G2: lane = tok; two terms each
+            bf16x8 wh, wl, gh[2], gl[2];
+            split8(W2t.b[s >> 1][0], s & 1, wh, wl);
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+              gh[i] = piece_rows<LDX>(s_gz2, tb[i], s, c, h);
+              gl[i] = piece_rows<LDX>(s_a, tb[i], s, c, h);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+              g1.b[0][i] = MFMA(wh, gl[i], g1.b[0][i]);
+              g1.b[0][i] = MFMA(wl, gh[i], g1.b[0][i]);
+              g1.b[0][i] = MFMA(wh, gh[i], g1.b[0][i]);
+            }
+          }
 #pragma unroll
           for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int t = 0; t < 2; t++) {
-              bf16x8 gv;
+              bf16x8 gv, gvl;
 #pragma unroll
-              for (int jj = 0; jj < 8; jj++) gv[jj] = (bf16)(g1.b[0][i][8 * t + jj] * (float)d1p[i][t][jj]);
-              store_piece_rows<LDH>(T1, tb[i], t, c, h, gv);
+              for (int jj = 0; jj < 8; jj++) {
+                const float g = g1.b[0][i][8 * t + jj] * d1f[i][8 * t + jj];
+                const bf16 gh = (bf16)g;
+                gv[jj] = gh;
+                gvl[jj] = (bf16)(g - (float)gh);
+              }
+              store_piece_rows<LDH>(T1, tb[i], t, c, h, gv);      // G1 rows [tok][hid], two terms
+              store_piece_rows<LDH>(T2, tb[i], t, c, h, gvl);
             }
         }
         WAVE_SYNC();
         {   // weight step
           LANE_VARS;
-        mma_jit<4>(W2s, [&](int, int s) { return piece_tr<LDH>(T0, 0, s, lane); },               // X2^T: lane = hid
-                   [&](int fb, int s) { return piece_tr<LDX>(s_gz2, fb, s, lane); });            // G2: lane = F
-        mma_jit<4>(W2t, [&](int fb, int s) { return piece_tr<LDX>(s_gz2, fb, s, lane); },
-                   [&](int, int s) { return piece_tr<LDH>(T0, 0, s, lane); });
-        if (v < 2) lds_rowsum_add_jit(s_b2 + 32 * v, [&](int s) { return piece_tr<LDX>(s_gz2, v, s, lane); }, ones, c, h);
-        mma_jit<4>(W1s, [&](int fb, int s) { return piece_tr<LDX>(s_xk, fb, s, lane); },         // XK^T: lane = F
-                   [&](int, int s) { return piece_tr<LDH>(T1, 0, s, lane); });                   // G1: lane = hid
-        lds_rowsum_add_jit(s_b1w, [&](int s) { return piece_tr<LDH>(T1, 0, s, lane); }, ones, c, h);
+#pragma unroll
+          for (int s = 0; s < 4; s++) {                        // W1[:, shard] += XK^T G1
+            bf16x8 xk[2];
+#pragma unroll
+            for (int fb = 0; fb < 2; fb++) xk[fb] = piece_tr<LDX>(s_xk, fb, s, lane);            // XK^T: lane = F
+            const bf16x8 gh = piece_tr<LDH>(T1, 0, s, lane), gl = piece_tr<LDH>(T2, 0, s, lane);   // G1: lane = hid
+#pragma unroll
+            for (int fb = 0; fb < 2; fb++) {
+              W1s.b[fb][0] = MFMA(xk[fb], gl, W1s.b[fb][0]);
+              W1s.b[fb][0] = MFMA(xk[fb], gh, W1s.b[fb][0]);
+            }
+          }
+          lds_rowsum_add_jit(s_b1w, [&](int s) { return piece_tr<LDH>(T2, 0, s, lane); }, ones, c, h);
+          lds_rowsum_add_jit(s_b1w, [&](int s) { return piece_tr<LDH>(T1, 0, s, lane); }, ones, c, h);
+          // the low-order term of X2 takes G1's place in T1 (rows [tok][hid])
+#pragma unroll
+          for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int t = 0; t < 2; t++) store_piece_rows<LDH>(T1, tb[i], t, c, h, x2lo[i][t]);
+          WAVE_SYNC();
+#pragma unroll
+          for (int s = 0; s < 4; s++) {                        // W2[shard, :] += X2^T G2, and its transpose
+            const bf16x8 xh = piece_tr<LDH>(T0, 0, s, lane), xl = piece_tr<LDH>(T1, 0, s, lane);   // X2^T: lane = hid
+            bf16x8 gh[2], gl[2];
+#pragma unroll
+            for (int fb = 0; fb < 2; fb++) {
+              gh[fb] = piece_tr<LDX>(s_gz2, fb, s, lane);                                        // G2: lane = F
+              gl[fb] = piece_tr<LDX>(s_a, fb, s, lane);
+            }
+#pragma unroll
+            for (int fb = 0; fb < 2; fb++) {
+              W2s.b[0][fb] = MFMA(xl, gh[fb], W2s.b[0][fb]);
+              W2s.b[0][fb] = MFMA(xh, gl[fb], W2s.b[0][fb]);
+              W2s.b[0][fb] = MFMA(xh, gh[fb], W2s.b[0][fb]);
+              W2t.b[fb][0] = MFMA(gh[fb], xl, W2t.b[fb][0]);
+              W2t.b[fb][0] = MFMA(gl[fb], xh, W2t.b[fb][0]);
+              W2t.b[fb][0] = MFMA(gh[fb], xh, W2t.b[fb][0]);
+            }
+          }
+          if (v < 2) {
+            lds_rowsum_add_jit(s_b2 + 32 * v, [&](int s) { return piece_tr<LDX>(s_a, v, s, lane); }, ones, c, h);
+            lds_rowsum_add_jit(s_b2 + 32 * v, [&](int s) { return piece_tr<LDX>(s_gz2, v, s, lane); }, ones, c, h);
+          }
+          WAVE_SYNC();   // this wave's readers of T1 / T2 are done
         }
         // operand images of the state after this step, for the reverse walk
         {
@@ -1381,7 +1439,7 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
     const gptr_t gGZ1B = gbuf((set ? p.alt_Z1_bar_group[set - 1] : p.Z1_bar_group) + uni64((size_t)bh * cgs * (CS * HID)));
     const gptr_t gDZ = gbuf(p.fin_dz + ofin * (CS * HID)), gGY = gbuf(p.fin_gy + ofin * (2 * CS * FD));
     const gptr_t gIMG1 = gbuf((set ? p.alt_X2_group[set - 1] : p.X2_group) + uni64((size_t)bh * cgs * (CS * HID)));
-    const unsigned ckW = k * (FD * HID * 4);
+    const unsigned ckW = static_cast<unsigned>(k) * (FD * HID * 4u);
     for (int j = n_mb - 1; j >= 0; j--) {
       const unsigned xo = (k * cgs + j) * TILE_BYTES, so = j * TILE_BYTES, ho = j * IMG_BYTES;
       const bf16x8 dxk_ld = g_ld_stream<bf16x8>(p.overwrite ? gbuf(zero_tile) : gDXK, vln, p.overwrite ? 0u : xo);

@@ -19,6 +19,8 @@ int check_sizes(int B, int NH, int NC, int K, int cgs) {
   if ((long long)B * NH > 0x7fffffffLL) return TTT_MLP_ERR_TOO_LARGE;
   // the kernels address one (batch, head) with 32-bit byte offsets: 8 KiB per mini-batch, 32 KiB per group slot
   if (NC > (1 << 18) || cgs > (1 << 16)) return TTT_MLP_ERR_TOO_LARGE;
+  // ... and one checkpoint slot (64 KiB) with a 32-bit byte offset too
+  if (K > (1 << 15)) return TTT_MLP_ERR_TOO_LARGE;
   return TTT_MLP_OK;
 }
 
@@ -39,7 +41,7 @@ extern "C" const char* ttt_mlp_error_string(int code) {
     case TTT_MLP_ERR_BAD_ARG: return "ttt_mlp: null pointer or non-positive size";
     case TTT_MLP_ERR_BAD_CKPT: return "ttt_mlp: number of checkpoints K must equal ceil(NC / checkpoint_group_size)";
     case TTT_MLP_ERR_ALIGN: return "ttt_mlp: every tensor pointer must be 16-byte aligned";
-    case TTT_MLP_ERR_TOO_LARGE: return "ttt_mlp: B*NH exceeds the launch grid limit, or NC > 262144, or checkpoint_group_size > 65536";
+    case TTT_MLP_ERR_TOO_LARGE: return "ttt_mlp: B*NH exceeds the launch grid limit, or NC > 262144, or checkpoint_group_size > 65536, or more than 32768 checkpoints";
     case TTT_MLP_ERR_NO_ROOM: return "ttt_mlp: two workgroups per (batch, head) do not fit the compute units of this device; use ttt_mlp_bwd_launch";
     case TTT_MLP_ERR_WORKSPACE: return "ttt_mlp: workspace smaller than ttt_mlp_bwd_workspace_bytes()";
     default: return hipGetErrorString(static_cast<hipError_t>(code));
@@ -84,9 +86,9 @@ int make_bwd_params(const ttt_mlp_bwd_args* a, ttt::BwdParams& p) {
   if (int rc = check_sizes(a->B, a->NH, a->NC, a->K, a->checkpoint_group_size)) return rc;
   if (!all_aligned(a->XQ, a->XK, a->XV, a->last_eta, a->ttt_norm_weight, a->ttt_norm_bias, a->W1_checkpoints,
                    a->b1_checkpoints, a->W2_checkpoints, a->b2_checkpoints, a->W1_init_group, a->b1_init_group,
-                   a->W2_init_group, a->b2_init_group, a->x_hat_ln_group, a->std_ln_group, a->Z1_group,
-                   a->Z1_bar_group, a->grad_l_wrt_Z2_group, a->x_hat_fused_group, a->grad_output_fused_group,
-                   a->std_fused_group, a->grad_L_W1_last, a->grad_L_b1_last, a->grad_L_W2_last, a->grad_L_b2_last,
+                   a->W2_init_group, a->b2_init_group, a->x_hat_ln_group, a->std_ln_group, a->X2_group, a->Z1_group,
+                   a->Z1_bar_group, a->X2_bar_group, a->grad_l_wrt_Z2_group, a->grad_l_wrt_Z1_group, a->x_hat_fused_group,
+                   a->grad_x_hat_fused_group, a->grad_output_fused_group, a->std_fused_group, a->grad_L_W1_last, a->grad_L_b1_last, a->grad_L_W2_last, a->grad_L_b2_last,
                    a->grad_L_XQW_mini_batch, a->grad_L_ttt_norm_weight, a->grad_L_ttt_norm_bias, a->grad_L_W1_init,
                    a->grad_L_b1_init, a->grad_L_W2_init, a->grad_L_b2_init, a->grad_L_last_eta, a->grad_L_XQ,
                    a->grad_L_XK, a->grad_L_XV))
@@ -333,6 +335,19 @@ extern "C" int ttt_mlp_fwd_launch_overlapped(const ttt_mlp_fwd_args* a, void* wo
   p.state_img = reinterpret_cast<__bf16*>(base + w.off[1]) - b0 * 2 * ttt::FWD_RING_MAX * (ttt::FWD_IMG_BYTES / 2);
   p.bias_img = reinterpret_cast<float*>(base + w.off[2]) - b0 * 2 * ttt::FWD_RING_MAX * ttt::FWD_BIAS_FLOATS;
   return static_cast<int>(ttt_mlp_fwd_enqueue(p, static_cast<hipStream_t>(stream)));
+}
+
+namespace {
+__global__ void ttt_mlp_or_status(const int* status, int* sticky) {
+  if (*status != 0) *sticky = 1;
+}
+}  // namespace
+
+extern "C" int ttt_mlp_status_accumulate(const void* status_word, int* sticky_word, void* stream) {
+  if (status_word == nullptr || sticky_word == nullptr) return TTT_MLP_ERR_BAD_ARG;
+  hipLaunchKernelGGL(ttt_mlp_or_status, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const int*>(status_word), sticky_word);
+  return static_cast<int>(hipGetLastError());
 }
 
 extern "C" int ttt_mlp_launch_plan(int which, long long pairs, int compute_units, long long* one_workgroup_pairs,

@@ -1,8 +1,8 @@
 // Shared device-side building blocks of the gfx950 TTT-MLP kernels.
 //
-// One workgroup of 4 wavefronts (256 threads) owns one (batch, head) recurrence.  Wave w owns
-// hidden columns [64w, 64w+64) of the inner MLP, so every per-wave contraction is a
-// 64x64x64 bf16 MFMA product with fp32 accumulate, built from 32x32x16 tiles.
+// One workgroup of 8 wavefronts (512 threads, two per SIMD) owns one (batch, head) recurrence, or one
+// role of it.  Wave v owns hidden columns [32v, 32v+32) of the inner MLP, so every per-wave contraction
+// is a 64x64x32 (or 64x32x64) bf16 MFMA product with fp32 accumulate, built from 32x32x16 tiles.
 //
 // Register tile conventions (lane = 32*h + c, h in {0,1}, c in 0..31), verified on hardware:
 //   accumulator block (32x32 fp32, 16 regs): reg i holds row 8*(i/4) + 4*h + (i%4), column c
@@ -31,36 +31,10 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr int CS = 64;         // tokens per mini-batch
 constexpr int FD = 64;         // head dimension
 constexpr int HID = 256;       // hidden dimension of the inner MLP
-constexpr int NWAVE = 4;       // wavefronts per workgroup = hidden shards
-constexpr int NTHREADS = 256;
-constexpr int LDB = 72;        // row stride (elements) of a 64x64 bf16 tile in LDS: 144 B
 constexpr int LDP = 68;        // row stride (floats) of a 64x64 fp32 partial tile in LDS: 272 B
 constexpr float LN_EPS = 1e-8f;
 
 #define TTT_DEV __device__ __forceinline__
-
-struct Acc { f32x16 b[2][2]; };   // 64x64 fp32 tile: b[row block][column block]
-struct Opd { bf16x8 v[2][4]; };   // 64x64 bf16 operand: v[free-index block][k step]
-
-TTT_DEV void acc_zero(Acc& a) {
-#pragma unroll
-  for (int r = 0; r < 2; r++)
-#pragma unroll
-    for (int c = 0; c < 2; c++)
-#pragma unroll
-      for (int i = 0; i < 16; i++) a.b[r][c][i] = 0.f;
-}
-
-// d[row block of a][column block of b] += a * b over the 64-long contraction.
-TTT_DEV void mma(Acc& d, const Opd& a, const Opd& b) {
-#pragma unroll
-  for (int s = 0; s < 4; s++)
-#pragma unroll
-    for (int r = 0; r < 2; r++)
-#pragma unroll
-      for (int c = 0; c < 2; c++)
-        d.b[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v[r][s], b.v[c][s], d.b[r][c], 0, 0, 0);
-}
 
 TTT_DEV bf16x8 pack8(const f32x16& x, int t) {
   bf16x8 o;
@@ -69,81 +43,36 @@ TTT_DEV bf16x8 pack8(const f32x16& x, int t) {
   return o;
 }
 
-// Accumulator tile (rows = contraction index, columns = free index) -> chained operand.
-TTT_DEV Opd cvt_chain(const Acc& x) {
-  Opd o;
+// Two-term bf16 representation of fp32 values: hi = bf16(x), lo = bf16(x - hi), so that hi + lo carries
+// about 16 significant bits.  A matrix product whose operand is split this way is the sum of one MFMA
+// product per term (fp32 accumulate), which keeps the operand rounding of the products that carry the
+// recurrence's state from one mini-batch to the next near 2^-17 instead of 2^-9.
+TTT_DEV void split8(const f32x16& x, int t, bf16x8& hi, bf16x8& lo) {
 #pragma unroll
-  for (int cb = 0; cb < 2; cb++)
+  for (int j = 0; j < 8; j++) {
+    const float v = x[8 * t + j];
+    const bf16 hv = (bf16)v;
+    hi[j] = hv;
+    lo[j] = (bf16)(v - (float)hv);
+  }
+}
+TTT_DEV void split8(const float (&x)[8], bf16x8& hi, bf16x8& lo) {
 #pragma unroll
-    for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-      for (int t = 0; t < 2; t++) o.v[cb][2 * rb + t] = pack8(x.b[rb][cb], t);
-  return o;
+  for (int j = 0; j < 8; j++) {
+    const bf16 hv = (bf16)x[j];
+    hi[j] = hv;
+    lo[j] = (bf16)(x[j] - (float)hv);
+  }
 }
 
 TTT_DEV bf16x8 cat(bf16x4 lo, bf16x4 hi) { return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7); }
 
-// Operand from an LDS tile stored [free index][contraction index] (contraction contiguous),
-// row stride LDB, in kappa order: two 8-byte reads per k-step.
-TTT_DEV Opd lds_rows_kappa(const bf16* base, int c, int h) {
-  Opd o;
-#pragma unroll
-  for (int fb = 0; fb < 2; fb++)
-#pragma unroll
-    for (int s = 0; s < 4; s++) {
-      const bf16* p = base + (32 * fb + c) * LDB + 16 * s + 4 * h;
-      o.v[fb][s] = cat(*reinterpret_cast<const bf16x4*>(p), *reinterpret_cast<const bf16x4*>(p + 8));
-    }
-  return o;
-}
-
+// Transposing LDS read: within each group of 16 lanes, lane i points at row k0 + i/4, columns m0 + 4*(i%4) .. +3,
+// and receives rows k0..k0+3 of column m0 + i.
 TTT_DEV bf16x4 lds_tr4(const bf16* p) {
   typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
   s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
   return __builtin_bit_cast(bf16x4, t);
-}
-
-// Operand from an LDS tile stored [contraction index][free index] (free index contiguous), row
-// stride LDB, in kappa order, using the transposing LDS read: within each group of 16 lanes, lane
-// i points at row k0 + i/4, columns m0 + 4*(i%4) .. +3, and receives rows k0..k0+3 of column m0 + i.
-TTT_DEV Opd lds_tr_kappa(const bf16* base, int lane) {
-  Opd o;
-  const int h = lane >> 5, c = lane & 31, i = lane & 15;
-#pragma unroll
-  for (int fb = 0; fb < 2; fb++)
-#pragma unroll
-    for (int s = 0; s < 4; s++) {
-      const bf16* p = base + (16 * s + 4 * h + (i >> 2)) * LDB + 32 * fb + 16 * (c >> 4) + 4 * (i & 3);
-      o.v[fb][s] = cat(lds_tr4(p), lds_tr4(p + 8 * LDB));
-    }
-  return o;
-}
-
-// Writes a chained operand (lane = free index, slots = contraction index in kappa order) as an LDS
-// tile stored [free index][contraction index]; the inverse of lds_rows_kappa.
-TTT_DEV void lds_store_rows_kappa(bf16* base, const Opd& o, int c, int h) {
-#pragma unroll
-  for (int fb = 0; fb < 2; fb++)
-#pragma unroll
-    for (int s = 0; s < 4; s++) {
-      bf16* p = base + (32 * fb + c) * LDB + 16 * s + 4 * h;
-      *reinterpret_cast<bf16x4*>(p) = __builtin_shufflevector(o.v[fb][s], o.v[fb][s], 0, 1, 2, 3);
-      *reinterpret_cast<bf16x4*>(p + 8) = __builtin_shufflevector(o.v[fb][s], o.v[fb][s], 4, 5, 6, 7);
-    }
-}
-
-// Writes an accumulator tile (lane = column, regs = rows) to an fp32 LDS tile stored
-// [column][row] with row stride LDP: 16-byte writes of 4 consecutive rows.
-TTT_DEV void lds_store_partial(float* base, const Acc& a, int c, int h) {
-#pragma unroll
-  for (int rb = 0; rb < 2; rb++)
-#pragma unroll
-    for (int cb = 0; cb < 2; cb++)
-#pragma unroll
-      for (int g = 0; g < 4; g++) {
-        f32x4 v = {a.b[rb][cb][4 * g], a.b[rb][cb][4 * g + 1], a.b[rb][cb][4 * g + 2], a.b[rb][cb][4 * g + 3]};
-        *reinterpret_cast<f32x4*>(base + (32 * cb + c) * LDP + 32 * rb + 8 * g + 4 * h) = v;
-      }
 }
 
 // ---------------------------------------------------------------------------- cross-lane
@@ -216,6 +145,56 @@ TTT_DEV OpdT<CB, 2 * RB> cvt_chain(const AccT<RB, CB>& x) {
 #pragma unroll
       for (int t = 0; t < 2; t++) o.v[cb][2 * rb + t] = pack8(x.b[rb][cb], t);
   return o;
+}
+
+// The same with the operand split into two bf16 terms.
+template <int RB, int CB>
+TTT_DEV void cvt_chain_split(const AccT<RB, CB>& x, OpdT<CB, 2 * RB>& hi, OpdT<CB, 2 * RB>& lo) {
+#pragma unroll
+  for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+      for (int t = 0; t < 2; t++) split8(x.b[rb][cb], t, hi.v[cb][2 * rb + t], lo.v[cb][2 * rb + t]);
+}
+
+// d += A * B over KS k-steps, operand pieces produced by the callables fa(row block, s) and fb(column block, s)
+// right before the MFMAs that consume them, so that no whole operand is resident in registers.
+template <int KS, int RB, int CB, class FA, class FB>
+TTT_DEV void mma_jit(AccT<RB, CB>& d, FA fa, FB fb) {
+#pragma unroll
+  for (int s = 0; s < KS; s++) {
+    bf16x8 a[RB], b[CB];
+#pragma unroll
+    for (int r = 0; r < RB; r++) a[r] = fa(r, s);
+#pragma unroll
+    for (int c = 0; c < CB; c++) b[c] = fb(c, s);
+#pragma unroll
+    for (int r = 0; r < RB; r++)
+#pragma unroll
+      for (int c = 0; c < CB; c++) d.b[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[r], b[c], d.b[r][c], 0, 0, 0);
+  }
+}
+
+// ---------------------------------------------------------------------------- just-in-time operand pieces
+// One MFMA operand piece = 8 bf16 per lane = (free block blk, k-step s).  Loading pieces right
+// before the MFMA that consumes them keeps whole operands out of the register file.
+template <int LD>
+TTT_DEV bf16x8 piece_rows(const bf16* tile, int blk, int s, int c, int h) {
+  const bf16* q = tile + (32 * blk + c) * LD + 16 * s + 4 * h;
+  return cat(*reinterpret_cast<const bf16x4*>(q), *reinterpret_cast<const bf16x4*>(q + 8));
+}
+template <int LD>
+TTT_DEV bf16x8 piece_tr(const bf16* tile, int blk, int s, int lane) {
+  const int h = lane >> 5, c = lane & 31, i = lane & 15;
+  const bf16* q = tile + (16 * s + 4 * h + (i >> 2)) * LD + 32 * blk + 16 * (c >> 4) + 4 * (i & 3);
+  return cat(lds_tr4(q), lds_tr4(q + 8 * LD));
+}
+template <int LD>
+TTT_DEV void store_piece_rows(bf16* tile, int blk, int s, int c, int h, bf16x8 v) {
+  bf16* q = tile + (32 * blk + c) * LD + 16 * s + 4 * h;
+  *reinterpret_cast<bf16x4*>(q) = __builtin_shufflevector(v, v, 0, 1, 2, 3);
+  *reinterpret_cast<bf16x4*>(q + 8) = __builtin_shufflevector(v, v, 4, 5, 6, 7);
 }
 
 // Operand from an LDS tile stored [free index][contraction index], row stride ld elements.
@@ -395,10 +374,12 @@ TTT_DEV bool wait_at_least(int* word, int target, int* status, int* s_flag, uint
   return *s_flag != 0;
 }
 // Everything this workgroup has written (or read) so far is ordered before the new value of `word`: every
-// wave's accesses are complete at the barrier, then one thread releases them at agent scope (a release by
-// every wave would write the L2 back eight times over).
+// wave drains its own outstanding memory operations (a workgroup-scope release alone does not wait for
+// stores that are still in flight), the barrier collects the waves, then one thread writes the L2 back at
+// agent scope (a release by every wave would write it back eight times over) and stores the counter.
 TTT_DEV void publish(int* word, int value) {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
   __syncthreads();
   if (threadIdx.x == 0) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");

@@ -13,6 +13,11 @@
 //   W2s = W2[shard, :]      (rows hid, columns F)    -> chained operand of (X2*W2)^T
 //   W2t = W2[shard, :]^T    (rows F,   columns hid)  -> chained operand of gZ2*W2^T
 // so no weight ever goes through LDS; the eta-scaled updates are MFMA accumulations into them.
+// Operand precision: the products that carry the state from one mini-batch to the next (XK W1, X2 W2,
+// G2 W2^T and the two weight steps) take their fp32 operands - the weights, G2 = -eta dl/dZ2, G1 and, in
+// the W2 step, X2 - as two bf16 terms (hi + lo, one MFMA product per term; XK is bf16 already), because
+// a single bf16 rounding of them, repeated over thousands of mini-batches, moves the gradients of the
+// remat backward further from the fp32 mathematics than cosine 0.9999.  The output branch uses one term.
 // Sums over the hidden dimension (Z2) are formed in two steps: waves v and v+4 exchange halves of
 // their partial tiles through LDS and each finishes one half, then every wave LayerNorms 8 of the
 // 64 tokens (8 lanes per token) from the four pair sums.  All sums have a fixed order.
@@ -28,6 +33,7 @@ constexpr int FW_NS = HID / FW_NWAVE;                  // hidden columns per wav
 // an operand piece on 64 distinct banks (measured: 8.6 clocks per piece against 16 with 144-byte
 // rows); rows are 8-byte aligned, so 16-byte accesses are made as two 8-byte ones.
 constexpr int FLD = 68;
+#define MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16((a), (b), (c), 0, 0, 0)
 
 // LDS carve-up (bytes)
 constexpr int SM_TILE = 64 * FLD * 2;                   // one bf16 tile: 8704
@@ -35,7 +41,8 @@ constexpr int SM_XQ = 0;                                // two buffers, alternat
 constexpr int SM_XK = SM_XQ + 2 * SM_TILE;
 constexpr int SM_XV = SM_XK + SM_TILE;
 constexpr int SM_G2 = SM_XV + SM_TILE;
-constexpr int SM_P = SM_G2 + SM_TILE;                    // 4 fp32 pair-sum tiles [tok][F]
+constexpr int SM_G2L = SM_G2 + SM_TILE;                  // low-order bf16 term of G2
+constexpr int SM_P = SM_G2L + SM_TILE;                   // 4 fp32 pair-sum tiles [tok][F]
 constexpr int SM_PTILE = 64 * LDP * 4;
 constexpr int SM_X2T = SM_P + 4 * SM_PTILE;             // per wave: X2 shard stored [hid][tok], bf16
 constexpr int SM_X2T_TILE = FW_NS * FLD * 2;
@@ -158,6 +165,7 @@ TTT_DEV void output_layernorm(const float* s_P, const float* s_b2, const float* 
 template <int ROLE, int RING>
 TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
   bf16* s_g2 = reinterpret_cast<bf16*>(smem + SM_G2);
+  bf16* s_g2l = reinterpret_cast<bf16*>(smem + SM_G2L);
   float* s_P = reinterpret_cast<float*>(smem + SM_P);
   float* s_b1 = reinterpret_cast<float*>(smem + SM_B1);
   float* s_b2 = reinterpret_cast<float*>(smem + SM_B2);
@@ -250,7 +258,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
       LANE_VARS;
       if constexpr (ROLE == 1) __syncthreads();   // b2 as waves 0 and 1 left it (no barrier ends a mini-batch in this role)
       const size_t slot = (size_t)bh * p.K + mb / p.cgs;
-      const unsigned ck = (mb / p.cgs) * (FD * HID * 4);   // byte offset of the slot in gW1ck / gW2ck
+      const unsigned ck = static_cast<unsigned>(mb / p.cgs) * (FD * HID * 4u);   // byte offset of the slot in gW1ck / gW2ck
 #pragma unroll
       for (int b = 0; b < 2; b++)
 #pragma unroll
@@ -267,13 +275,15 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
     AccT<2, 1> x2, d1;
     {
       LANE_VARS;
-      const OpdT<1, 4> w1op = cvt_chain(W1s);
+      OpdT<1, 4> w1h, w1l;
+      cvt_chain_split(W1s, w1h, w1l);
       const OpdT<2, 4> xkA = lds_rows_kappa<2, 4>(s_xk, FLD, c, h);
 #pragma unroll
       for (int rb = 0; rb < 2; rb++)
 #pragma unroll
         for (int i = 0; i < 16; i++) x2.b[rb][0][i] = b1L;
-      mma(x2, xkA, w1op);
+      mma(x2, xkA, w1l);
+      mma(x2, xkA, w1h);
 #pragma unroll
       for (int rb = 0; rb < 2; rb++)
 #pragma unroll
@@ -284,7 +294,8 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
           d1.b[rb][0][i] = d;
         }
     }
-    const OpdT<1, 4> x2op = cvt_chain(x2);                  // lane = hid, contraction = tok
+    OpdT<1, 4> x2op, x2lo;                                  // lane = hid, contraction = tok; two terms for the W2 step
+    cvt_chain_split(x2, x2op, x2lo);
     {
       LANE_VARS;
       lds_store_rows_kappa<1, 4>(s_x2t, FLD, x2op, c, h);   // stored [hid][tok], private to the wave
@@ -294,11 +305,13 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
     // ---- Z2^T partial = W2s^T X2^T (rows F, lane = tok), summed over the pair into [tok][F]
     {
       LANE_VARS;
-      const OpdT<2, 2> w2A = cvt_chain(W2s);
+      OpdT<2, 2> w2h, w2l;
+      cvt_chain_split(W2s, w2h, w2l);
       const OpdT<2, 2> x2B = lds_tr_kappa<2, 2>(s_x2t, FLD, lane);
       AccT<2, 2> z2;
       acc_zero(z2);
-      mma(z2, w2A, x2B);
+      mma(z2, w2l, x2B);
+      mma(z2, w2h, x2B);
       pair_sum_to_lds(s_Pp, z2, pr, c, h);
     }
 
@@ -356,10 +369,12 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
       s1 = oct_sum(s1);
       s2 = oct_sum(s2);
       const float scale = -s_eta[tok] * rstd * (1.f / FD);  // G2 = -eta * dl/dZ2
-      bf16x8 o;
+      bf16x8 o, ol;
 #pragma unroll
-      for (int e = 0; e < 8; e++) o[e] = (bf16)((FD * gx[e] - s1 - z[e] * s2) * scale);
+      for (int e = 0; e < 8; e++) gx[e] = (FD * gx[e] - s1 - z[e] * s2) * scale;
+      split8(gx, o, ol);
       lds_put16(s_g2 + tok * FLD + f0, __builtin_bit_cast(u32x4, o));
+      lds_put16(s_g2l + tok * FLD + f0, __builtin_bit_cast(u32x4, ol));
       if constexpr (ROLE == 1) {
         if (mb + 1 < p.NC) {
           const int off = ((tid >> 3) * FLD + (tid & 7) * 8) * 2;
@@ -374,11 +389,28 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
     // ---- G1 = (G2 W2^T) * gelu'(Z1);  state += X^T G
     {
       LANE_VARS;
-      const OpdT<2, 4> g2A = lds_rows_kappa<2, 4>(s_g2, FLD, c, h);   // lane = tok, contraction = F
-      const OpdT<1, 4> w2tB = cvt_chain(W2t);                          // lane = hid, contraction = F
+      // g1 = G2 W2^T: G2 rows from LDS (lane = tok, contraction = F), W2t chained (lane = hid, contraction = F)
       AccT<2, 1> g1;
       acc_zero(g1);
-      mma(g1, g2A, w2tB);                                              // rows tok, lane = hid
+      {
+        OpdT<1, 4> wh, wl;
+        cvt_chain_split(W2t, wh, wl);
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+          bf16x8 ah[2], al[2];
+#pragma unroll
+          for (int rb = 0; rb < 2; rb++) {
+            ah[rb] = piece_rows<FLD>(s_g2, rb, s, c, h);
+            al[rb] = piece_rows<FLD>(s_g2l, rb, s, c, h);
+          }
+#pragma unroll
+          for (int rb = 0; rb < 2; rb++) {
+            g1.b[rb][0] = MFMA(al[rb], wh.v[0][s], g1.b[rb][0]);
+            g1.b[rb][0] = MFMA(ah[rb], wl.v[0][s], g1.b[rb][0]);
+            g1.b[rb][0] = MFMA(ah[rb], wh.v[0][s], g1.b[rb][0]);
+          }
+        }
+      }
       float colsum = 0.f;
 #pragma unroll
       for (int rb = 0; rb < 2; rb++)
@@ -387,33 +419,64 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
           g1.b[rb][0][i] *= d1.b[rb][0][i];
           colsum += g1.b[rb][0][i];
         }
-      const OpdT<1, 4> g1op = cvt_chain(g1);                           // lane = hid, contraction = tok
       b1L += half_sum(colsum);
-      const OpdT<2, 4> g2T = lds_tr_kappa<2, 4>(s_g2, FLD, lane);      // lane = F, contraction = tok
-      mma(W2s, x2op, g2T);                                             // W2[shard,:]   += X2^T G2
-      mma(W2t, g2T, x2op);                                             // W2[shard,:]^T += G2^T X2
-      if (v < 2) {                                                     // b2 += column sums of G2 (rows 32v..32v+32)
-        f32x16 b2acc;
+      {   // W1[:,shard] += XK^T G1, G1 chained in two terms (lane = hid, contraction = tok)
+        OpdT<1, 4> g1h, g1l;
+        cvt_chain_split(g1, g1h, g1l);
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+          bf16x8 xk[2];
+#pragma unroll
+          for (int fb = 0; fb < 2; fb++) xk[fb] = piece_tr<FLD>(s_xk, fb, s, lane);      // lane = F, contraction = tok
+#pragma unroll
+          for (int fb = 0; fb < 2; fb++) {
+            W1s.b[fb][0] = MFMA(xk[fb], g1l.v[0][s], W1s.b[fb][0]);
+            W1s.b[fb][0] = MFMA(xk[fb], g1h.v[0][s], W1s.b[fb][0]);
+          }
+        }
+      }
+      // W2[shard,:] += X2^T G2 and its transpose: X2 chained (two terms), G2 through the transposing read
+      // (lane = F, contraction = tok; two terms); b2 += column sums of G2 (waves 0 and 1, rows 32v..32v+32)
+      f32x16 b2acc;
+      if (v < 2) {
 #pragma unroll
         for (int g = 0; g < 4; g++) {
           const f32x4 x = *reinterpret_cast<const f32x4*>(s_b2 + 32 * v + 8 * g + 4 * h);
 #pragma unroll
           for (int e = 0; e < 4; e++) b2acc[4 * g + e] = x[e];
         }
+      }
 #pragma unroll
-        for (int s = 0; s < 4; s++)
-          b2acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v == 0 ? g2T.v[0][s] : g2T.v[1][s], ones, b2acc, 0, 0, 0);
-        if (c == 0) {                                                  // read after the next workgroup barrier
+      for (int s = 0; s < 4; s++) {
+        bf16x8 gh[2], gl[2];
 #pragma unroll
-          for (int g = 0; g < 4; g++) {
-            f32x4 x = {b2acc[4 * g], b2acc[4 * g + 1], b2acc[4 * g + 2], b2acc[4 * g + 3]};
-            *reinterpret_cast<f32x4*>(s_b2 + 32 * v + 8 * g + 4 * h) = x;
-            if constexpr (ROLE == 1) *reinterpret_cast<f32x4*>(gB + HID + 32 * v + 8 * g + 4 * h) = x;
-          }
+        for (int fb = 0; fb < 2; fb++) {
+          gh[fb] = piece_tr<FLD>(s_g2, fb, s, lane);
+          gl[fb] = piece_tr<FLD>(s_g2l, fb, s, lane);
+        }
+        const bf16x8 xh = x2op.v[0][s], xl = x2lo.v[0][s];
+#pragma unroll
+        for (int fb = 0; fb < 2; fb++) {
+          W2s.b[0][fb] = MFMA(xl, gh[fb], W2s.b[0][fb]);
+          W2s.b[0][fb] = MFMA(xh, gl[fb], W2s.b[0][fb]);
+          W2s.b[0][fb] = MFMA(xh, gh[fb], W2s.b[0][fb]);
+          W2t.b[fb][0] = MFMA(gh[fb], xl, W2t.b[fb][0]);
+          W2t.b[fb][0] = MFMA(gl[fb], xh, W2t.b[fb][0]);
+          W2t.b[fb][0] = MFMA(gh[fb], xh, W2t.b[fb][0]);
+        }
+        if (v < 2) {
+          b2acc = MFMA(v == 0 ? gl[0] : gl[1], ones, b2acc);
+          b2acc = MFMA(v == 0 ? gh[0] : gh[1], ones, b2acc);
         }
       }
-      const OpdT<2, 4> xkT = lds_tr_kappa<2, 4>(s_xk, FLD, lane);      // lane = F, contraction = tok
-      mma(W1s, xkT, g1op);                                             // W1[:,shard]   += XK^T G1
+      if (v < 2 && c == 0) {                                           // read after the next workgroup barrier
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          f32x4 x = {b2acc[4 * g], b2acc[4 * g + 1], b2acc[4 * g + 2], b2acc[4 * g + 3]};
+          *reinterpret_cast<f32x4*>(s_b2 + 32 * v + 8 * g + 4 * h) = x;
+          if constexpr (ROLE == 1) *reinterpret_cast<f32x4*>(gB + HID + 32 * v + 8 * g + 4 * h) = x;
+        }
+      }
     }
     if constexpr (ROLE != 1) {
       LANE_VARS;
