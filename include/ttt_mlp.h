@@ -43,6 +43,7 @@ extern "C" {
 #define TTT_MLP_ERR_TOO_LARGE 1004 /* B*NH > 2^31-1, NC > 2^18, cgs > 2^16 or K > 2^15 */
 #define TTT_MLP_ERR_NO_ROOM 1005   /* 2*B*NH workgroups exceed the CUs of the device */
 #define TTT_MLP_ERR_WORKSPACE 1006 /* workspace smaller than required              */
+#define TTT_MLP_ERR_SCRATCH 1007   /* more (batch, head) pairs than the fixed scratch of ttt_mlp_fwd_launch_static serves */
 
 /* Forward scan.  Replaces the 16 positional arguments of `ttt_forward`
  * (test_time_training.cpp:25-42).  bf16 tensors are passed as uint16_t bit patterns. */
@@ -171,6 +172,17 @@ size_t ttt_mlp_fwd_workspace_bytes(int32_t B, int32_t NH);
 size_t ttt_mlp_fwd_status_offset(int32_t B, int32_t NH);
 int ttt_mlp_fwd_launch_overlapped(const ttt_mlp_fwd_args* args, void* workspace, size_t workspace_bytes, void* stream);
 int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* args, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ttt_mlp_fwd_launch_overlapped for callers that cannot allocate device memory and have no workspace to
+ * pass - code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart
+ * in the reference.  Same kernels and bit-identical results; the workspace is a fixed array in the
+ * library's device memory (32.6 MiB per GPU, held until the process ends), so the call allocates nothing
+ * and serves at most 8 (batch, head) pairs: B*NH > 8 returns TTT_MLP_ERR_SCRATCH, a device without room
+ * for two workgroups per pair TTT_MLP_ERR_NO_ROOM, before anything is enqueued.  Every call on a GPU uses
+ * that GPU's one array: calls that overlap in time on one GPU (two streams, two threads) race - serialise
+ * them.  `sticky_word` (may be NULL): a device int owned by the caller; as ttt_mlp_status_accumulate, the
+ * call enqueues `if (status != 0) *sticky_word = 1` behind the kernels. */
+int ttt_mlp_fwd_launch_static(const ttt_mlp_fwd_args* args, int* sticky_word, void* stream);
 
 /* For callers that do not wait for the stream after an overlapped launch (and may free or reuse the
  * workspace before they do): enqueues, behind the launch on the same stream, `if (*status_word != 0)

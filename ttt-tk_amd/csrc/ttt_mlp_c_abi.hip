@@ -44,6 +44,7 @@ extern "C" const char* ttt_mlp_error_string(int code) {
     case TTT_MLP_ERR_TOO_LARGE: return "ttt_mlp: B*NH exceeds the launch grid limit, or NC > 262144, or checkpoint_group_size > 65536, or more than 32768 checkpoints";
     case TTT_MLP_ERR_NO_ROOM: return "ttt_mlp: two workgroups per (batch, head) do not fit the compute units of this device; use ttt_mlp_bwd_launch";
     case TTT_MLP_ERR_WORKSPACE: return "ttt_mlp: workspace smaller than ttt_mlp_bwd_workspace_bytes()";
+    case TTT_MLP_ERR_SCRATCH: return "ttt_mlp: ttt_mlp_fwd_launch_static serves at most 8 (batch, head) pairs (B*NH <= 8): its workspace is a fixed array in device memory";
     default: return hipGetErrorString(static_cast<hipError_t>(code));
   }
 }
@@ -337,7 +338,41 @@ extern "C" int ttt_mlp_fwd_launch_overlapped(const ttt_mlp_fwd_args* a, void* wo
   return static_cast<int>(ttt_mlp_fwd_enqueue(p, static_cast<hipStream_t>(stream)));
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// The two-workgroup forward for callers that cannot allocate and have no workspace to bring: its workspace
+// is this fixed array (one copy per GPU, held until the process ends).  Host code never passes the array's
+// name to a kernel - the name is a host-side stand-in, not a device address; the address on each device
+// comes from hipGetSymbolAddress, once per device.
 namespace {
+constexpr int STATIC_MAX_PAIRS = 8;
+constexpr size_t static_scratch_bytes() {
+  // FwdWorkspace(STATIC_MAX_PAIRS): synchronisation words, state images, bias vectors; each part 256-byte aligned
+  const size_t slots = (size_t)STATIC_MAX_PAIRS * 2 * ttt::FWD_RING_MAX;
+  const size_t a = ((STATIC_MAX_PAIRS * ttt::BWD_SYNC_STRIDE + 32) * sizeof(int) + 255) & ~(size_t)255;
+  const size_t b = (slots * ttt::FWD_IMG_BYTES + 255) & ~(size_t)255;
+  const size_t c = (slots * ttt::FWD_BIAS_FLOATS * sizeof(float) + 255) & ~(size_t)255;
+  return a + b + c;
+}
+static __device__ __align__(256) unsigned char scratch[static_scratch_bytes()];   // 32.6 MiB
+
+constexpr int MAX_DEVICES = 64;
+void* g_scratch_ptr[MAX_DEVICES] = {};   // address of `scratch` on each device, looked up at the first call there
+
+// The current device's copy of the array (the device that the launch goes to).  Looked up once per device.
+int static_scratch(void** ptr) {
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev)) return static_cast<int>(e);
+  if (dev < 0 || dev >= MAX_DEVICES) return TTT_MLP_ERR_BAD_ARG;
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch))) return static_cast<int>(e);
+    if (p == nullptr) return TTT_MLP_ERR_BAD_ARG;
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return TTT_MLP_OK;
+}
+
 __global__ void ttt_mlp_or_status(const int* status, int* sticky) {
   if (*status != 0) *sticky = 1;
 }
@@ -348,6 +383,29 @@ extern "C" int ttt_mlp_status_accumulate(const void* status_word, int* sticky_wo
   hipLaunchKernelGGL(ttt_mlp_or_status, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream),
                      static_cast<const int*>(status_word), sticky_word);
   return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int ttt_mlp_fwd_launch_static(const ttt_mlp_fwd_args* a, int* sticky_word, void* stream) {
+  ttt::FwdParams p;
+  if (int rc = make_fwd_params(a, p)) return rc;
+  const long long pairs = (long long)p.B * p.NH;
+  if (pairs > STATIC_MAX_PAIRS) return TTT_MLP_ERR_SCRATCH;
+  const LaunchPlan pl = plan_launches(pairs, false, false);
+  if (!pl.rest_split || pl.n_single != 0) return TTT_MLP_ERR_NO_ROOM;
+  const FwdWorkspace w(pl.n_rest);
+  static_assert(static_scratch_bytes() % 256 == 0, "scratch parts are 256-byte aligned");
+  if (w.total > static_scratch_bytes()) return TTT_MLP_ERR_SCRATCH;
+  void* ws = nullptr;
+  if (int rc = static_scratch(&ws)) return rc;
+  // From here on as ttt_mlp_fwd_launch_overlapped with `ws` as the workspace: the launch clears the
+  // synchronisation words and the status word itself (a small kernel ahead of the main one), everything
+  // else in the workspace is written before it is read.
+  if (int rc = ttt_mlp_fwd_launch_overlapped(a, ws, static_scratch_bytes(), stream)) return rc;
+  if (sticky_word != nullptr) {
+    const int* status = reinterpret_cast<const int*>(static_cast<const char*>(ws) + w.off[0]) + (size_t)pl.n_rest * ttt::BWD_SYNC_STRIDE;
+    return ttt_mlp_status_accumulate(status, sticky_word, stream);
+  }
+  return TTT_MLP_OK;
 }
 
 extern "C" int ttt_mlp_launch_plan(int which, long long pairs, int compute_units, long long* one_workgroup_pairs,
