@@ -11,8 +11,10 @@
 // as MFMA accumulator tiles:
 //   W1s = W1[:, shard]      (rows F,   columns hid)  -> chained operand of XK*W1 and of (XQ*W1)^T
 //   W2s = W2[shard, :]      (rows hid, columns F)    -> chained operand of (X2*W2)^T
-//   W2t = W2[shard, :]^T    (rows F,   columns hid)  -> chained operand of gZ2*W2^T
-// so no weight ever goes through LDS; the eta-scaled updates are MFMA accumulations into them.
+// and the eta-scaled updates are MFMA accumulations into them.  Only gZ2*W2^T needs W2 with the other index
+// contracted: for it the two bf16 terms of W2s are transposed through a wave-private LDS tile once per mini-batch
+// (a second resident copy W2^T, kept up to date by a second set of update products, cost 32 registers and a
+// third more MFMA work, and the registers are what this kernel is short of).
 // Operand precision: the products that carry the state from one mini-batch to the next (XK W1, X2 W2,
 // G2 W2^T and the two weight steps) take their fp32 operands - the weights, G2 = -eta dl/dZ2, G1 and, in
 // the W2 step, X2 - as two bf16 terms (hi + lo, one MFMA product per term; XK is bf16 already), because
@@ -34,9 +36,33 @@ constexpr int FW_NS = HID / FW_NWAVE;                  // hidden columns per wav
 // rows); rows are 8-byte aligned, so 16-byte accesses are made as two 8-byte ones.
 constexpr int FLD = 68;
 #define MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16((a), (b), (c), 0, 0, 0)
+// The input tiles (XQ, XK, XV) sit in LDS as pairs of rows: two rows of 128 bytes back to back, pairs 264 bytes
+// apart.  A pair is what one wave-wide 4-byte LDS-direct load (global_load_lds_dword: lane l writes base + 4 l)
+// delivers, so a tile can travel from HBM to LDS without passing through registers, and the 8 bytes between
+// pairs put the 32 row-wise 8-byte reads of an operand piece on 64 distinct banks.
+constexpr int XPAIR = 132;   // elements from one pair of rows to the next
+TTT_DEV int xrow(int r) { return (r >> 1) * XPAIR + (r & 1) * 64; }
+TTT_DEV bf16x8 xpiece_rows(const bf16* tile, int blk, int s, int c, int h) {
+  const bf16* q = tile + xrow(32 * blk + c) + 16 * s + 4 * h;
+  return cat(*reinterpret_cast<const bf16x4*>(q), *reinterpret_cast<const bf16x4*>(q + 8));
+}
+TTT_DEV bf16x8 xpiece_tr(const bf16* tile, int blk, int s, int lane) {
+  const int h = lane >> 5, c = lane & 31, i = lane & 15;
+  const bf16* q = tile + xrow(16 * s + 4 * h + (i >> 2)) + 32 * blk + 16 * (c >> 4) + 4 * (i & 3);
+  return cat(lds_tr4(q), lds_tr4(q + 4 * XPAIR));   // 8 rows on = 4 pairs on
+}
+TTT_DEV OpdT<2, 4> x_rows_kappa(const bf16* tile, int c, int h) {
+  OpdT<2, 4> o;
+#pragma unroll
+  for (int fb = 0; fb < 2; fb++)
+#pragma unroll
+    for (int s = 0; s < 4; s++) o.v[fb][s] = xpiece_rows(tile, fb, s, c, h);
+  return o;
+}
 
 // LDS carve-up (bytes)
 constexpr int SM_TILE = 64 * FLD * 2;                   // one bf16 tile: 8704
+static_assert(32 * 132 * 2 <= SM_TILE, "a tile of row pairs fits a tile slot");
 constexpr int SM_XQ = 0;                                // two buffers, alternating per mini-batch
 constexpr int SM_XK = SM_XQ + 2 * SM_TILE;
 constexpr int SM_XV = SM_XK + SM_TILE;
@@ -65,7 +91,7 @@ TTT_DEV bf16x8 lds_get8h(const bf16* p) { return cat(*reinterpret_cast<const bf1
 
 struct Staged {  // one mini-batch of inputs in flight from HBM: one 16-byte chunk per tile per thread
   u32x4 q, k, v;
-  float eta;
+  bf16 eta;
 };
 
 // gq / gk / gv / ge = this (batch, head)'s XQ, XK, XV, last_eta; thread tid moves 16-byte chunk tid
@@ -75,15 +101,15 @@ TTT_DEV void stage_load(Staged& s, gptr_t gq, gptr_t gk, gptr_t gv, gptr_t ge, i
   s.q = g_ld16(gq, 16 * tid, mb * TILE_BYTES);
   s.k = g_ld16(gk, 16 * tid, mb * TILE_BYTES);
   s.v = g_ld16(gv, 16 * tid, mb * TILE_BYTES);
-  s.eta = bf2f(g_ldh(ge, 2 * (tid & (CS - 1)), mb * (CS * 2)));   // threads >= CS drop it
+  s.eta = g_ldh(ge, 2 * (tid & (CS - 1)), mb * (CS * 2));   // threads >= CS drop it
 }
 
 TTT_DEV void stage_store(const Staged& s, unsigned char* smem, int xq_buf, int tid) {
-  const int off = ((tid >> 3) * FLD + (tid & 7) * 8) * 2;
+  const int off = (xrow(tid >> 3) + (tid & 7) * 8) * 2;
   lds_put16(smem + SM_XQ + xq_buf * SM_TILE + off, s.q);
   lds_put16(smem + SM_XK + off, s.k);
   lds_put16(smem + SM_XV + off, s.v);
-  if (tid < CS) reinterpret_cast<float*>(smem + SM_ETA)[tid] = s.eta;
+  if (tid < CS) reinterpret_cast<bf16*>(smem + SM_ETA)[tid] = s.eta;   // eta stays bf16 in LDS
 }
 
 // Two-step sum over the wave pair (v, v ^ 4) of a partial tile z (rows F, columns tok): the wave
@@ -120,6 +146,43 @@ TTT_DEV void pair_sum_to_lds(float* tile, const AccT<2, 2>& z, int r, int c, int
   __syncthreads();
 }
 
+// The same sum with the product formed one F block at a time - `half(rb)` returns rows [32 rb, 32 rb + 32) of
+// the partial tile - so that 32 accumulator registers are live instead of 64: first the block that is given away,
+// then the one that is kept.
+template <int R, class HALF>
+TTT_DEV void pair_sum_halves_r(float* tile, HALF half, int c, int h) {
+  {
+    const AccT<1, 2> z = half(1 - R);
+#pragma unroll
+    for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const f32x16& x = z.b[0][cb];
+        f32x4 v = {x[4 * g], x[4 * g + 1], x[4 * g + 2], x[4 * g + 3]};
+        *reinterpret_cast<f32x4*>(tile + (32 * cb + c) * LDP + 32 * (1 - R) + 8 * g + 4 * h) = v;
+      }
+  }
+  const AccT<1, 2> z = half(R);
+  __syncthreads();
+#pragma unroll
+  for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      float* q = tile + (32 * cb + c) * LDP + 32 * R + 8 * g + 4 * h;
+      const f32x16& x = z.b[0][cb];
+      f32x4 v = *reinterpret_cast<const f32x4*>(q);
+      v[0] += x[4 * g]; v[1] += x[4 * g + 1]; v[2] += x[4 * g + 2]; v[3] += x[4 * g + 3];
+      *reinterpret_cast<f32x4*>(q) = v;
+    }
+  __syncthreads();
+}
+template <class HALF0, class HALF1>
+TTT_DEV void pair_sum_halves(float* tile, HALF0 half0, HALF1 half1, int r, int c, int h) {
+  // half0 / half1: the product's F block 0 / 1 (two callables so that each indexes the state registers statically)
+  if (r == 0) pair_sum_halves_r<0>(tile, [&](int rb) { return rb == 0 ? half0() : half1(); }, c, h);
+  else pair_sum_halves_r<1>(tile, [&](int rb) { return rb == 0 ? half0() : half1(); }, c, h);
+}
+
 // Output LayerNorm + residual for the 8 features [f0, f0+8) of token `tok`: Out = XQ + LN(sum of the four
 // pair sums + b2).  8 lanes per token, 8 tokens per wave.
 TTT_DEV void output_layernorm(const float* s_P, const float* s_b2, const float* s_gam, const float* s_bet,
@@ -144,7 +207,7 @@ TTT_DEV void output_layernorm(const float* s_P, const float* s_b2, const float* 
 #pragma unroll
   for (int e = 0; e < 8; e++) { z[e] -= mu; var = __builtin_fmaf(z[e], z[e], var); }
   const float rstd = __builtin_amdgcn_rsqf(oct_sum(var) * (1.f / FD) + LN_EPS);
-  const bf16x8 qv = lds_get8h(s_xq + tok * FLD + f0);
+  const bf16x8 qv = lds_get8h(s_xq + xrow(tok) + f0);
   float gam[8], bet[8];
 #pragma unroll
   for (int q = 0; q < 2; q++) {
@@ -191,7 +254,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
   (void)h; (void)c; (void)tid; (void)tok; (void)f0
 
   // ---- state -> registers
-  AccT<2, 1> W1s, W2t;
+  AccT<2, 1> W1s;
   AccT<1, 2> W2s;
   float b1L;      // b1 of hidden column hid0 + c; b2 lives in LDS (fp32) and is updated there by waves 0 and 1
   {
@@ -202,7 +265,6 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
       for (int i = 0; i < 16; i++) {
         const int row = 8 * (i >> 2) + (i & 3);   // + 4h in the lane offset
         W1s.b[b][0][i] = g_ldf(W1, (4 * h * HID + c) * 4, ((32 * b + row) * HID + hid0) * 4);
-        W2t.b[b][0][i] = g_ldf(W2, (c * FD + 4 * h) * 4, (hid0 * FD + 32 * b + row) * 4);
         W2s.b[0][b][i] = g_ldf(W2, (4 * h * FD + c) * 4, ((hid0 + row) * FD + 32 * b) * 4);
       }
     b1L = p.b1[(size_t)bh * HID + hid0 + c];
@@ -243,7 +305,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
     const int alt = ROLE == 1 ? (mb & 1) : 0;
     const bf16* s_xk = reinterpret_cast<const bf16*>(smem + (alt ? SM_XQ : SM_XK));
     const bf16* s_xv = reinterpret_cast<const bf16*>(smem + (alt ? SM_XQ + SM_TILE : SM_XV));
-    const float* s_eta = reinterpret_cast<const float*>(smem + (alt ? SM_B1 : SM_ETA));
+    const bf16* s_eta = reinterpret_cast<const bf16*>(smem + (alt ? SM_B1 : SM_ETA));
     // ROLE 1: where the state after this mini-batch goes (a ring of 2 * ring slots)
     constexpr int ring = RING; const int grp = mb / ring, at = mb % ring, slot = (grp & 1) * ring + at;
     float* const gB = p.bias_img + ((size_t)bh * 2 * FWD_RING_MAX + slot) * FWD_BIAS_FLOATS;
@@ -253,10 +315,14 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
       }
     }
 
+    // ROLE 1 ends a mini-batch without a barrier: this one makes the inputs staged at the end of the last mini-batch
+    // visible, and b2 as waves 0 and 1 left it
+    if constexpr (ROLE == 1) {
+      if (mb > 0) __syncthreads();
+    }
     // ---- checkpoint: the state before this mini-batch
     if (mb % p.cgs == 0) {
       LANE_VARS;
-      if constexpr (ROLE == 1) __syncthreads();   // b2 as waves 0 and 1 left it (no barrier ends a mini-batch in this role)
       const size_t slot = (size_t)bh * p.K + mb / p.cgs;
       const unsigned ck = static_cast<unsigned>(mb / p.cgs) * (FD * HID * 4u);   // byte offset of the slot in gW1ck / gW2ck
 #pragma unroll
@@ -277,7 +343,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
       LANE_VARS;
       OpdT<1, 4> w1h, w1l;
       cvt_chain_split(W1s, w1h, w1l);
-      const OpdT<2, 4> xkA = lds_rows_kappa<2, 4>(s_xk, FLD, c, h);
+      const OpdT<2, 4> xkA = x_rows_kappa(s_xk, c, h);
 #pragma unroll
       for (int rb = 0; rb < 2; rb++)
 #pragma unroll
@@ -294,35 +360,60 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
           d1.b[rb][0][i] = d;
         }
     }
-    OpdT<1, 4> x2op, x2lo;                                  // lane = hid, contraction = tok; two terms for the W2 step
-    cvt_chain_split(x2, x2op, x2lo);
+    OpdT<1, 4> x2lo;                                        // lane = hid, contraction = tok: the low-order term, for the W2 step
     {
       LANE_VARS;
-      lds_store_rows_kappa<1, 4>(s_x2t, FLD, x2op, c, h);   // stored [hid][tok], private to the wave
+      OpdT<1, 4> x2op;
+      cvt_chain_split(x2, x2op, x2lo);
+      lds_store_rows_kappa<1, 4>(s_x2t, FLD, x2op, c, h);   // stored [hid][tok], private to the wave; read back as rows by the W2 step
     }
     TTT_WAVE_SYNC();
 
     // ---- Z2^T partial = W2s^T X2^T (rows F, lane = tok), summed over the pair into [tok][F]
     {
       LANE_VARS;
-      OpdT<2, 2> w2h, w2l;
-      cvt_chain_split(W2s, w2h, w2l);
-      const OpdT<2, 2> x2B = lds_tr_kappa<2, 2>(s_x2t, FLD, lane);
-      AccT<2, 2> z2;
-      acc_zero(z2);
-      mma(z2, w2l, x2B);
-      mma(z2, w2h, x2B);
-      pair_sum_to_lds(s_Pp, z2, pr, c, h);
+      auto z2_block = [&](const f32x16& w2) {   // one F block of W2s^T X2^T: W2s in two terms, X2^T from the bounce tile
+        AccT<1, 2> z;
+        acc_zero(z);
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+          bf16x8 wh, wl, xb[2];
+          split8(w2, s, wh, wl);
+#pragma unroll
+          for (int cb = 0; cb < 2; cb++) xb[cb] = piece_tr<FLD>(s_x2t, cb, s, lane);
+#pragma unroll
+          for (int cb = 0; cb < 2; cb++) {
+            z.b[0][cb] = MFMA(wl, xb[cb], z.b[0][cb]);
+            z.b[0][cb] = MFMA(wh, xb[cb], z.b[0][cb]);
+          }
+        }
+        return z;
+      };
+      pair_sum_halves(s_Pp, [&]() { return z2_block(W2s.b[0][0]); }, [&]() { return z2_block(W2s.b[0][1]); }, pr, c, h);
     }
 
     // ---- LayerNorm-fused reconstruction-loss gradient: 8 tokens per wave, 8 lanes per token
     {
       LANE_VARS;
-      if constexpr (ROLE == 1) {   // next XK / XV / eta leave HBM now and land in the other buffers at the end of this stage
+      if constexpr (ROLE == 1) {
+        // The next mini-batch's XK / XV / eta leave HBM for the other LDS buffers now (last read a mini-batch ago,
+        // two barriers back) without passing through registers: wave v fetches rows 8v .. 8v+7 of both tiles,
+        // one pair of rows (256 contiguous bytes) per load, wave 0 also the 128 bytes of eta.
         if (mb + 1 < p.NC) {
-          st.k = g_ld16(gXK, 16 * tid, (mb + 1) * TILE_BYTES);
-          st.v = g_ld16(gXV, 16 * tid, (mb + 1) * TILE_BYTES);
-          st.eta = bf2f(g_ldh(gEta, 2 * (tid & (CS - 1)), (mb + 1) * (CS * 2)));
+          typedef const __attribute__((address_space(1))) unsigned* gword_t;
+          typedef __attribute__((address_space(3))) unsigned* lword_t;
+          unsigned char* const nk = smem + (alt ? SM_XK : SM_XQ);
+          unsigned char* const nv = smem + (alt ? SM_XV : SM_XQ + SM_TILE);
+          const gptr_t srck = gXK + static_cast<uint64_t>(uni((mb + 1) * TILE_BYTES + v * 1024)) + static_cast<uint64_t>(4u * lane);
+          const gptr_t srcv = gXV + static_cast<uint64_t>(uni((mb + 1) * TILE_BYTES + v * 1024)) + static_cast<uint64_t>(4u * lane);
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            __builtin_amdgcn_global_load_lds((gword_t)(srck + 256 * j), (lword_t)(nk + (4 * v + j) * (XPAIR * 2)), 4, 0, 0);
+            __builtin_amdgcn_global_load_lds((gword_t)(srcv + 256 * j), (lword_t)(nv + (4 * v + j) * (XPAIR * 2)), 4, 0, 0);
+          }
+          if (v == 0 && lane < 32)
+            __builtin_amdgcn_global_load_lds((gword_t)(gEta + static_cast<uint64_t>(uni((mb + 1) * (CS * 2))) + static_cast<uint64_t>(4u * lane)),
+                                             (lword_t)(smem + (alt ? SM_ETA : SM_B1)), 4, 0, 0);
         }
       }
       float z[8];
@@ -345,8 +436,8 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
 #pragma unroll
       for (int e = 0; e < 8; e++) { z[e] -= mu; var = __builtin_fmaf(z[e], z[e], var); }
       const float rstd = __builtin_amdgcn_rsqf(oct_sum(var) * (1.f / FD) + LN_EPS);
-      const bf16x8 kv = lds_get8h(s_xk + tok * FLD + f0);
-      const bf16x8 vv = lds_get8h(s_xv + tok * FLD + f0);
+      const bf16x8 kv = lds_get8h(s_xk + xrow(tok) + f0);
+      const bf16x8 vv = lds_get8h(s_xv + xrow(tok) + f0);
       float gam[8], bet[8];
 #pragma unroll
       for (int q = 0; q < 2; q++) {
@@ -368,33 +459,47 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
       }
       s1 = oct_sum(s1);
       s2 = oct_sum(s2);
-      const float scale = -s_eta[tok] * rstd * (1.f / FD);  // G2 = -eta * dl/dZ2
+      const float scale = -bf2f(s_eta[tok]) * rstd * (1.f / FD);  // G2 = -eta * dl/dZ2
       bf16x8 o, ol;
 #pragma unroll
       for (int e = 0; e < 8; e++) gx[e] = (FD * gx[e] - s1 - z[e] * s2) * scale;
       split8(gx, o, ol);
       lds_put16(s_g2 + tok * FLD + f0, __builtin_bit_cast(u32x4, o));
       lds_put16(s_g2l + tok * FLD + f0, __builtin_bit_cast(u32x4, ol));
-      if constexpr (ROLE == 1) {
-        if (mb + 1 < p.NC) {
-          const int off = ((tid >> 3) * FLD + (tid & 7) * 8) * 2;
-          lds_put16(smem + (alt ? SM_XK : SM_XQ) + off, st.k);
-          lds_put16(smem + (alt ? SM_XV : SM_XQ + SM_TILE) + off, st.v);
-          if (tid < CS) reinterpret_cast<float*>(smem + (alt ? SM_ETA : SM_B1))[tid] = st.eta;
-        }
-      }
     }
     __syncthreads();
 
     // ---- G1 = (G2 W2^T) * gelu'(Z1);  state += X^T G
     {
       LANE_VARS;
-      // g1 = G2 W2^T: G2 rows from LDS (lane = tok, contraction = F), W2t chained (lane = hid, contraction = F)
+      // g1 = G2 W2^T: G2 rows from LDS (lane = tok, contraction = F); W2 as (lane = hid, contraction = F): the two
+      // terms of W2s, written as rows [F][hid] into two wave-private tiles and read back transposed.  The tiles sit in
+      // this wave's own part of the pair-sum tile (the part it writes when it gives; dead from the barrier above
+      // until this wave's next pair sum).
       AccT<2, 1> g1;
       acc_zero(g1);
       {
         OpdT<1, 4> wh, wl;
-        cvt_chain_split(W2t, wh, wl);
+        {
+          constexpr int LDT = 2 * LDP, LDU = 2 * LDP;       // row stride (bf16 elements): a row of the pair-sum tile
+          bf16* const t_hi = reinterpret_cast<bf16*>(s_Pp) + 64 * (1 - pr);   // 64 of the row's elements are this wave's:
+          bf16* const t_lo = t_hi + 32;                                       // 32 for each term
+#pragma unroll
+          for (int fb = 0; fb < 2; fb++)
+#pragma unroll
+            for (int s = 0; s < 2; s++) {
+              bf16x8 ph, pl;
+              split8(W2s.b[0][fb], s, ph, pl);
+              store_piece_rows<LDT>(t_hi, fb, s, c, h, ph);
+              store_piece_rows<LDU>(t_lo, fb, s, c, h, pl);
+            }
+          TTT_WAVE_SYNC();
+#pragma unroll
+          for (int s = 0; s < 4; s++) {
+            wh.v[0][s] = piece_tr<LDT>(t_hi, 0, s, lane);
+            wl.v[0][s] = piece_tr<LDU>(t_lo, 0, s, lane);
+          }
+        }
 #pragma unroll
         for (int s = 0; s < 4; s++) {
           bf16x8 ah[2], al[2];
@@ -427,7 +532,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
         for (int s = 0; s < 4; s++) {
           bf16x8 xk[2];
 #pragma unroll
-          for (int fb = 0; fb < 2; fb++) xk[fb] = piece_tr<FLD>(s_xk, fb, s, lane);      // lane = F, contraction = tok
+          for (int fb = 0; fb < 2; fb++) xk[fb] = xpiece_tr(s_xk, fb, s, lane);      // lane = F, contraction = tok
 #pragma unroll
           for (int fb = 0; fb < 2; fb++) {
             W1s.b[fb][0] = MFMA(xk[fb], g1l.v[0][s], W1s.b[fb][0]);
@@ -435,7 +540,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
           }
         }
       }
-      // W2[shard,:] += X2^T G2 and its transpose: X2 chained (two terms), G2 through the transposing read
+      // W2[shard,:] += X2^T G2: X2 chained (two terms), G2 through the transposing read
       // (lane = F, contraction = tok; two terms); b2 += column sums of G2 (waves 0 and 1, rows 32v..32v+32)
       f32x16 b2acc;
       if (v < 2) {
@@ -454,15 +559,12 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
           gh[fb] = piece_tr<FLD>(s_g2, fb, s, lane);
           gl[fb] = piece_tr<FLD>(s_g2l, fb, s, lane);
         }
-        const bf16x8 xh = x2op.v[0][s], xl = x2lo.v[0][s];
+        const bf16x8 xh = piece_rows<FLD>(s_x2t, 0, s, c, h), xl = x2lo.v[0][s];
 #pragma unroll
         for (int fb = 0; fb < 2; fb++) {
           W2s.b[0][fb] = MFMA(xl, gh[fb], W2s.b[0][fb]);
           W2s.b[0][fb] = MFMA(xh, gl[fb], W2s.b[0][fb]);
           W2s.b[0][fb] = MFMA(xh, gh[fb], W2s.b[0][fb]);
-          W2t.b[fb][0] = MFMA(gh[fb], xl, W2t.b[fb][0]);
-          W2t.b[fb][0] = MFMA(gl[fb], xh, W2t.b[fb][0]);
-          W2t.b[fb][0] = MFMA(gh[fb], xh, W2t.b[fb][0]);
         }
         if (v < 2) {
           b2acc = MFMA(v == 0 ? gl[0] : gl[1], ones, b2acc);
@@ -488,6 +590,9 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
       // ---- hand the state after this mini-batch to the output branch: W1s and W2s exactly as the
       //      post-update forward would convert them, and the two bias vectors
       LANE_VARS;
+      // the next mini-batch's inputs, under way to LDS since the LayerNorm stage, have arrived before the barrier
+      // that opens the next mini-batch
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       const gptr_t gImg = gbuf(p.state_img + ((size_t)bh * 2 * FWD_RING_MAX + slot) * (FWD_IMG_BYTES / 2));
       const OpdT<1, 4> w1A = cvt_chain(W1s);
       const OpdT<2, 2> w2A = cvt_chain(W2s);
@@ -499,8 +604,6 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
         for (int s = 0; s < 2; s++) g_st_stream<bf16x8>(gImg, 16 * tid, (4 + 2 * fb + s) * 8192, w2A.v[fb][s]);
       if (h == 0) gB[hid0 + c] = b1L;
       if (at == ring - 1 || mb == p.NC - 1) publish(w_given, grp + 1);
-      // No barrier ends a mini-batch here: every LDS buffer written from now on was last read before a
-      // barrier that its writers have yet to pass (the pair sum's, or the one after the LayerNorm stage).
       continue;
     }
 
@@ -508,7 +611,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
     {
       LANE_VARS;
       const OpdT<1, 4> w1A = cvt_chain(W1s);
-      const OpdT<2, 4> xqB = lds_rows_kappa<2, 4>(s_xq, FLD, c, h);
+      const OpdT<2, 4> xqB = x_rows_kappa(s_xq, c, h);
       AccT<1, 2> z1b;
 #pragma unroll
       for (int g = 0; g < 4; g++) {
@@ -524,14 +627,21 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
 #pragma unroll
         for (int i = 0; i < 16; i++) z1b.b[0][cb][i] = gelu_f(z1b.b[0][cb][i]);
       const OpdT<2, 2> x2bB = cvt_chain(z1b);      // lane = tok, contraction = hid
-      const OpdT<2, 2> w2A = cvt_chain(W2s);
-      AccT<2, 2> z2;
-      acc_zero(z2);
-      mma(z2, w2A, x2bB);                          // rows F, lane = tok
       // The next mini-batch's inputs leave HBM now and are written to LDS at the end of this one.  (Fetched
       // before the weight step they would be spilled at once, each spill waiting for its load.)
       if (mb + 1 < p.NC) stage_load(st, gXQ, gXK, gXV, gEta, mb + 1, tid);
-      pair_sum_to_lds(s_Pp, z2, pr, c, h);
+      auto z2_block = [&](const f32x16& w2) {      // one F block of W2s^T X2b^T: rows F, lane = tok
+        AccT<1, 2> z;
+        acc_zero(z);
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+          const bf16x8 wa = pack8(w2, s);
+#pragma unroll
+          for (int cb = 0; cb < 2; cb++) z.b[0][cb] = MFMA(wa, x2bB.v[cb][s], z.b[0][cb]);
+        }
+        return z;
+      };
+      pair_sum_halves(s_Pp, [&]() { return z2_block(W2s.b[0][0]); }, [&]() { return z2_block(W2s.b[0][1]); }, pr, c, h);
     }
 
     // ---- output LayerNorm + residual, 8 tokens per wave; next mini-batch's inputs into LDS
@@ -616,7 +726,7 @@ TTT_DEV void fwd_output_branch(const FwdParams& p, unsigned char* smem, const in
       const u32x4 q = g_ld16(gXQ, 16 * tid, mb * TILE_BYTES);
       float bv = 0.f;
       if (tid < FWD_BIAS_FLOATS) bv = gB[tid];
-      lds_put16(smem + SM_XQ + (mb & 1) * SM_TILE + ((tid >> 3) * FLD + (tid & 7) * 8) * 2, q);
+      lds_put16(smem + SM_XQ + (mb & 1) * SM_TILE + (xrow(tid >> 3) + (tid & 7) * 8) * 2, q);
       if (tid < HID) s_b1[tid] = bv;
       else if (tid < FWD_BIAS_FLOATS) s_b2[(mb & 1) * FD + tid - HID] = bv;
     }
@@ -631,7 +741,7 @@ TTT_DEV void fwd_output_branch(const FwdParams& p, unsigned char* smem, const in
       for (int fb = 0; fb < 2; fb++)
 #pragma unroll
         for (int s = 0; s < 2; s++) w2A.v[fb][s] = g_ld_stream<bf16x8>(gImg, 16 * tid, (4 + 2 * fb + s) * 8192);
-      const OpdT<2, 4> xqB = lds_rows_kappa<2, 4>(s_xq, FLD, c, h);
+      const OpdT<2, 4> xqB = x_rows_kappa(s_xq, c, h);
       AccT<1, 2> z1b;
 #pragma unroll
       for (int g = 0; g < 4; g++) {
