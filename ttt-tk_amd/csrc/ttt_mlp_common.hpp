@@ -47,21 +47,32 @@ TTT_DEV bf16x8 pack8(const f32x16& x, int t) {
 // about 16 significant bits.  A matrix product whose operand is split this way is the sum of one MFMA
 // product per term (fp32 accumulate), which keeps the operand rounding of the products that carry the
 // recurrence's state from one mini-batch to the next near 2^-17 instead of 2^-9.
+// Two values at a time: one packed conversion for the high-order terms, a shift and a mask to read them back as
+// fp32, two subtractions, one packed conversion for the low-order terms (6 instructions per pair).
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+TTT_DEV void split2(float a, float b, bf16x2& hi, bf16x2& lo) {
+  const f32x2 ab = {a, b};
+  hi = __builtin_convertvector(ab, bf16x2);
+  const uint32_t hp = __builtin_bit_cast(uint32_t, hi);
+  const f32x2 r = {a - __builtin_bit_cast(float, hp << 16), b - __builtin_bit_cast(float, hp & 0xffff0000u)};
+  lo = __builtin_convertvector(r, bf16x2);
+}
 TTT_DEV void split8(const f32x16& x, int t, bf16x8& hi, bf16x8& lo) {
 #pragma unroll
-  for (int j = 0; j < 8; j++) {
-    const float v = x[8 * t + j];
-    const bf16 hv = (bf16)v;
-    hi[j] = hv;
-    lo[j] = (bf16)(v - (float)hv);
+  for (int j = 0; j < 8; j += 2) {
+    bf16x2 h2, l2;
+    split2(x[8 * t + j], x[8 * t + j + 1], h2, l2);
+    hi[j] = h2[0]; hi[j + 1] = h2[1];
+    lo[j] = l2[0]; lo[j + 1] = l2[1];
   }
 }
 TTT_DEV void split8(const float (&x)[8], bf16x8& hi, bf16x8& lo) {
 #pragma unroll
-  for (int j = 0; j < 8; j++) {
-    const bf16 hv = (bf16)x[j];
-    hi[j] = hv;
-    lo[j] = (bf16)(x[j] - (float)hv);
+  for (int j = 0; j < 8; j += 2) {
+    bf16x2 h2, l2;
+    split2(x[j], x[j + 1], h2, l2);
+    hi[j] = h2[0]; hi[j + 1] = h2[1];
+    lo[j] = l2[0]; lo[j + 1] = l2[1];
   }
 }
 
