@@ -51,6 +51,22 @@ TTT_DEV bf16x8 xpiece_tr(const bf16* tile, int blk, int s, int lane) {
   const bf16* q = tile + xrow(16 * s + 4 * h + (i >> 2)) + 32 * blk + 16 * (c >> 4) + 4 * (i & 3);
   return cat(lds_tr4(q), lds_tr4(q + 4 * XPAIR));   // 8 rows on = 4 pairs on
 }
+// One [64][64] bf16 tile (8 KiB at byte offset `off` of g) from HBM straight into an LDS tile of row pairs, without
+// passing through registers: wave v fetches rows 8v .. 8v+7, one pair of rows (256 contiguous bytes) per load.
+// Asynchronous: the data is in LDS once the wave's vmcnt has drained (and visible to other waves after a barrier).
+typedef const __attribute__((address_space(1))) unsigned* gword_t;
+typedef __attribute__((address_space(3))) unsigned* lword_t;
+TTT_DEV void tile_to_lds(gptr_t g, unsigned off, unsigned char* tile, int v, int lane) {
+  const gptr_t src = g + static_cast<uint64_t>(uni(off + v * 1024)) + static_cast<uint64_t>(4u * lane);
+#pragma unroll
+  for (int j = 0; j < 4; j++)
+    __builtin_amdgcn_global_load_lds((gword_t)(src + 256 * j), (lword_t)(tile + (4 * v + j) * (XPAIR * 2)), 4, 0, 0);
+}
+// The 64 bf16 step sizes of a mini-batch (128 bytes), by wave 0.
+TTT_DEV void eta_to_lds(gptr_t g, unsigned off, unsigned char* dst, int v, int lane) {
+  if (v == 0 && lane < 32)
+    __builtin_amdgcn_global_load_lds((gword_t)(g + static_cast<uint64_t>(uni(off)) + static_cast<uint64_t>(4u * lane)), (lword_t)dst, 4, 0, 0);
+}
 TTT_DEV OpdT<2, 4> x_rows_kappa(const bf16* tile, int c, int h) {
   OpdT<2, 4> o;
 #pragma unroll
@@ -298,7 +314,6 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
 
   for (int mb = 0; mb < p.NC; mb++) {
     LANE_VARS;
-    Staged st;   // the next mini-batch's inputs on their way from HBM to LDS (not carried around the loop)
     const bf16* s_xq = reinterpret_cast<const bf16*>(smem + SM_XQ + (mb & 1) * SM_TILE);
     // ROLE 1 has no use for XQ (nor for b1 in LDS): their space holds a second XK / XV / eta buffer, so that
     // the next mini-batch's inputs can be written while this one's are still being read.
@@ -400,21 +415,14 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
         // two barriers back) without passing through registers: wave v fetches rows 8v .. 8v+7 of both tiles,
         // one pair of rows (256 contiguous bytes) per load, wave 0 also the 128 bytes of eta.
         if (mb + 1 < p.NC) {
-          typedef const __attribute__((address_space(1))) unsigned* gword_t;
-          typedef __attribute__((address_space(3))) unsigned* lword_t;
-          unsigned char* const nk = smem + (alt ? SM_XK : SM_XQ);
-          unsigned char* const nv = smem + (alt ? SM_XV : SM_XQ + SM_TILE);
-          const gptr_t srck = gXK + static_cast<uint64_t>(uni((mb + 1) * TILE_BYTES + v * 1024)) + static_cast<uint64_t>(4u * lane);
-          const gptr_t srcv = gXV + static_cast<uint64_t>(uni((mb + 1) * TILE_BYTES + v * 1024)) + static_cast<uint64_t>(4u * lane);
-#pragma unroll
-          for (int j = 0; j < 4; j++) {
-            __builtin_amdgcn_global_load_lds((gword_t)(srck + 256 * j), (lword_t)(nk + (4 * v + j) * (XPAIR * 2)), 4, 0, 0);
-            __builtin_amdgcn_global_load_lds((gword_t)(srcv + 256 * j), (lword_t)(nv + (4 * v + j) * (XPAIR * 2)), 4, 0, 0);
-          }
-          if (v == 0 && lane < 32)
-            __builtin_amdgcn_global_load_lds((gword_t)(gEta + static_cast<uint64_t>(uni((mb + 1) * (CS * 2))) + static_cast<uint64_t>(4u * lane)),
-                                             (lword_t)(smem + (alt ? SM_ETA : SM_B1)), 4, 0, 0);
+          tile_to_lds(gXK, (mb + 1) * TILE_BYTES, smem + (alt ? SM_XK : SM_XQ), v, lane);
+          tile_to_lds(gXV, (mb + 1) * TILE_BYTES, smem + (alt ? SM_XV : SM_XQ + SM_TILE), v, lane);
+          eta_to_lds(gEta, (mb + 1) * (CS * 2), smem + (alt ? SM_ETA : SM_B1), v, lane);
         }
+      } else {
+        // One workgroup: XQ has two buffers, so the next XQ can leave HBM now; XK / XV / eta follow once their
+        // last readers are done (after the pair sum of the output branch).
+        if (mb + 1 < p.NC) tile_to_lds(gXQ, (mb + 1) * TILE_BYTES, smem + SM_XQ + ((mb + 1) & 1) * SM_TILE, v, lane);
       }
       float z[8];
       {
@@ -627,9 +635,6 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
 #pragma unroll
         for (int i = 0; i < 16; i++) z1b.b[0][cb][i] = gelu_f(z1b.b[0][cb][i]);
       const OpdT<2, 2> x2bB = cvt_chain(z1b);      // lane = tok, contraction = hid
-      // The next mini-batch's inputs leave HBM now and are written to LDS at the end of this one.  (Fetched
-      // before the weight step they would be spilled at once, each spill waiting for its load.)
-      if (mb + 1 < p.NC) stage_load(st, gXQ, gXK, gXV, gEta, mb + 1, tid);
       auto z2_block = [&](const f32x16& w2) {      // one F block of W2s^T X2b^T: rows F, lane = tok
         AccT<1, 2> z;
         acc_zero(z);
@@ -644,16 +649,18 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
       pair_sum_halves(s_Pp, [&]() { return z2_block(W2s.b[0][0]); }, [&]() { return z2_block(W2s.b[0][1]); }, pr, c, h);
     }
 
-    // ---- output LayerNorm + residual, 8 tokens per wave; next mini-batch's inputs into LDS
+    // ---- output LayerNorm + residual, 8 tokens per wave.  XK / XV / eta were last read before the pair sum
+    //      above: the next mini-batch's leave HBM for LDS now.
     {
       LANE_VARS;
+      if (mb + 1 < p.NC) {
+        tile_to_lds(gXK, (mb + 1) * TILE_BYTES, smem + SM_XK, v, lane);
+        tile_to_lds(gXV, (mb + 1) * TILE_BYTES, smem + SM_XV, v, lane);
+        eta_to_lds(gEta, (mb + 1) * (CS * 2), smem + SM_ETA, v, lane);
+      }
       output_layernorm(s_P, s_b2, s_gam, s_bet, s_xq, gOut, mb, tok, f0);
     }
-    // XK / XV were last read before the pair sum above; the XQ buffer written here is the other one.
-    {
-      LANE_VARS;
-      if (mb + 1 < p.NC) stage_store(st, smem, (mb + 1) & 1, tid);
-    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the next mini-batch's inputs have arrived in LDS
     __syncthreads();
   }
 }
