@@ -19,7 +19,8 @@
 // 8 tokens per wave) then add the four pair sums.  Every sum has a fixed order.
 //
 // State in registers:
-//   replay : W1s [F x hid], W2s [hid x F], W2t [F x hid] (fp32 accumulator tiles); b1, b2 in LDS
+//   replay : W1s [F x hid], W2s [hid x F] (fp32 accumulator tiles; where W2 is needed with F contracted, the bf16
+//            terms of W2s are transposed through a wave-private LDS tile); b1, b2 in LDS
 //   reverse: gW1s [F x hid], gW2s [hid x F] (running gradients) only; gb1, gb2 in LDS.  The weights
 //            enter the reverse walk as ready-made bf16 MFMA operands: after every mini-batch the replay
 //            stores the operand images of W1^T[shard] and W2[shard]^T, and the walk reads the image of
@@ -61,6 +62,7 @@ constexpr int SB_XK = SB_E2 + SB_TILE;
 constexpr int SB_GZ2 = SB_XK + SB_TILE;   // replay: G2 = -eta*dl/dZ2 ; reverse: raw dl/dZ2
 constexpr int SB_A = SB_GZ2 + SB_TILE;    // reverse: gZ2_bar, later dZ2
 static_assert(2 * SB_TILE >= CS * FD * 4, "g_y park does not fit");
+static_assert(32 * XPAIR * 2 <= SB_TILE, "a tile of row pairs fits a tile slot");
 constexpr int SB_P = SB_A + SB_TILE;      // 8 pair-sum regions (one per wave), fp32 [32][LDR]
 constexpr int SB_REGION = RGN * 4;        // 9216: also two wave-private bf16 tiles
 static_assert(32 * LDR <= RGN, "pair-sum rows do not fit their region");
@@ -239,6 +241,12 @@ TTT_DEV void ln_token_sum_add(float* s_acc, const float (&x)[8], int q8, int f0)
 
 // 16-byte chunk staging of one [64][64] bf16 tile from HBM into an LDS tile with row stride LDX
 // (rows are 8-byte aligned): thread tid moves chunk tid.
+// The same into a tile of row pairs (XQ, XK, XV: the layout LDS-direct loads deliver).
+TTT_DEV void lds_put16x(bf16* s_tile, int tid, u32x4 v) {
+  uint2* d = reinterpret_cast<uint2*>(s_tile + xrow(tid >> 3) + (tid & 7) * 8);
+  d[0] = make_uint2(v[0], v[1]);
+  d[1] = make_uint2(v[2], v[3]);
+}
 TTT_DEV void lds_put16(bf16* s_tile, int tid, u32x4 v) {
   uint2* d = reinterpret_cast<uint2*>(s_tile + (tid >> 3) * LDX + (tid & 7) * 8);
   d[0] = make_uint2(v[0], v[1]);
@@ -336,20 +344,20 @@ TTT_DEV void pair_sum(float* own, float* partner, const AccT<2, 2>& z, int c, in
 // Three [64][64] bf16 tiles + the eta vector of one mini-batch in flight from HBM (per thread).
 struct Staged3 {
   u32x4 a, b, c;
-  float eta;
+  bf16 eta;
 };
 // `mb` = mini-batch index inside this (batch, head); t16 = 16 * tid.
 TTT_DEV void stage3_load(Staged3& s, gptr_t ga, gptr_t gb, gptr_t gc, gptr_t geta, int mb, int tid, unsigned t16) {
   s.a = g_ld16(ga, t16, mb * TILE_BYTES);
   s.b = g_ld16(gb, t16, mb * TILE_BYTES);
   s.c = g_ld16(gc, t16, mb * TILE_BYTES);
-  s.eta = bf2f(g_ldh(geta, 2 * (tid & (CS - 1)), mb * (CS * 2)));   // in bounds for every thread; threads >= CS drop it
+  s.eta = g_ldh(geta, 2 * (tid & (CS - 1)), mb * (CS * 2));   // in bounds for every thread; threads >= CS drop it
 }
-TTT_DEV void stage3_store(const Staged3& s, bf16* sa, bf16* sb, bf16* sc, float* s_eta, int tid) {
-  lds_put16(sa, tid, s.a);
-  lds_put16(sb, tid, s.b);
-  lds_put16(sc, tid, s.c);
-  if (tid < CS) s_eta[tid] = s.eta;
+TTT_DEV void stage3_store(const Staged3& s, bf16* sa, bf16* sb, bf16* sc, bf16* s_eta, int tid) {
+  lds_put16x(sa, tid, s.a);
+  lds_put16x(sb, tid, s.b);
+  lds_put16x(sc, tid, s.c);
+  if (tid < CS) s_eta[tid] = s.eta;   // the replay keeps eta as bf16 in LDS
 }
 
 // Piece s of W2[shard] before mini-batch j of the group as an operand (lane = hid row, contraction =
@@ -397,6 +405,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
   float* s_gam = reinterpret_cast<float*>(smem + SB_GAM);
   float* s_bet = reinterpret_cast<float*>(smem + SB_BET);
   float* s_eta = reinterpret_cast<float*>(smem + SB_ETA);
+  bf16* s_etah = reinterpret_cast<bf16*>(smem + SB_ETA);     // the replay's view: eta as it sits in HBM
   float* s_deta = reinterpret_cast<float*>(smem + SB_DETA);
   float* s_red = reinterpret_cast<float*>(smem + SB_RED);
 
@@ -574,11 +583,10 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         acc_store_rows(gW2s, bPW2, 0, FD, hid0, 0, c, h);
         norm_swap(done & 1);   // the walk's sum out, the replay's sum of this parity in
       }
-      AccT<2, 1> W1s, W2t;
+      AccT<2, 1> W1s;
       AccT<1, 2> W2s;
       acc_load_rows(W1s, bCW1, ckW, HID, 0, hid0, c, h);
       acc_load_rows(W2s, bCW2, ckW, FD, hid0, 0, c, h);
-      acc_load_cols(W2t, bCW2, ckW, FD, hid0, 0, c, h);
       __syncthreads();  // previous group's readers of the bias vectors are done
       if (tid < HID) s_b1[tid] = p.b1_ck[slot * HID + tid];
       if (tid < FD) s_b2[tid] = p.b2_ck[slot * FD + tid];
@@ -586,11 +594,10 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
       {
         Staged3 st;
         stage3_load(st, bXQ, bXK, bXV, bETA, k * cgs, tid, t16);
-        stage3_store(st, s_xq, s_xk, s_e2, s_eta, tid);
+        stage3_store(st, s_xq, s_xk, s_e2, s_etah, tid);
       }
       for (int j = 0; j < n_mb; j++) {
         const int mb = k * cgs + j;
-        Staged3 st;   // the next mini-batch's inputs on their way from HBM to LDS (not carried around the loop)
         REFRESH_OFFSETS();
         LANE_VARS;
         __syncthreads();   // the staged inputs (and, for j = 0, the biases) are visible
@@ -609,7 +616,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
             bf16x8 wh, wl, xk[2];
             split8(W1s.b[s >> 1][0], s & 1, wh, wl);
 #pragma unroll
-            for (int i = 0; i < 2; i++) xk[i] = piece_rows<LDX>(s_xk, tb[i], s, c, h);
+            for (int i = 0; i < 2; i++) xk[i] = xpiece_rows(s_xk, tb[i], s, c, h);
 #pragma unroll
             for (int i = 0; i < 2; i++) {
               x2.b[0][i] = MFMA(wl, xk[i], x2.b[0][i]);
@@ -691,8 +698,8 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           float go[8], gx[8];
           {
             float kv[8], vv[8], bet[8];
-            ln_load(kv, s_xk + tok * LDX + f0);
-            ln_load(vv, s_e2 + tok * LDX + f0);
+            ln_load(kv, s_xk + xrow(tok) + f0);
+            ln_load(vv, s_e2 + xrow(tok) + f0);
             ln_load_f32(bet, s_bet + f0);
 #pragma unroll
             for (int e = 0; e < 8; e++) {
@@ -703,7 +710,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           ln_store_g<ROLE != 0>(bXHF, vln, j * TILE_BYTES, z);
           ln_store_g<ROLE != 0>(bGOF, vln, j * TILE_BYTES, go);
           const float s1 = oct_sum(sum8(gx)), s2 = oct_sum(dot8(gx, z));
-          const float sc = rstd * (1.f / FD), neg_eta = -s_eta[tok];
+          const float sc = rstd * (1.f / FD), neg_eta = -bf2f(s_etah[tok]);
 #pragma unroll
           for (int e = 0; e < 8; e++) gx[e] = (FD * gx[e] - s1 - z[e] * s2) * sc;   // dl/dZ2
           ln_store_g<ROLE != 0>(bGZ2, vln, j * TILE_BYTES, gx);
@@ -723,10 +730,29 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           LANE_VARS;
           AccT<1, 2> g1;
           acc_zero(g1);
+          // W2[shard, :] with F contracted (lane = hid): the two terms of W2s, written as rows [F][hid] into T1 / T2
+          // and read back transposed
+          bf16x8 w2h[4], w2l[4];
 #pragma unroll
-          for (int s = 0; s < 4; s++) {                      // W2t: lane = hid, contraction = F; G2: lane = tok; two terms each
-            bf16x8 wh, wl, gh[2], gl[2];
-            split8(W2t.b[s >> 1][0], s & 1, wh, wl);
+          for (int fb = 0; fb < 2; fb++)
+#pragma unroll
+            for (int s = 0; s < 2; s++) {
+              bf16x8 ph, pl;
+              split8(W2s.b[0][fb], s, ph, pl);
+              store_piece_rows<LDH>(T1, fb, s, c, h, ph);
+              store_piece_rows<LDH>(T2, fb, s, c, h, pl);
+            }
+          WAVE_SYNC();
+#pragma unroll
+          for (int s = 0; s < 4; s++) {
+            w2h[s] = piece_tr<LDH>(T1, 0, s, lane);
+            w2l[s] = piece_tr<LDH>(T2, 0, s, lane);
+          }
+          WAVE_SYNC();   // read before G1 takes the tiles' place below
+#pragma unroll
+          for (int s = 0; s < 4; s++) {                      // W2: lane = hid, contraction = F; G2: lane = tok; two terms each
+            const bf16x8 wh = w2h[s], wl = w2l[s];
+            bf16x8 gh[2], gl[2];
 #pragma unroll
             for (int i = 0; i < 2; i++) {
               gh[i] = piece_rows<LDX>(s_gz2, tb[i], s, c, h);
@@ -762,7 +788,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           for (int s = 0; s < 4; s++) {                        // W1[:, shard] += XK^T G1
             bf16x8 xk[2];
 #pragma unroll
-            for (int fb = 0; fb < 2; fb++) xk[fb] = piece_tr<LDX>(s_xk, fb, s, lane);            // XK^T: lane = F
+            for (int fb = 0; fb < 2; fb++) xk[fb] = xpiece_tr(s_xk, fb, s, lane);               // XK^T: lane = F
             const bf16x8 gh = piece_tr<LDH>(T1, 0, s, lane), gl = piece_tr<LDH>(T2, 0, s, lane);   // G1: lane = hid
 #pragma unroll
             for (int fb = 0; fb < 2; fb++) {
@@ -779,7 +805,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
             for (int t = 0; t < 2; t++) store_piece_rows<LDH>(T1, tb[i], t, c, h, x2lo[i][t]);
           WAVE_SYNC();
 #pragma unroll
-          for (int s = 0; s < 4; s++) {                        // W2[shard, :] += X2^T G2, and its transpose
+          for (int s = 0; s < 4; s++) {                        // W2[shard, :] += X2^T G2
             const bf16x8 xh = piece_tr<LDH>(T0, 0, s, lane), xl = piece_tr<LDH>(T1, 0, s, lane);   // X2^T: lane = hid
             bf16x8 gh[2], gl[2];
 #pragma unroll
@@ -792,9 +818,6 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
               W2s.b[0][fb] = MFMA(xl, gh[fb], W2s.b[0][fb]);
               W2s.b[0][fb] = MFMA(xh, gl[fb], W2s.b[0][fb]);
               W2s.b[0][fb] = MFMA(xh, gh[fb], W2s.b[0][fb]);
-              W2t.b[fb][0] = MFMA(gh[fb], xl, W2t.b[fb][0]);
-              W2t.b[fb][0] = MFMA(gl[fb], xh, W2t.b[fb][0]);
-              W2t.b[fb][0] = MFMA(gh[fb], xh, W2t.b[fb][0]);
             }
           }
           if (v < 2) {
@@ -803,14 +826,20 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           }
           WAVE_SYNC();   // this wave's readers of T1 / T2 are done
         }
-        // operand images of the state after this step, for the reverse walk
+        // operand images of the state after this step, for the reverse walk; the image of W2 (lane = hid,
+        // contraction = F) also serves the output branch below
+        bf16x8 w2a[4];
         {
           LANE_VARS;
           // bIMG2: W2, lane = hid, contraction = F;  bIMG1: W1^T, lane = F, contraction = hid
           store_state_rows<LDF>(T2, W1s, c, h);                                 // rows [hid][F]
-#pragma unroll
-          for (int s = 0; s < 4; s++) image_store<ROLE != 0>(bIMG2, j * IMG_BYTES, s, t16, piece_state(W2t, 0, s));
+          store_state_rows<LDH>(T1, W2s, c, h);                                 // rows [F][hid]
           WAVE_SYNC();
+#pragma unroll
+          for (int s = 0; s < 4; s++) {
+            w2a[s] = piece_tr<LDH>(T1, 0, s, lane);
+            image_store<ROLE != 0>(bIMG2, j * IMG_BYTES, s, t16, w2a[s]);
+          }
 #pragma unroll
           for (int fb = 0; fb < 2; fb++)
 #pragma unroll
@@ -823,7 +852,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           AccT<1, 2> z1b;
           acc_init_rows_lds(z1b, s_b1w, h);
           mma_jit<4>(z1b, [&](int, int s) { return piece_state(W1s, 0, s); },
-                     [&](int i, int s) { return piece_rows<LDX>(s_xq, tb[i], s, c, h); });
+                     [&](int i, int s) { return xpiece_rows(s_xq, tb[i], s, c, h); });
           bf16x8 x2bQ[2][2];
           WAVE_SYNC();   // the weight step's readers of T0 are done
 #pragma unroll
@@ -852,10 +881,15 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         bf16x8 dxq_old;
         {
           LANE_VARS;
-          // Every reader of this mini-batch's XQ / XK / XV tiles is past the barriers of the pair sum: the
-          // next ones are fetched now and land in LDS at the end of this stage, which covers their latency.
-          // (Fetched any earlier they would sit in registers across the pair sum, and be spilled.)
-          if (j + 1 < n_mb) stage3_load(st, bXQ, bXK, bXV, bETA, mb + 1, tid, t16);
+          // Every reader of this mini-batch's XQ / XK / XV / eta is past the barriers of the pair sum: the next
+          // mini-batch's leave HBM now - straight to LDS, no registers involved - and have the rest of this
+          // mini-batch to arrive.
+          if (j + 1 < n_mb) {
+            tile_to_lds(bXQ, (mb + 1) * TILE_BYTES, smem + SB_XQ, v, lane);
+            tile_to_lds(bXK, (mb + 1) * TILE_BYTES, smem + SB_XK, v, lane);
+            tile_to_lds(bXV, (mb + 1) * TILE_BYTES, smem + SB_E2, v, lane);
+            eta_to_lds(bETA, (mb + 1) * (CS * 2), smem + SB_ETA, v, lane);
+          }
           float z[8], gx[8], gam[8];
           {
             float b2v[8];
@@ -880,7 +914,6 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           for (int e = 0; e < 8; e++) gx[e] = (FD * gx[e] - s1 - z[e] * s2) * sc;
           ln_store(s_a + tok * LDX + f0, gx);            // gZ2_bar
           ln_store_g<ROLE != 0>(bGZB, vln, j * TILE_BYTES, gx);
-          if (j + 1 < n_mb) stage3_store(st, s_xq, s_xk, s_e2, s_eta, tid);
         }
         __syncthreads();
         {
@@ -894,7 +927,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
             LANE_VARS;
             AccT<1, 2> gz1b;   // (gZ2_bar W2^T) * gelu'(Z1_bar): rows hid, lane = tok
             acc_zero(gz1b);
-            mma_jit<4>(gz1b, [&](int, int s) { return piece_state(W2t, 0, s); },
+            mma_jit<4>(gz1b, [&](int, int s) { return w2a[s]; },
                        [&](int i, int s) { return piece_rows<LDX>(s_a, tb[i], s, c, h); });
 #pragma unroll
             for (int i = 0; i < 2; i++)
@@ -932,6 +965,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           for (int e = 0; e < 8; e++) dxq_old[e] = (bf16)((float)dxq_old[e] + (z[e] + gO[e]));
           g_st_stream<bf16x8>(bDXQ, vln, mb * TILE_BYTES, dxq_old);
         }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the next mini-batch's inputs are in LDS before the barrier at the loop's top
       }
       if constexpr (ROLE == 1) {
         if (done + n_replay >= p.K) {   // this workgroup's last group: hand its norm-gradient sums to the walk
@@ -987,8 +1021,8 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         const u32x4 gzb = ST ? g_ld_stream<u32x4>(bGZB, t16, so) : g_ld16(bGZB, t16, so);
         const float eta = bf2f(g_ldh(bETA, 2 * (tid & (CS - 1)), mb * (CS * 2)));
         __syncthreads();   // the previous mini-batch's readers of these tiles are done (the loads are under way)
-        lds_put16(s_xq, tid, xq);
-        lds_put16(s_xk, tid, xk);
+        lds_put16x(s_xq, tid, xq);
+        lds_put16x(s_xk, tid, xk);
         lds_put16(s_gz2, tid, gz);
         lds_put16(s_a, tid, gzb);
         if (tid < CS) s_eta[tid] = eta;
@@ -1025,7 +1059,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         mma_jit<4>(gW2s, [&](int, int s) { return x2b[s]; },                                   // X2_bar^T: lane = hid
                    [&](int fb, int s) { return piece_tr<LDX>(s_a, fb, s, lane); });            // gZ2_bar: lane = F
         if (v < 2) lds_rowsum_add_jit(s_gb2 + 32 * v, [&](int s) { return piece_tr<LDX>(s_a, v, s, lane); }, ones, c, h);
-        mma_jit<4>(gW1s, [&](int fb, int s) { return piece_tr<LDX>(s_xq, fb, s, lane); },      // XQ^T: lane = F
+        mma_jit<4>(gW1s, [&](int fb, int s) { return xpiece_tr(s_xq, fb, s, lane); },         // XQ^T: lane = F
                    [&](int, int s) { return g1b[s]; });                                        // gZ1_bar: lane = hid
         lds_rowsum_add_jit(s_gb1w, [&](int s) { return g1b[s]; }, ones, c, h);
       }
@@ -1057,7 +1091,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           mma_jit<4>(R, [&](int, int s) { return piece_rows<LDF>(T1, 0, s, c, h); },
                      [&](int, int s) { return piece_rows<LDX>(s_gz2, tb[i], s, c, h); });
           mma_jit<4>(S, [&](int, int s) { return piece_rows<LDF>(T2, 0, s, c, h); },
-                     [&](int, int s) { return piece_rows<LDX>(s_xk, tb[i], s, c, h); });
+                     [&](int, int s) { return xpiece_rows(s_xk, tb[i], s, c, h); });
           bf16x8 x2c[2], uc[2];
           // gelu(Z1), gelu'(Z1), gelu''(Z1), each rounded to bf16: computed here from the image of Z1, or
           // fetched as three images that a replaying workgroup computed the same way
@@ -1297,7 +1331,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         mma_jit<4>(gW2s, [&](int, int s) { return piece_tr<LDH>(T0, 0, s, lane); },            // X2^T: lane = hid
                    [&](int fb, int s) { return piece_tr<LDX>(s_a, fb, s, lane); });            // dZ2: lane = F
         if (v < 2) lds_rowsum_add_jit(s_gb2 + 32 * v, [&](int s) { return piece_tr<LDX>(s_a, v, s, lane); }, ones, c, h);
-        mma_jit<4>(gW1s, [&](int fb, int s) { return piece_tr<LDX>(s_xk, fb, s, lane); },      // XK^T: lane = F
+        mma_jit<4>(gW1s, [&](int fb, int s) { return xpiece_tr(s_xk, fb, s, lane); },         // XK^T: lane = F
                    [&](int, int s) { return piece_tr<LDH>(T1, 0, s, lane); });                 // dZ1: lane = hid
         lds_rowsum_add_jit(s_gb1w, [&](int s) { return piece_tr<LDH>(T1, 0, s, lane); }, ones, c, h);
         WAVE_SYNC();   // this wave's readers of T1 / T2 are done
@@ -1467,11 +1501,11 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
           dz[a][t] = image_load<true>(gDZ, ho, 2 * tb[a] + t, t16);
           w1b[a][t] = w1_before(gIMG1, gCW1, ckW, j, a, t, hid0, c, h, t16);
         }
-      lds_put16(s_xq, tid, xq);
-      lds_put16(s_xk, tid, xk);
+      lds_put16x(s_xq, tid, xq);
+      lds_put16x(s_xk, tid, xk);
       lds_put16(s_gz2, tid, gz);
       __syncthreads();
-      mma_jit<4>(gW1s, [&](int fb, int s) { return piece_tr<LDX>(s_xq, fb, s, lane); },      // + XQ^T gZ1_bar
+      mma_jit<4>(gW1s, [&](int fb, int s) { return xpiece_tr(s_xq, fb, s, lane); },         // + XQ^T gZ1_bar
                  [&](int, int s) { return g1b[s]; });
       store_state_rows<LDF>(T2, gW1s, c, h);                                                  // gW1 rows [hid][F]
 #pragma unroll
@@ -1505,7 +1539,7 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
         for (int t = 0; t < 2; t++) store_piece_rows<LDH>(T1, tb[i], t, c, h, dz[i][t]);     // dZ1 rows [tok][hid]
       WAVE_SYNC();
       mma_jit<2>(dk, [&](int rb, int s) { return w1b[rb][s]; }, [&](int i, int s) { return dz[i][s]; });
-      mma_jit<4>(gW1s, [&](int fb, int s) { return piece_tr<LDX>(s_xk, fb, s, lane); },      // + XK^T dZ1
+      mma_jit<4>(gW1s, [&](int fb, int s) { return xpiece_tr(s_xk, fb, s, lane); },         // + XK^T dZ1
                  [&](int, int s) { return piece_tr<LDH>(T1, 0, s, lane); });
       WAVE_SYNC();   // this wave's readers of T1 / T2 are done
       pair_sum(s_own, s_partner, dk, c, h);

@@ -36,37 +36,6 @@ constexpr int FW_NS = HID / FW_NWAVE;                  // hidden columns per wav
 // rows); rows are 8-byte aligned, so 16-byte accesses are made as two 8-byte ones.
 constexpr int FLD = 68;
 #define MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16((a), (b), (c), 0, 0, 0)
-// The input tiles (XQ, XK, XV) sit in LDS as pairs of rows: two rows of 128 bytes back to back, pairs 264 bytes
-// apart.  A pair is what one wave-wide 4-byte LDS-direct load (global_load_lds_dword: lane l writes base + 4 l)
-// delivers, so a tile can travel from HBM to LDS without passing through registers, and the 8 bytes between
-// pairs put the 32 row-wise 8-byte reads of an operand piece on 64 distinct banks.
-constexpr int XPAIR = 132;   // elements from one pair of rows to the next
-TTT_DEV int xrow(int r) { return (r >> 1) * XPAIR + (r & 1) * 64; }
-TTT_DEV bf16x8 xpiece_rows(const bf16* tile, int blk, int s, int c, int h) {
-  const bf16* q = tile + xrow(32 * blk + c) + 16 * s + 4 * h;
-  return cat(*reinterpret_cast<const bf16x4*>(q), *reinterpret_cast<const bf16x4*>(q + 8));
-}
-TTT_DEV bf16x8 xpiece_tr(const bf16* tile, int blk, int s, int lane) {
-  const int h = lane >> 5, c = lane & 31, i = lane & 15;
-  const bf16* q = tile + xrow(16 * s + 4 * h + (i >> 2)) + 32 * blk + 16 * (c >> 4) + 4 * (i & 3);
-  return cat(lds_tr4(q), lds_tr4(q + 4 * XPAIR));   // 8 rows on = 4 pairs on
-}
-// One [64][64] bf16 tile (8 KiB at byte offset `off` of g) from HBM straight into an LDS tile of row pairs, without
-// passing through registers: wave v fetches rows 8v .. 8v+7, one pair of rows (256 contiguous bytes) per load.
-// Asynchronous: the data is in LDS once the wave's vmcnt has drained (and visible to other waves after a barrier).
-typedef const __attribute__((address_space(1))) unsigned* gword_t;
-typedef __attribute__((address_space(3))) unsigned* lword_t;
-TTT_DEV void tile_to_lds(gptr_t g, unsigned off, unsigned char* tile, int v, int lane) {
-  const gptr_t src = g + static_cast<uint64_t>(uni(off + v * 1024)) + static_cast<uint64_t>(4u * lane);
-#pragma unroll
-  for (int j = 0; j < 4; j++)
-    __builtin_amdgcn_global_load_lds((gword_t)(src + 256 * j), (lword_t)(tile + (4 * v + j) * (XPAIR * 2)), 4, 0, 0);
-}
-// The 64 bf16 step sizes of a mini-batch (128 bytes), by wave 0.
-TTT_DEV void eta_to_lds(gptr_t g, unsigned off, unsigned char* dst, int v, int lane) {
-  if (v == 0 && lane < 32)
-    __builtin_amdgcn_global_load_lds((gword_t)(g + static_cast<uint64_t>(uni(off)) + static_cast<uint64_t>(4u * lane)), (lword_t)dst, 4, 0, 0);
-}
 TTT_DEV OpdT<2, 4> x_rows_kappa(const bf16* tile, int c, int h) {
   OpdT<2, 4> o;
 #pragma unroll
