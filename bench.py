@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the TTT-MLP forward + remat-backward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c5|c3] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c5|c3|c2] [--no-cpu-baseline]
 
 A "step" is one forward + one remat backward over one batch of synthetic input that is already
 resident in HBM (zero-filling the four accumulating gradient outputs is part of the step, as the
@@ -27,13 +27,25 @@ G_FLOP = 2 * 64 * 64 * 256                 # one 64x64x256 contraction
 FWD_G, BWD_G = 7, 21                        # contractions per mini-batch per (batch, head): forward; replay 7 + reverse 14
 PEAK_BF16_TFLOPS = 2516.6                   # MI355X dense bf16 MFMA: 256 CU x 4096 FLOP/clk x 2.4 GHz
 WORKLOADS = {
-    # name: (B, NH, NC, checkpoint_group_size, eta logit std, description)
+    # name: (B, NH, NC, checkpoint_group_size, eta logit std, description); c2 is the forward alone
+    "c2": (1, 48, 256, 16, 1.0, "forward only B=1 NH=48 16,384 tokens cgs=16"),
     "c3": (1, 48, 256, 16, 1.0, "fwd+bwd B=1 NH=48 16,384 tokens cgs=16"),
     "c4": (1, 48, 4096, 64, 1.0, "fwd+bwd B=1 NH=48 262,144 tokens cgs=64 (the configuration the metric is quoted on)"),
     "c5": (8, 48, 512, 32, 2.0, "fwd+bwd B=8 NH=48 32,768 tokens/sequence cgs=32 (fill-the-chip)"),
 }
-# HBM bytes per backward launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/), or None.
-MEASURED_TRAFFIC_BYTES = {"c4": 2.15e11}    # FETCH_SIZE 56,436,600 KiB x 2.0 + WRITE_SIZE 97,333,000 KiB x 1.0
+
+
+def measured_traffic(workload, which):
+    """HBM bytes per launch of the forward (`which` = "fwd") or backward ("bwd") kernels of a workload, from the
+    rocprofv3 counter summary that `ttt-tk_amd/profile_counters.py` leaves under profiles/ (FETCH_SIZE + WRITE_SIZE,
+    each scaled by what the same counter reads for a copy of known size); None if that workload was not profiled."""
+    path = os.path.join(ROOT, "profiles", f"ttt_mlp_{workload}_counters.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        kernels = json.load(f)["kernels"]
+    vals = [k["hbm_bytes"] for name, k in kernels.items() if f"ttt_mlp_{which}" in name and "hbm_bytes" in k]
+    return sum(vals) if vals else None
 
 
 def make_device_inputs(B, NH, NC, eta_std, dev):
@@ -60,7 +72,7 @@ def make_device_inputs(B, NH, NC, eta_std, dev):
     return t
 
 
-def cpu_baseline(NH, cgs, nc_sample):
+def cpu_baseline(NH, cgs, nc_sample, backward=True):
     """fp32 oracle forward + backward on the host cores over the first nc_sample mini-batches."""
     import torch
     from oracle import ttt_mlp_oracle as orc
@@ -74,12 +86,13 @@ def cpu_baseline(NH, cgs, nc_sample):
     t0 = time.perf_counter()
     with torch.no_grad():
         _, ck, _ = orc.ttt_forward(*[d[k] for k in keys], cgs)
-        orc.ttt_backward(d["XQ"], d["XK"], d["XV"], d["last_eta"], d["ttt_norm_weight"], d["ttt_norm_bias"], ck,
-                         orc.State(d["grad_L_W1_last"], d["grad_L_b1_last"], d["grad_L_W2_last"], d["grad_L_b2_last"]),
-                         d["grad_L_XQW_mini_batch"], cgs)
+        if backward:
+            orc.ttt_backward(d["XQ"], d["XK"], d["XV"], d["last_eta"], d["ttt_norm_weight"], d["ttt_norm_bias"], ck,
+                             orc.State(d["grad_L_W1_last"], d["grad_L_b1_last"], d["grad_L_W2_last"], d["grad_L_b2_last"]),
+                             d["grad_L_XQW_mini_batch"], cgs)
     dt = time.perf_counter() - t0
     return {"value": nc_sample * 64 / dt, "unit": "tokens/s", "cores": threads, "kind": "port",
-            "sample": f"fp32 PyTorch oracle, forward + backward, B=1 NH={NH} first {nc_sample} mini-batches "
+            "sample": f"fp32 PyTorch oracle, {'forward + backward' if backward else 'forward'}, B=1 NH={NH} first {nc_sample} mini-batches "
                       f"({nc_sample * 64} tokens) cgs={cgs}, {dt:.1f} s"}
 
 
@@ -112,21 +125,24 @@ def main():
     B, NH, NC, cgs, eta_std, desc = WORKLOADS[a.workload]
     t = make_device_inputs(B, NH, NC, eta_std, dev)
     t.update(host.alloc_forward_buffers(B, NH, NC, cgs, dev))
-    t.update(host.alloc_backward_buffers(B, NH, NC, cgs, dev))
+    backward = a.workload != "c2"
+    if backward:
+        t.update(host.alloc_backward_buffers(B, NH, NC, cgs, dev))
     host.set_synchronize(False)           # time with events; the operator's default host sync is not part of the kernel
     import test_time_training as ext
     ext.set_overlap(not a.no_overlap)
     ext.set_accumulate(not a.overwrite)
 
     def step(ev=None):
-        if not a.overwrite:
+        if backward and not a.overwrite:
             host.zero_accumulating_grads(t)    # the operator adds to four of its outputs, as upstream does
         if ev:
             ev[0].record()
         host.forward(t, cgs)
         if ev:
             ev[1].record()
-        host.backward(t, cgs)
+        if backward:
+            host.backward(t, cgs)
         if ev:
             ev[2].record()
 
@@ -147,7 +163,8 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    assert bool(torch.isfinite(t["grad_L_W1_init"]).all()) and bool(torch.isfinite(t["Out"].float()).all())
+    assert bool(torch.isfinite(t["Out"].float()).all())
+    assert not backward or bool(torch.isfinite(t["grad_L_W1_init"]).all())
 
     fwd_ms = sum(e[0].elapsed_time(e[1]) for e in events) / a.steps
     bwd_ms = sum(e[1].elapsed_time(e[2]) for e in events) / a.steps
@@ -155,12 +172,13 @@ def main():
     tokens = B * NC * 64
     value = tokens / (ms_per_step * 1e-3)
     mb_steps = B * NH * NC
-    bwd_tflops = BWD_G * G_FLOP * mb_steps / (bwd_ms * 1e-3) / 1e12
+    bwd_tflops = BWD_G * G_FLOP * mb_steps / (bwd_ms * 1e-3) / 1e12 if backward else 0.0
     fwd_tflops = FWD_G * G_FLOP * mb_steps / (fwd_ms * 1e-3) / 1e12
-    all_tflops = (FWD_G + BWD_G) * G_FLOP * mb_steps / (ms_per_step * 1e-3) / 1e12
+    all_tflops = (FWD_G + (BWD_G if backward else 0)) * G_FLOP * mb_steps / (ms_per_step * 1e-3) / 1e12
     # one kernel per combination of roles: ttt_mlp_bwd_split_kernel<replaying workgroups, grad_L_XK workgroup>
     bwd_kernel = "ttt_mlp_bwd_kernel"
-    if ext.last_backward_mode() == 1:
+    fwd_kernel = "ttt_mlp_fwd_kernel" if ext.last_forward_mode() == 0 else f"ttt_mlp_fwd_split_kernel<{32 if NC >= 512 else 8}>"
+    if backward and ext.last_backward_mode() == 1:
         import ctypes
         lib = ctypes.CDLL(os.path.join(os.path.dirname(os.path.abspath(host.__file__)), "libttt_mlp.so"))
         one, rest, per = ctypes.c_longlong(), ctypes.c_longlong(), ctypes.c_int()
@@ -170,7 +188,8 @@ def main():
         if one.value:
             bwd_kernel = "ttt_mlp_bwd_kernel + " + bwd_kernel
     out = {
-        "metric": "TTT-MLP fwd+bwd tokens/sec on 1 MI355X (B=1,NH=48,256K tok); % bf16 MFMA peak",
+        "metric": "TTT-MLP fwd+bwd tokens/sec on 1 MI355X (B=1,NH=48,256K tok); % bf16 MFMA peak" if backward
+                  else "TTT-MLP forward tokens/sec on 1 MI355X; % bf16 MFMA peak",
         "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
@@ -178,13 +197,16 @@ def main():
                    "checkpoint_group_size": cgs},
         "fwd_ms": fwd_ms, "bwd_ms": bwd_ms, "fwd_tflops": fwd_tflops, "fwd_bwd_tflops": all_tflops,
         "pct_of_bf16_mfma_peak": 100.0 * all_tflops / PEAK_BF16_TFLOPS,
-        "roofline": {"bound": "mfma", "kernel": bwd_kernel, "achieved": bwd_tflops, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": bwd_tflops / PEAK_BF16_TFLOPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload),
-                     "flop_per_launch": BWD_G * G_FLOP * mb_steps, "avg_launch_ms": bwd_ms},
+        # the dominant kernel: the backward (the forward where there is no backward)
+        "roofline": {"bound": "mfma", "kernel": bwd_kernel if backward else fwd_kernel,
+                     "achieved": bwd_tflops if backward else fwd_tflops, "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": (bwd_tflops if backward else fwd_tflops) / PEAK_BF16_TFLOPS,
+                     "traffic": measured_traffic(a.workload, "bwd" if backward else "fwd"),
+                     "flop_per_launch": (BWD_G if backward else FWD_G) * G_FLOP * mb_steps,
+                     "avg_launch_ms": bwd_ms if backward else fwd_ms},
     }
     if not a.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(NH, cgs, min(a.cpu_sample_mb, NC))
+        out["cpu_baseline"] = cpu_baseline(NH, cgs, min(a.cpu_sample_mb, NC), backward)
     print(json.dumps(out), flush=True)
 
 

@@ -1,0 +1,194 @@
+#!/usr/bin/env python3
+"""rocprofv3 counter harness for the TTT-MLP kernels: one JSON per workload under profiles/.
+
+    python ttt-tk_amd/profile_counters.py --workload c4 [--workload c5 ...] [--raw gpurun_out/counters]
+
+For each workload it runs `python3 bench.py --workload W ...` under rocprofv3 five times, each pass a run of its own
+(counters are never combined with tracing options other than the kernel trace):
+  1. --kernel-trace --stats                      -> calls and average duration per kernel
+  2. --pmc FETCH_SIZE    (+ a 1 GiB copy kernel) -> KiB read from HBM per dispatch, scaled by what the same
+  3. --pmc WRITE_SIZE    (+ a 1 GiB copy kernel)    counter reads for the copy of known size
+  4. --pmc SQ_INSTS_VALU SQ_INSTS_MFMA SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CYCLES SQ_WAVE_CYCLES
+           SQ_LDS_BANK_CONFLICT SQ_ACTIVE_INST_LDS SQ_WAIT_ANY
+  5. --pmc SQ_INSTS_LDS SQ_INSTS_VMEM_RD SQ_INSTS_VMEM_WR SQ_INSTS_SALU SQ_ACTIVE_INST_VALU SQ_WAIT_INST_ANY
+           SQ_INSTS_VALU_TRANS_F32 SQ_WAIT_INST_LDS
+and writes profiles/ttt_mlp_<W>_counters.json with, per TTT-MLP kernel: average duration, HBM bytes read / written
+per launch and the GB/s they amount to, MFMA-pipe busy %, vector-ALU busy %, the share of LDS-pipeline cycles lost
+to bank conflicts, the share of wave cycles spent waiting, instruction counts, waves per SIMD and LDS bytes per
+workgroup.  `bench.py` takes `roofline.traffic` from that file.
+
+Derived figures (SQ_* cycle counters tick once per 4 clocks; a 32x32x16 MFMA occupies the matrix pipe of its SIMD
+for 32 clocks; every workgroup has 8 waves on the 4 SIMDs of one CU, which its LDS use fills):
+  simd_clocks        = SQ_WAVE_CYCLES * 4 / waves_per_simd
+  mfma_busy_pct      = 100 * SQ_INSTS_MFMA * 32 / simd_clocks
+  valu_busy_pct      = 100 * SQ_ACTIVE_INST_VALU * 4 / simd_clocks
+  lds_conflict_share = SQ_LDS_BANK_CONFLICT / (SQ_ACTIVE_INST_LDS * 4)
+  wait_share         = SQ_WAIT_ANY / SQ_WAVE_CYCLES
+"""
+from __future__ import annotations
+
+import argparse
+import collections
+import csv
+import ctypes
+import glob
+import json
+import os
+import signal
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+GIB_KIB = 1 << 20   # the calibration copy reads 1 GiB and writes 1 GiB
+
+PASSES = (
+    ("trace", ["--kernel-trace", "--stats"], ["--steps", "2", "--warmup", "1"]),
+    ("fetch", ["--pmc", "FETCH_SIZE"], ["--steps", "1", "--warmup", "0", "--calibrate-copy"]),
+    ("write", ["--pmc", "WRITE_SIZE"], ["--steps", "1", "--warmup", "0", "--calibrate-copy"]),
+    ("sq1", ["--pmc", "SQ_INSTS_VALU", "SQ_INSTS_MFMA", "SQ_VALU_MFMA_BUSY_CYCLES", "SQ_BUSY_CYCLES", "SQ_WAVE_CYCLES",
+             "SQ_LDS_BANK_CONFLICT", "SQ_ACTIVE_INST_LDS", "SQ_WAIT_ANY"], ["--steps", "1", "--warmup", "0"]),
+    ("sq2", ["--pmc", "SQ_INSTS_LDS", "SQ_INSTS_VMEM_RD", "SQ_INSTS_VMEM_WR", "SQ_INSTS_SALU", "SQ_ACTIVE_INST_VALU",
+             "SQ_WAIT_INST_ANY", "SQ_INSTS_VALU_TRANS_F32", "SQ_WAIT_INST_LDS"], ["--steps", "1", "--warmup", "0"]),
+)
+
+
+def run_pass(workload: str, tag: str, prof_args, bench_args, raw_dir: str, limit_s: int) -> str:
+    out_dir = os.path.join(raw_dir, f"{workload}_{tag}")
+    os.makedirs(out_dir, exist_ok=True)
+    cmd = ["rocprofv3", *prof_args, "--output-format", "csv", "-d", out_dir, "-o", workload, "--",
+           "python3", os.path.join(ROOT, "bench.py"), "--workload", workload, "--no-cpu-baseline", *bench_args]
+    env = dict(os.environ, TMPDIR="/tmp")
+    print("+", " ".join(cmd), flush=True)
+    with open(os.path.join(out_dir, "run.log"), "w") as log:
+        proc = subprocess.Popen(cmd, cwd="/tmp", env=env, stdout=log, stderr=subprocess.STDOUT, start_new_session=True)
+        try:
+            rc = proc.wait(timeout=limit_s)
+        except subprocess.TimeoutExpired:
+            os.killpg(proc.pid, signal.SIGKILL)      # the group this call started, nothing else
+            proc.wait()
+            raise RuntimeError(f"rocprofv3 pass {tag} of {workload} exceeded {limit_s} s; see {out_dir}/run.log")
+    if rc != 0:
+        raise RuntimeError(f"rocprofv3 pass {tag} of {workload} failed with exit code {rc}; see {out_dir}/run.log")
+    return out_dir
+
+
+def find_csv(out_dir: str, suffix: str) -> str:
+    hits = glob.glob(os.path.join(out_dir, "**", f"*{suffix}"), recursive=True)
+    if not hits:
+        raise RuntimeError(f"no *{suffix} under {out_dir}")
+    return hits[0]
+
+
+def short_name(kernel_name: str) -> str:
+    """ttt::ttt_mlp_bwd_split_kernel<2, true>(ttt::BwdParams) -> ttt_mlp_bwd_split_kernel<2, true>"""
+    n = kernel_name.split("(")[0]
+    return n.split("::")[-1].replace("void ", "").strip()
+
+
+def is_ours(name: str) -> bool:
+    return "ttt_mlp_fwd" in name or "ttt_mlp_bwd" in name or "ttt_mlp_export" in name
+
+
+def is_copy(name: str) -> bool:
+    return "copy" in name.lower() and "ttt_mlp" not in name
+
+
+def kernel_stats(out_dir: str):
+    rows = {}
+    for r in csv.DictReader(open(find_csv(out_dir, "kernel_stats.csv"))):
+        rows[r["Name"]] = dict(calls=int(r["Calls"]), avg_ns=float(r["AverageNs"]), total_ns=float(r["TotalDurationNs"]),
+                               pct=float(r["Percentage"]))
+    return rows
+
+
+def counter_sums(out_dir: str):
+    """{kernel: {counter: [value per dispatch]}} - the per-dimension rows of one dispatch are added up."""
+    per_dispatch = collections.defaultdict(float)
+    for r in csv.DictReader(open(find_csv(out_dir, "counter_collection.csv"))):
+        per_dispatch[(r["Kernel_Name"], r["Dispatch_Id"], r["Counter_Name"])] += float(r["Counter_Value"])
+    out = collections.defaultdict(lambda: collections.defaultdict(list))
+    for (k, _, c), v in per_dispatch.items():
+        out[k][c].append(v)
+    return out
+
+
+def kernel_geometry():
+    lib = ctypes.CDLL(os.path.join(HERE, "libttt_mlp.so"))
+    geo = {}
+    for which, key in ((0, "fwd"), (1, "bwd")):
+        lds, thr = ctypes.c_int(), ctypes.c_int()
+        lib.ttt_mlp_kernel_info(which, ctypes.byref(lds), ctypes.byref(thr))
+        geo[key] = dict(lds_bytes_per_workgroup=lds.value, threads_per_workgroup=thr.value,
+                        waves_per_simd=thr.value // 64 // 4)
+    return geo
+
+
+def profile(workload: str, raw_dir: str, limit_s: int):
+    dirs = {tag: run_pass(workload, tag, pa, ba, raw_dir, limit_s) for tag, pa, ba in PASSES}
+    stats = kernel_stats(dirs["trace"])
+    fetch, write = counter_sums(dirs["fetch"]), counter_sums(dirs["write"])
+    sq = counter_sums(dirs["sq1"])
+    for k, v in counter_sums(dirs["sq2"]).items():
+        sq[k].update(v)
+    # calibration: what FETCH_SIZE / WRITE_SIZE read for a copy of 1 GiB
+    cal = {}
+    for label, table, counter in (("fetch", fetch, "FETCH_SIZE"), ("write", write, "WRITE_SIZE")):
+        vals = [max(v[counter]) for k, v in table.items() if is_copy(k) and counter in v]
+        if not vals:
+            raise RuntimeError(f"calibration copy kernel not found in the {label} pass")
+        cal[label] = dict(copy_kernel_kib=max(vals), factor=GIB_KIB / max(vals))
+    geo = kernel_geometry()
+    kernels = {}
+    for name, st in stats.items():
+        if not is_ours(name) or "zero_words" in name:
+            continue
+        key = short_name(name)
+        g = geo["fwd" if "fwd" in key else "bwd"]
+        e = dict(calls=st["calls"], avg_ns=st["avg_ns"], **g)
+        rd = [v["FETCH_SIZE"] for k, v in fetch.items() if short_name(k) == key and "FETCH_SIZE" in v]
+        wr = [v["WRITE_SIZE"] for k, v in write.items() if short_name(k) == key and "WRITE_SIZE" in v]
+        if rd and wr:
+            e["hbm_read_bytes"] = sum(rd[0]) / len(rd[0]) * 1024 * cal["fetch"]["factor"]
+            e["hbm_write_bytes"] = sum(wr[0]) / len(wr[0]) * 1024 * cal["write"]["factor"]
+            e["hbm_bytes"] = e["hbm_read_bytes"] + e["hbm_write_bytes"]
+            e["hbm_gbs"] = e["hbm_bytes"] / e["avg_ns"]
+        c = {}
+        for k, v in sq.items():
+            if short_name(k) == key:
+                c = {cn: sum(vals) / len(vals) for cn, vals in v.items()}
+        if c:
+            e["counters"] = c
+            simd_clocks = c["SQ_WAVE_CYCLES"] * 4 / g["waves_per_simd"]
+            e["mfma_busy_pct"] = 100 * c["SQ_INSTS_MFMA"] * 32 / simd_clocks
+            e["valu_busy_pct"] = 100 * c["SQ_ACTIVE_INST_VALU"] * 4 / simd_clocks
+            e["lds_conflict_share"] = c["SQ_LDS_BANK_CONFLICT"] / max(c["SQ_ACTIVE_INST_LDS"] * 4, 1)
+            e["wait_share"] = c["SQ_WAIT_ANY"] / c["SQ_WAVE_CYCLES"]
+        kernels[key] = e
+    return dict(workload=workload, device="MI355X (gfx950), one GPU", calibration=cal, kernels=kernels,
+                commands=[" ".join(["rocprofv3", *pa, "--output-format csv -d <raw>/" + f"{workload}_{tag}", "-o", workload, "--",
+                                    "python3 bench.py --workload", workload, "--no-cpu-baseline", *ba]) for tag, pa, ba in PASSES],
+                note="each pass is its own run from /tmp with TMPDIR=/tmp; HBM bytes = counter KiB x 1024 x calibration factor")
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--workload", action="append", choices=["c2", "c3", "c4", "c5"])
+    ap.add_argument("--raw", default=os.path.join(ROOT, "gpurun_out", "counters"), help="where rocprofv3 writes its CSVs")
+    ap.add_argument("--out", default=os.path.join(ROOT, "profiles"))
+    ap.add_argument("--limit", type=int, default=170, help="seconds allowed per rocprofv3 pass")
+    a = ap.parse_args()
+    for w in a.workload or ["c4"]:
+        res = profile(w, a.raw, a.limit)
+        path = os.path.join(a.out, f"ttt_mlp_{w}_counters.json")
+        with open(path, "w") as f:
+            json.dump(res, f, indent=1, sort_keys=True)
+        print("wrote", path, flush=True)
+        for k, e in res["kernels"].items():
+            print(f"  {k:40s} {e['avg_ns'] / 1e6:9.3f} ms  HBM {e.get('hbm_bytes', 0) / 1e9:8.2f} GB ({e.get('hbm_gbs', 0):6.0f} GB/s)  "
+                  f"MFMA {e.get('mfma_busy_pct', 0):5.1f} %  VALU {e.get('valu_busy_pct', 0):5.1f} %  "
+                  f"LDS conflicts {100 * e.get('lds_conflict_share', 0):4.1f} %  waiting {100 * e.get('wait_share', 0):4.1f} %", flush=True)
+
+
+if __name__ == "__main__":
+    sys.exit(main())
