@@ -178,9 +178,11 @@ def main():
     ap.add_argument("--out", default=os.path.join(ROOT, "profiles"))
     ap.add_argument("--limit", type=int, default=170, help="seconds allowed per rocprofv3 pass")
     a = ap.parse_args()
+    raw, out = os.path.abspath(a.raw), os.path.abspath(a.out)    # rocprofv3 runs from /tmp
+    os.makedirs(out, exist_ok=True)
     for w in a.workload or ["c4"]:
-        res = profile(w, a.raw, a.limit)
-        path = os.path.join(a.out, f"ttt_mlp_{w}_counters.json")
+        res = profile(w, raw, a.limit)
+        path = os.path.join(out, f"ttt_mlp_{w}_counters.json")
         with open(path, "w") as f:
             json.dump(res, f, indent=1, sort_keys=True)
         print("wrote", path, flush=True)
