@@ -235,6 +235,31 @@ def test_bf16_operand_variant_stays_close_to_fp32_oracle():
     assert orc.parity_stats(ckb.W1, cka.W1)["cosine"] > 0.9999
 
 
+def test_operand_rounding_classes_separate_the_sources_of_error():
+    """The rounding switches per operand class (weights / activations / activation gradients) that located what the
+    kernels must carry in two bf16 terms: rounding nothing reproduces the oracle, rounding one class costs
+    less than rounding all three, and every variant stays within the parity bar at this length."""
+    d = orc.make_inputs(1, 2, 48, seed=3)
+    ref, ck, _ = orc.ttt_forward(*[d[k] for k in FWD_KEYS], 8)
+    up = orc.State(d["grad_L_W1_last"], d["grad_L_b1_last"], d["grad_L_W2_last"], d["grad_L_b2_last"])
+    args = (d["XQ"], d["XK"], d["XV"], d["last_eta"], d["ttt_norm_weight"], d["ttt_norm_bias"])
+    gref = orc.ttt_backward(*args, ck, up, d["grad_L_XQW_mini_batch"], 8)
+
+    def err(rounding):
+        out, c, _ = orc.ttt_forward(*[d[k] for k in FWD_KEYS], 8, emulate_bf16_operands=rounding)
+        g = orc.ttt_backward(*args, c, up, d["grad_L_XQW_mini_batch"], 8, emulate_bf16_operands=rounding)
+        worst = max(1 - orc.parity_stats(g[k], gref[k])["cosine"] for k in gref)
+        return worst, out
+
+    none, out = err(orc.OperandRounding(w=False, a=False, g=False))
+    assert none < 1e-12 and torch.equal(out, ref)      # cosine of identical tensors, up to its own rounding
+    all3, _ = err(orc.OperandRounding())
+    assert 0 < all3 < 1e-4
+    for kw in (dict(w=True, a=False, g=False), dict(w=False, a=True, g=False), dict(w=False, a=False, g=True)):
+        one, _ = err(orc.OperandRounding(**kw))
+        assert 0 < one < all3, kw
+
+
 # ------------------------------------------------- per-group tensors (what the kernel leaves for group 0)
 @pytest.mark.parametrize("NC,cgs,group", [(5, 2, 0), (5, 2, 2), (3, 4, 0), (4, 4, 0)])
 def test_group_tensors_match_library_routines_and_autograd(NC, cgs, group):

@@ -1,0 +1,39 @@
+"""The counter harness's arithmetic on synthetic rocprofv3 CSVs (no GPU, no rocprofv3): per-dispatch sums over the
+counter's dimension rows, the copy calibration, and the derived busy / conflict / wait figures."""
+import csv
+import os
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "ttt-tk_amd"))
+
+import profile_counters as pc  # noqa: E402
+
+
+def _write(path, header, rows):
+    os.makedirs(os.path.dirname(path), exist_ok=True)
+    with open(path, "w", newline="") as f:
+        w = csv.writer(f)
+        w.writerow(header)
+        w.writerows(rows)
+
+
+def test_kernel_names_are_shortened_and_classified():
+    assert pc.short_name("ttt::ttt_mlp_bwd_split_kernel<2, true>(ttt::BwdParams)") == "ttt_mlp_bwd_split_kernel<2, true>"
+    assert pc.is_ours("void ttt::ttt_mlp_fwd_kernel(ttt::FwdParams)") and not pc.is_ours("at::native::copy_kernel")
+    assert pc.is_copy("void at::native::elementwise_kernel<direct_copy_kernel_cuda>") and not pc.is_copy("ttt_mlp_fwd_kernel")
+
+
+def test_counter_rows_of_one_dispatch_are_summed_and_dispatches_kept_apart(tmp_path):
+    hdr = ["Dispatch_Id", "Kernel_Name", "Counter_Name", "Counter_Value"]
+    rows = [[1, "k", "FETCH_SIZE", 10], [1, "k", "FETCH_SIZE", 5], [2, "k", "FETCH_SIZE", 7], [3, "copy", "FETCH_SIZE", 4]]
+    _write(str(tmp_path / "x" / "c4_counter_collection.csv"), hdr, rows)
+    got = pc.counter_sums(str(tmp_path / "x"))
+    assert sorted(got["k"]["FETCH_SIZE"]) == [7.0, 15.0] and got["copy"]["FETCH_SIZE"] == [4.0]
+
+
+def test_kernel_stats_are_read_by_name(tmp_path):
+    hdr = ["Name", "Calls", "TotalDurationNs", "AverageNs", "Percentage", "MinNs", "MaxNs", "StdDev"]
+    _write(str(tmp_path / "t" / "c4_kernel_stats.csv"), hdr, [["ttt::ttt_mlp_fwd_kernel(ttt::FwdParams)", 3, 300, 100.0, 50.0, 90, 110, 1]])
+    st = pc.kernel_stats(str(tmp_path / "t"))
+    assert st["ttt::ttt_mlp_fwd_kernel(ttt::FwdParams)"]["avg_ns"] == 100.0
