@@ -165,8 +165,8 @@ size_t ttt_mlp_bwd_status_offset(int32_t B, int32_t NH);
  * results): one workgroup carries the state through the mini-batches and leaves every new state
  * in the workspace as bf16 operands, the other computes Out from them, 8 mini-batches behind
  * (32 when NC >= 512).
- * Used only when all pairs fit at two workgroups each (2*B*NH <= CUs): behind full rounds the
- * forward gains nothing from it.
+ * Pairs are covered as in the backward: full rounds of the device with one workgroup per pair, then the
+ * remaining n pairs with two each if 2*n fits the CUs.
  * No counterpart in the reference launcher (kernels/ttt/ttt.cu:594-721). */
 size_t ttt_mlp_fwd_workspace_bytes(int32_t B, int32_t NH);
 size_t ttt_mlp_fwd_status_offset(int32_t B, int32_t NH);

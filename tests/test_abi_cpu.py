@@ -193,8 +193,9 @@ def test_launch_plan_keeps_waiting_workgroups_within_the_device(lib):
     assert plan(1, 384, 256) == (256, 128, 2)      # one full round, the rest with two each
     assert plan(1, 260, 256) == (256, 4, 4)
     assert plan(1, 512, 256) == (512, 0, 0)
-    assert plan(0, 48, 256) == (0, 48, 2)          # forward: two, and only if everything fits
-    assert plan(0, 384, 256) == (384, 0, 0)
+    assert plan(0, 48, 256) == (0, 48, 2)          # forward: two per pair at most
+    assert plan(0, 384, 256) == (256, 128, 2)
+    assert plan(0, 200, 256) == (200, 0, 0)
     assert plan(1, 48, 0) == (48, 0, 0)            # no device: nothing to overlap
     for which in (0, 1):
         for cus in (1, 8, 104, 256, 304):

@@ -80,6 +80,8 @@ def test_forward_matches_oracle(B, NH, NC, cgs, seed, rand_affine):
     (2, 3, 9, 4),        # one full hand-over and a ragged one; (batch, head) count not a multiple of 8
     (1, 8, 40, 8),       # five hand-overs: both halves of the ring are reused, the recurrence waits for the output branch
     (1, 4, 33, 16),
+    (2, 130, 5, 2),      # more pairs than CUs: a full round with one workgroup each, the remaining 4 pairs with two
+    (1, 72, 5, 2),
 ])
 def test_overlapped_forward_is_bit_identical(B, NH, NC, cgs):
     """Computing Out on a second workgroup changes the schedule, not one bit of the results."""

@@ -130,9 +130,8 @@ struct LaunchPlan {
   bool rest_split = false;
   int per_pair = 1;         // workgroups per pair of the rest: 2, or 3 / 4 where the kernel can use them and they fit
 };
-// `after_full_rounds`: whether the rest may be split when full rounds precede it.  That pays for the
-// backward; the forward's gain from splitting is smaller than what a full device costs it (measured).
-LaunchPlan plan_for(long long BH, int cus, bool after_full_rounds, bool three_way) {
+// `three_way`: the backward can use three or four workgroups per pair, the forward two.
+LaunchPlan plan_for(long long BH, int cus, bool three_way) {
   LaunchPlan pl;
   if (BH <= 0 || cus <= 0) {
     pl.n_single = BH > 0 ? BH : 0;
@@ -140,16 +139,16 @@ LaunchPlan plan_for(long long BH, int cus, bool after_full_rounds, bool three_wa
   }
   pl.n_single = BH / cus * cus;
   pl.n_rest = BH - pl.n_single;
-  pl.rest_split = pl.n_rest > 0 && 2 * pl.n_rest <= cus && (after_full_rounds || pl.n_single == 0);
+  pl.rest_split = pl.n_rest > 0 && 2 * pl.n_rest <= cus;
   if (!pl.rest_split) { pl.n_single = BH; pl.n_rest = 0; }
   else pl.per_pair = !three_way ? 2 : 4 * pl.n_rest <= cus ? 4 : 3 * pl.n_rest <= cus ? 3 : 2;
   return pl;
 }
-LaunchPlan plan_launches(long long BH, bool after_full_rounds, bool three_way) {
+LaunchPlan plan_launches(long long BH, bool three_way) {
   int dev = 0, cus = 0;
   if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
     cus = 0;
-  return plan_for(BH, cus, after_full_rounds, three_way);
+  return plan_for(BH, cus, three_way);
 }
 
 // Workspace of the backward with 2 or 3 workgroups per pair, for n (batch, head) pairs: the synchronisation
@@ -227,7 +226,7 @@ extern "C" int ttt_mlp_bwd_export_group0(const ttt_mlp_bwd_args* a, void* stream
 
 extern "C" size_t ttt_mlp_bwd_workspace_bytes(int B, int NH, int checkpoint_group_size) {
   if (B <= 0 || NH <= 0 || checkpoint_group_size <= 0 || checkpoint_group_size > (1 << 16)) return 0;
-  const LaunchPlan pl = plan_launches((long long)B * NH, true, true);
+  const LaunchPlan pl = plan_launches((long long)B * NH, true);
   if (!pl.rest_split) return 0;
   const int n_replay = pl.per_pair >= 3 ? 2 : 1;
   return BwdWorkspace(pl.n_rest, checkpoint_group_size, 2 * n_replay - 1, pl.per_pair == 4).total;
@@ -235,7 +234,7 @@ extern "C" size_t ttt_mlp_bwd_workspace_bytes(int B, int NH, int checkpoint_grou
 
 extern "C" size_t ttt_mlp_bwd_status_offset(int B, int NH) {
   if (B <= 0 || NH <= 0) return 0;
-  const LaunchPlan pl = plan_launches((long long)B * NH, true, true);
+  const LaunchPlan pl = plan_launches((long long)B * NH, true);
   return pl.rest_split ? (size_t)pl.n_rest * ttt::BWD_SYNC_STRIDE * sizeof(int) : 0;
 }
 
@@ -243,7 +242,7 @@ extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* wo
   ttt::BwdParams p;
   if (int rc = make_bwd_params(a, p)) return rc;
   if (int rc = check_workspace(workspace)) return rc;
-  const LaunchPlan pl = plan_launches((long long)p.B * p.NH, true, true);
+  const LaunchPlan pl = plan_launches((long long)p.B * p.NH, true);
   if (!pl.rest_split) return TTT_MLP_ERR_NO_ROOM;
   const int n_replay = pl.per_pair >= 3 ? 2 : 1, alt_sets = 2 * n_replay - 1;
   const bool finish = pl.per_pair == 4;
@@ -301,13 +300,13 @@ extern "C" int ttt_mlp_fwd_launch(const ttt_mlp_fwd_args* a, void* stream) {
 
 extern "C" size_t ttt_mlp_fwd_workspace_bytes(int B, int NH) {
   if (B <= 0 || NH <= 0) return 0;
-  const LaunchPlan pl = plan_launches((long long)B * NH, false, false);
+  const LaunchPlan pl = plan_launches((long long)B * NH, false);
   return pl.rest_split ? FwdWorkspace(pl.n_rest).total : 0;
 }
 
 extern "C" size_t ttt_mlp_fwd_status_offset(int B, int NH) {
   if (B <= 0 || NH <= 0) return 0;
-  const LaunchPlan pl = plan_launches((long long)B * NH, false, false);
+  const LaunchPlan pl = plan_launches((long long)B * NH, false);
   return pl.rest_split ? (size_t)pl.n_rest * ttt::BWD_SYNC_STRIDE * sizeof(int) : 0;
 }
 
@@ -315,7 +314,7 @@ extern "C" int ttt_mlp_fwd_launch_overlapped(const ttt_mlp_fwd_args* a, void* wo
   ttt::FwdParams p;
   if (int rc = make_fwd_params(a, p)) return rc;
   if (int rc = check_workspace(workspace)) return rc;
-  const LaunchPlan pl = plan_launches((long long)p.B * p.NH, false, false);
+  const LaunchPlan pl = plan_launches((long long)p.B * p.NH, false);
   if (!pl.rest_split) return TTT_MLP_ERR_NO_ROOM;
   const FwdWorkspace w(pl.n_rest);
   if (workspace_bytes < w.total) return TTT_MLP_ERR_WORKSPACE;
@@ -390,7 +389,7 @@ extern "C" int ttt_mlp_fwd_launch_static(const ttt_mlp_fwd_args* a, int* sticky_
   if (int rc = make_fwd_params(a, p)) return rc;
   const long long pairs = (long long)p.B * p.NH;
   if (pairs > STATIC_MAX_PAIRS) return TTT_MLP_ERR_SCRATCH;
-  const LaunchPlan pl = plan_launches(pairs, false, false);
+  const LaunchPlan pl = plan_launches(pairs, false);
   if (!pl.rest_split || pl.n_single != 0) return TTT_MLP_ERR_NO_ROOM;
   const FwdWorkspace w(pl.n_rest);
   static_assert(static_scratch_bytes() % 256 == 0, "scratch parts are 256-byte aligned");
@@ -412,7 +411,7 @@ extern "C" int ttt_mlp_launch_plan(int which, long long pairs, int compute_units
                                    long long* other_pairs, int* workgroups_per_other_pair) {
   if (one_workgroup_pairs == nullptr || other_pairs == nullptr || workgroups_per_other_pair == nullptr || (which != 0 && which != 1))
     return TTT_MLP_ERR_BAD_ARG;
-  const LaunchPlan pl = plan_for(pairs, compute_units, which == 1, which == 1);
+  const LaunchPlan pl = plan_for(pairs, compute_units, which == 1);
   *one_workgroup_pairs = pl.n_single;
   *other_pairs = pl.n_rest;
   *workgroups_per_other_pair = pl.n_rest > 0 ? pl.per_pair : 0;
