@@ -658,32 +658,10 @@ TTT_DEV void fwd_output_branch(const FwdParams& p, unsigned char* smem, const in
   }
   const size_t x_base = uni64((size_t)bh * p.NC * (CS * FD));
   const gptr_t gXQ = gbuf(p.XQ + x_base), gOut = gbuf(p.Out + x_base);
-  const gptr_t gXK = gbuf(p.XK + x_base), gXV = gbuf(p.XV + x_base), gEta = gbuf(p.last_eta + uni64((size_t)bh * p.NC * CS));
   int* const w_given = p.sync + (size_t)bh * BWD_SYNC_STRIDE;
   int* const w_taken = w_given + 16;
   int* const w_status = p.status;
   int* const s_flag = reinterpret_cast<int*>(smem + SM_FLAG);
-
-  // The recurrence workgroup of this (batch, head) sits on the same XCD and shares its L2.  It reads XK, XV and
-  // eta of a mini-batch one LayerNorm stage before it needs them, which does not cover the latency of HBM; this
-  // workgroup has time to spare, so it reads those tiles ahead of the recurrence - which is about a hand-over
-  // group ahead of this workgroup - and the recurrence finds them in the L2.  The values are not used.
-  constexpr int AHEAD = RING + 4;   // measured: RING + 1 .. RING + 4 alike; RING + 10 and more slower (the tiles leave the L2
-                                    // again), RING - 4 slower and RING - 12 no gain at all (the recurrence is that far ahead)
-  static_assert(AHEAD > 0, "the tiles read ahead must lie ahead: a negative mini-batch index would address memory before the tensor");
-  u32x4 warm_k = {0, 0, 0, 0}, warm_v = {0, 0, 0, 0};
-  unsigned warm = 0;
-#define WARM(mbn)                                                                       \
-  do {                                                                                  \
-    LANE_VARS;                                                                          \
-    warm ^= warm_k[0] ^ warm_v[0];                                                      \
-    if ((mbn) < p.NC) {                                                                 \
-      warm_k = g_ld16(gXK, 16 * tid, (mbn) * TILE_BYTES);                               \
-      warm_v = g_ld16(gXV, 16 * tid, (mbn) * TILE_BYTES);                               \
-      if (tid < 2) warm ^= (unsigned)g_ld<unsigned>(gEta, 64 * tid, (mbn) * (CS * 2));  \
-    }                                                                                   \
-  } while (0)
-  for (int mbn = 1; mbn < AHEAD; mbn++) WARM(mbn);   // the start of the sequence, while the first group is being produced
 
   for (int mb = 0; mb < p.NC; mb++) {
     LANE_VARS;
@@ -691,7 +669,6 @@ TTT_DEV void fwd_output_branch(const FwdParams& p, unsigned char* smem, const in
     if (at == 0) {
       if (!wait_at_least(w_given, grp + 1, w_status, s_flag, p.wait_limit)) return;
     }
-    WARM(mb + AHEAD);
     bf16* s_xq = reinterpret_cast<bf16*>(smem + SM_XQ + (mb & 1) * SM_TILE);
     const gptr_t gImg = gbuf(p.state_img + ((size_t)bh * 2 * FWD_RING_MAX + slot) * (FWD_IMG_BYTES / 2));
     const float* gB = p.bias_img + ((size_t)bh * 2 * FWD_RING_MAX + slot) * FWD_BIAS_FLOATS;
@@ -744,8 +721,6 @@ TTT_DEV void fwd_output_branch(const FwdParams& p, unsigned char* smem, const in
     }
     if (at == ring - 1 || mb == p.NC - 1) publish(w_taken, grp + 1);
   }
-  asm volatile("" ::"v"(warm ^ warm_k[0] ^ warm_v[0]));   // keeps the loads above alive
-#undef WARM
 #undef LANE_VARS
 }
 
