@@ -732,7 +732,6 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           acc_zero(g1);
           // W2[shard, :] with F contracted (lane = hid): the two terms of W2s, written as rows [F][hid] into T1 / T2
           // and read back transposed
-          bf16x8 w2h[4], w2l[4];
 #pragma unroll
           for (int fb = 0; fb < 2; fb++)
 #pragma unroll
@@ -744,14 +743,8 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
             }
           WAVE_SYNC();
 #pragma unroll
-          for (int s = 0; s < 4; s++) {
-            w2h[s] = piece_tr<LDH>(T1, 0, s, lane);
-            w2l[s] = piece_tr<LDH>(T2, 0, s, lane);
-          }
-          WAVE_SYNC();   // read before G1 takes the tiles' place below
-#pragma unroll
           for (int s = 0; s < 4; s++) {                      // W2: lane = hid, contraction = F; G2: lane = tok; two terms each
-            const bf16x8 wh = w2h[s], wl = w2l[s];
+            const bf16x8 wh = piece_tr<LDH>(T1, 0, s, lane), wl = piece_tr<LDH>(T2, 0, s, lane);
             bf16x8 gh[2], gl[2];
 #pragma unroll
             for (int i = 0; i < 2; i++) {
@@ -765,6 +758,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
               g1.b[0][i] = MFMA(wh, gh[i], g1.b[0][i]);
             }
           }
+          WAVE_SYNC();   // W2's terms are read before G1 takes their place
 #pragma unroll
           for (int i = 0; i < 2; i++)
 #pragma unroll
