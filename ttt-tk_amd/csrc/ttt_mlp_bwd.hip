@@ -655,6 +655,9 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
                 xv[jj] = gh;
                 x2lo[i][t][jj] = (bf16)(g - (float)gh);
                 d1f[i][8 * t + jj] = d;
+                // pinned: left to itself the compiler finishes gelu' only where it is used, two stages on, and keeps
+                // three values per element alive until then instead of one (a dozen of them in scratch memory)
+                asm volatile("" : "+v"(d1f[i][8 * t + jj]));
               }
               store_piece_rows<LDH>(T0, tb[i], t, c, h, xv);
             }
@@ -860,6 +863,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
                 x2bQ[i][t][jj] = (bf16)g;
                 d1b[i][t][jj] = (bf16)d;
               }
+              asm volatile("" : "+v"(d1b[i][t]));   // finished here, not where it is used (see gelu'(Z1) above)
               store_piece_rows<LDH>(T0, tb[i], t, c, h, x2bQ[i][t]);
             }
           AccT<2, 2> z2;
