@@ -9,6 +9,8 @@ sys.path.insert(0, os.path.join(ROOT, "ttt-tk_amd"))
 
 import profile_counters as pc  # noqa: E402
 
+PKG = os.path.join(ROOT, "ttt-tk_amd")
+
 
 def _write(path, header, rows):
     os.makedirs(os.path.dirname(path), exist_ok=True)
@@ -37,3 +39,32 @@ def test_kernel_stats_are_read_by_name(tmp_path):
     _write(str(tmp_path / "t" / "c4_kernel_stats.csv"), hdr, [["ttt::ttt_mlp_fwd_kernel(ttt::FwdParams)", 3, 300, 100.0, 50.0, 90, 110, 1]])
     st = pc.kernel_stats(str(tmp_path / "t"))
     assert st["ttt::ttt_mlp_fwd_kernel(ttt::FwdParams)"]["avg_ns"] == 100.0
+
+
+def test_stage_names_come_from_the_kernels_header_and_fit_the_slots():
+    """stage_clocks.py labels the clock slots with the enum entries of csrc/ttt_mlp_kernels.hpp, in order."""
+    import re
+    import stage_clocks as sc
+    header = open(os.path.join(PKG, "csrc", "ttt_mlp_kernels.hpp")).read()
+    fwd, bwd = sc.stage_names(header, "FwdStage"), sc.stage_names(header, "BwdStage")
+    assert [n for n, _ in fwd][:3] == ["FS_TOP", "FS_F1_GELU", "FS_X2_SPLIT"] and fwd[-1][0] == "FS_OUT_LN"
+    assert bwd[0][0] == "BS_GROUP" and bwd[-1][0] == "BS_PUBLISH"
+    assert all(desc for _, desc in fwd + bwd), "every stage carries its description"
+    slots = int(re.search(r"constexpr int STAGE_SLOTS = (\d+);", header).group(1))
+    assert slots == sc.SLOTS and len(fwd) <= slots and len(bwd) <= slots
+    # every stage is marked in the kernel it belongs to
+    fsrc = open(os.path.join(PKG, "csrc", "ttt_mlp_fwd.hip")).read()
+    bsrc = open(os.path.join(PKG, "csrc", "ttt_mlp_bwd.hip")).read()
+    for n, _ in fwd:
+        assert f"TTT_STAGE({n})" in fsrc, n
+    for n, _ in bwd:
+        assert f"TTT_STAGE({n})" in bsrc, n
+
+
+def test_the_product_library_contains_no_stage_clocks():
+    import ctypes
+    lib = ctypes.CDLL(os.path.join(PKG, "libttt_mlp.so"))
+    assert not hasattr(lib, "ttt_mlp_set_stage_clocks")
+    stages = os.path.join(PKG, "libttt_mlp_stages.so")
+    if os.path.exists(stages):
+        assert hasattr(ctypes.CDLL(stages), "ttt_mlp_set_stage_clocks")

@@ -2,6 +2,7 @@
 
     python ttt-tk_amd/build.py            # kernels + C ABI library + Python module
     python ttt-tk_amd/build.py --lib      # kernels + C ABI library only
+    python ttt-tk_amd/build.py --stages   # libttt_mlp_stages.so: the library with stage clocks, for stage_clocks.py
 
 Outputs (next to this file, picked up by `import test_time_training` once this directory is on
 sys.path):
@@ -37,12 +38,13 @@ def module_path() -> str:
     return os.path.join(HERE, "test_time_training" + sysconfig.get_config_var("EXT_SUFFIX"))
 
 
-def build_lib(extra_flags=()) -> str:
+def build_lib(extra_flags=(), lib: str = LIB, objdir: str = "build") -> str:
+    """Compiles the four HIP sources and links them into `lib` (objects under `objdir`, next to this file)."""
     objs = []
-    os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
+    os.makedirs(os.path.join(HERE, objdir), exist_ok=True)
     procs = []
     for src in HIP_SOURCES:
-        obj = os.path.join(HERE, "build", src.replace(".hip", ".o"))
+        obj = os.path.join(HERE, objdir, src.replace(".hip", ".o"))
         cmd = ["hipcc", *HIP_FLAGS, *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj]
         print("+", " ".join(cmd), flush=True)
         procs.append((cmd, subprocess.Popen(cmd)))
@@ -50,8 +52,16 @@ def build_lib(extra_flags=()) -> str:
     for cmd, p in procs:
         if p.wait() != 0:
             raise subprocess.CalledProcessError(p.returncode, cmd)
-    _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB])
-    return LIB
+    _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", lib])
+    return lib
+
+
+STAGES_LIB = os.path.join(HERE, "libttt_mlp_stages.so")
+
+
+def build_stages_lib() -> str:
+    """The same library with the stage clocks compiled in (-DTTT_STAGE_CLOCKS), for stage_clocks.py only."""
+    return build_lib(("-DTTT_STAGE_CLOCKS",), STAGES_LIB, os.path.join("build", "stages"))
 
 
 def build_module() -> str:
@@ -79,7 +89,11 @@ def build_all() -> None:
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--lib", action="store_true", help="build only libttt_mlp.so")
+    ap.add_argument("--stages", action="store_true", help="build only libttt_mlp_stages.so (stage clocks compiled in)")
     a = ap.parse_args()
+    if a.stages:
+        print("built:", build_stages_lib())
+        sys.exit(0)
     build_lib()
     if not a.lib:
         build_module()

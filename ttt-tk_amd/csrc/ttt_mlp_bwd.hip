@@ -557,6 +557,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
     WAVE_SYNC();
   };
 
+  TTT_STAGES_BEGIN();
   for (int k = p.K - 1; k >= 0; k--) {
     const int n_mb = min(cgs, p.NC - k * cgs);
     const int done = p.K - 1 - k;                    // number of this group, counted from the end of the sequence
@@ -596,11 +597,13 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         stage3_load(st, bXQ, bXK, bXV, bETA, k * cgs, tid, t16);
         stage3_store(st, s_xq, s_xk, s_e2, s_etah, tid);
       }
+      TTT_STAGE(BS_GROUP);
       for (int j = 0; j < n_mb; j++) {
         const int mb = k * cgs + j;
         REFRESH_OFFSETS();
         LANE_VARS;
         __syncthreads();   // the staged inputs (and, for j = 0, the biases) are visible
+        TTT_STAGE(BS_R_TOP);
 
         // Z1^T = W1s^T XK^T + b1  (rows hid, lane = tok); X2 rows [tok][hid] -> T0; gelu'(Z1) (fp32) and the
         // low-order term of X2 stay in registers.  The products that carry the state to the next mini-batch
@@ -662,6 +665,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
               store_piece_rows<LDH>(T0, tb[i], t, c, h, xv);
             }
         }
+        TTT_STAGE(BS_R_F1_GELU);
         WAVE_SYNC();
         {
           LANE_VARS;
@@ -684,6 +688,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           }
           pair_sum(s_own, s_partner, z2, c, h);
         }
+        TTT_STAGE(BS_R_F2_PAIRSUM);
         // fused LayerNorm + reconstruction-loss gradient; saves for the reverse walk
         {
           LANE_VARS;
@@ -728,6 +733,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           if ((lane & 7) == 0) g_stf(bSDF, vtok, j * (CS * 4), sd);
         }
         __syncthreads();
+        TTT_STAGE(BS_R_LN);
         // G1 = (W2 G2^T) * gelu'(Z1)  (rows hid, lane = tok) -> T1 rows [tok][hid]; weight step
         {
           LANE_VARS;
@@ -779,6 +785,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
             }
         }
         WAVE_SYNC();
+        TTT_STAGE(BS_R_F3);
         {   // weight step
           LANE_VARS;
 #pragma unroll
@@ -823,6 +830,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           }
           WAVE_SYNC();   // this wave's readers of T1 / T2 are done
         }
+        TTT_STAGE(BS_R_WSTEP);
         // operand images of the state after this step, for the reverse walk; the image of W2 (lane = hid,
         // contraction = F) also serves the output branch below
         bf16x8 w2a[4];
@@ -842,6 +850,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
 #pragma unroll
             for (int s = 0; s < 2; s++) image_store<ROLE != 0>(bIMG1, j * IMG_BYTES, 2 * fb + s, t16, piece_tr<LDF>(T2, fb, s, lane));
         }
+        TTT_STAGE(BS_R_IMAGES);
         // post-update forward on XQ; X2_bar rows [tok][hid] -> T0, gelu'(Z1_bar) packed
         bf16x8 d1b[2][2];
         {
@@ -873,6 +882,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           WAVE_SYNC();   // this wave's readers of T1 / T2 are done
           pair_sum(s_own, s_partner, z2, c, h);
         }
+        TTT_STAGE(BS_R_OUT_FORWARD);
         // ---- the output branch, backwards: it needs the state after this step, which is in registers
         //      right now, and nothing of the running gradients.  Output LayerNorm forward and backward:
         float gO[8];
@@ -914,6 +924,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           ln_store_g<ROLE != 0>(bGZB, vln, j * TILE_BYTES, gx);
         }
         __syncthreads();
+        TTT_STAGE(BS_R_OUT_LN);
         {
           LANE_VARS;
           bf16x8 w1a[2][2];   // W1 after the step (lane = F, contraction = hid): the image stored above, fetched ahead of its use
@@ -964,6 +975,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           g_st_stream<bf16x8>(bDXQ, vln, mb * TILE_BYTES, dxq_old);
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the next mini-batch's inputs are in LDS before the barrier at the loop's top
+        TTT_STAGE(BS_R_OUT_BACKWARD);
       }
       if constexpr (ROLE == 1) {
         if (done + n_replay >= p.K) {   // this workgroup's last group: hand its norm-gradient sums to the walk
@@ -985,6 +997,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         norm_swap(done & 1);
       }
       if constexpr (ROLE == 1) publish(w_replayed, done / n_replay + 1);
+      TTT_STAGE(BS_PUBLISH);
     }
 
     // ================================================================= reverse walk
@@ -1001,6 +1014,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
     const size_t ofin = uni64(((size_t)bh * 2 + (done & 1)) * cgs);
 #define bFDZ gbuf(ka->fin_dz + ofin * (CS * HID))
 #define bFGY gbuf(ka->fin_gy + ofin * (2 * CS * FD))
+    TTT_STAGE(BS_GROUP);
     if constexpr (ROLE != 1)
     for (int j = n_mb - 1; j >= 0; j--) {
       const int mb = k * cgs + j;
@@ -1038,6 +1052,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
       }
       __syncthreads();
 
+      TTT_STAGE(BS_W_TOP);
       bf16x8 w2bf[4];   // W2 before this step (lane = hid, contraction = F): fetched now, needed by the next stage
       bf16x8 gq[2][2], aq[2][2], bq[2][2];
       {
@@ -1063,6 +1078,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
       }
       // gb2 holds its value after the first update
 
+      TTT_STAGE(BS_W_BAR_TERMS);
       // ---- the weight step, backwards (uses the state BEFORE this mini-batch).
       //      Parked across the LayerNorm stage: X2 in T0; packed d1 = gelu'(Z1), g1 = -eta * dl/dZ1 and
       //      t2 = -eta * (gZ2 W2^T) * (XK gW1 + gb1) * gelu''(Z1).
@@ -1159,6 +1175,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           if (h == 0) s_deta[v * CS + 32 * tb[i] + c] = a;
         }
         WAVE_SYNC();   // this wave's readers of T1 / T2 are done
+        TTT_STAGE(BS_W_STEP_BACK);
         {   // what the LayerNorm stage reads from HBM is under way during the pair sum
           LANE_VARS;
           if constexpr (!FIN) dxv_old = g_ld_stream<bf16x8>(OLD_VALUE(bDXV, xo));
@@ -1169,6 +1186,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         }
         pair_sum(s_own, s_partner, pz, c, h);
       }
+      TTT_STAGE(BS_W_PAIRSUM);
       // all pair sums of ggZ2 and the dEta partial sums are in LDS
 
       // ---- second-order pass through the fused LayerNorm loss (LayerNorm lanes)
@@ -1242,7 +1260,9 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         ln_store(s_a + tok * LDX + f0, gx);
         if constexpr (!FIN) g_st_stream<bf16x8>(bDXV, vln, xo, dxv_old);
       }
+      TTT_STAGE(BS_W_LN);
       __syncthreads();  // dZ2 tile complete; regions (T1 / T2) free again
+      TTT_STAGE(BS_W_LN_BARRIER);
 
       // ---- inner MLP, backwards (uses the state BEFORE this mini-batch)
       bf16x8 dxk_old;
@@ -1312,6 +1332,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
 #pragma unroll
             for (int t = 0; t < 2; t++) image_store<true>(bFDZ, ho, 2 * tb[i] + t, t16, dzp[i][t]);
         }
+        TTT_STAGE(BS_W_MLP_BACK);
         WAVE_SYNC();   // S, P2 and gW1 G1^T have consumed T2 / T1
 #pragma unroll
         for (int i = 0; i < 2; i++)
@@ -1332,6 +1353,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         mma_jit<4>(gW1s, [&](int fb, int s) { return xpiece_tr(s_xk, fb, s, lane); },         // XK^T: lane = F
                    [&](int, int s) { return piece_tr<LDH>(T1, 0, s, lane); });                 // dZ1: lane = hid
         lds_rowsum_add_jit(s_gb1w, [&](int s) { return piece_tr<LDH>(T1, 0, s, lane); }, ones, c, h);
+        TTT_STAGE(BS_W_UPDATES);
         WAVE_SYNC();   // this wave's readers of T1 / T2 are done
         if constexpr (!FIN) {
           {
@@ -1351,11 +1373,14 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         for (int e = 0; e < 8; e++) dxk_old[e] = (bf16)((float)dxk_old[e] + (z[e] + gyv[e]));
         g_st_stream<bf16x8>(bDXK, vln, xo, dxk_old);
       }
+      TTT_STAGE(BS_W_DXK);
     }
     if constexpr (ROLE == 2) publish(w_walked, done + 1);
+    TTT_STAGE(BS_PUBLISH);
 #undef bFDZ
 #undef bFGY
   }
+  TTT_STAGES_END(p.stage_clocks == nullptr ? nullptr : p.stage_clocks + ((size_t)bh * 4 + (ROLE == 1 ? turn : 2)) * (BW_NWAVE * STAGE_SLOTS));
   if constexpr (ROLE == 1) return;
 
   // ---- outputs that are written once

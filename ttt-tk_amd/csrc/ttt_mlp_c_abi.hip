@@ -49,6 +49,17 @@ extern "C" const char* ttt_mlp_error_string(int code) {
   }
 }
 
+#ifdef TTT_STAGE_CLOCKS
+namespace {
+unsigned* g_stage_clocks_fwd = nullptr;
+unsigned* g_stage_clocks_bwd = nullptr;
+}  // namespace
+extern "C" void ttt_mlp_set_stage_clocks(unsigned* forward, unsigned* backward) {
+  g_stage_clocks_fwd = forward;
+  g_stage_clocks_bwd = backward;
+}
+#endif
+
 namespace {
 int make_fwd_params(const ttt_mlp_fwd_args* a, ttt::FwdParams& p) {
   if (a == nullptr) return TTT_MLP_ERR_BAD_ARG;
@@ -66,6 +77,9 @@ int make_fwd_params(const ttt_mlp_fwd_args* a, ttt::FwdParams& p) {
   p.W1_ck = a->W1_checkpoints; p.b1_ck = a->b1_checkpoints; p.W2_ck = a->W2_checkpoints; p.b2_ck = a->b2_checkpoints;
   p.Out = bf(a->Out);
   p.B = a->B; p.NH = a->NH; p.NC = a->NC; p.K = a->K; p.cgs = a->checkpoint_group_size;
+#ifdef TTT_STAGE_CLOCKS
+  p.stage_clocks = g_stage_clocks_fwd;
+#endif
   return TTT_MLP_OK;
 }
 }  // namespace
@@ -116,6 +130,9 @@ int make_bwd_params(const ttt_mlp_bwd_args* a, ttt::BwdParams& p) {
   p.grad_L_XQ = bf(a->grad_L_XQ); p.grad_L_XK = bf(a->grad_L_XK); p.grad_L_XV = bf(a->grad_L_XV);
   p.B = a->B; p.NH = a->NH; p.NC = a->NC; p.K = a->K; p.cgs = a->checkpoint_group_size;
   p.overwrite = a->overwrite != 0;
+#ifdef TTT_STAGE_CLOCKS
+  p.stage_clocks = g_stage_clocks_bwd;
+#endif
   return TTT_MLP_OK;
 }
 

@@ -326,6 +326,22 @@ TTT_DEV float bf_lo(uint32_t u) { return __builtin_bit_cast(float, u << 16); }
 TTT_DEV float bf_hi(uint32_t u) { return __builtin_bit_cast(float, u & 0xffff0000u); }
 TTT_DEV float bf2f(bf16 x) { return (float)x; }
 
+// ---------------------------------------------------------------------------- stage clocks (instrumented builds only)
+#ifdef TTT_STAGE_CLOCKS
+#define TTT_STAGES_BEGIN() unsigned stage_acc[STAGE_SLOTS] = {}; unsigned stage_last = (unsigned)clock64()
+#define TTT_STAGE(i) do { const unsigned t_ = (unsigned)clock64(); stage_acc[i] += t_ - stage_last; stage_last = t_; } while (0)
+// `buf` = this workgroup's [8 waves][STAGE_SLOTS] part of the buffer
+#define TTT_STAGES_END(buf)                                                                                \
+  do {                                                                                                     \
+    if ((buf) != nullptr && (threadIdx.x & 63) == 0)                                                       \
+      for (int i_ = 0; i_ < STAGE_SLOTS; i_++) (buf)[(threadIdx.x >> 6) * STAGE_SLOTS + i_] = stage_acc[i_]; \
+  } while (0)
+#else
+#define TTT_STAGES_BEGIN() ((void)0)
+#define TTT_STAGE(i) ((void)0)
+#define TTT_STAGES_END(buf) ((void)0)
+#endif
+
 // ---------------------------------------------------------------------------- tanh-GELU family
 // gelu(x) = x * r with r = sigmoid(2c), c = K0 * x * (1 + K1 x^2); 1 - tanh(c)^2 = 4 r (1 - r).
 constexpr float GK0 = 0.79788456f;

@@ -281,6 +281,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
   int* const w_status = p.status;
   int* const s_flag = reinterpret_cast<int*>(smem + SM_FLAG);
 
+  TTT_STAGES_BEGIN();
   for (int mb = 0; mb < p.NC; mb++) {
     LANE_VARS;
     const bf16* s_xq = reinterpret_cast<const bf16*>(smem + SM_XQ + (mb & 1) * SM_TILE);
@@ -321,6 +322,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
       if (tid < FD) p.b2_ck[slot * FD + tid] = s_b2[tid];
     }
 
+    TTT_STAGE(FS_TOP);
     // ---- Z1 = XK W1 + b1 (rows tok, lane = hid);  X2 = gelu(Z1), D1 = gelu'(Z1)
     AccT<2, 1> x2, d1;
     {
@@ -344,6 +346,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
           d1.b[rb][0][i] = d;
         }
     }
+    TTT_STAGE(FS_F1_GELU);
     OpdT<1, 4> x2lo;                                        // lane = hid, contraction = tok: the low-order term, for the W2 step
     {
       LANE_VARS;
@@ -353,6 +356,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
     }
     TTT_WAVE_SYNC();
 
+    TTT_STAGE(FS_X2_SPLIT);
     // ---- Z2^T partial = W2s^T X2^T (rows F, lane = tok), summed over the pair into [tok][F]
     {
       LANE_VARS;
@@ -376,6 +380,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
       pair_sum_halves(s_Pp, [&]() { return z2_block(W2s.b[0][0]); }, [&]() { return z2_block(W2s.b[0][1]); }, pr, c, h);
     }
 
+    TTT_STAGE(FS_F2_PAIRSUM);
     // ---- LayerNorm-fused reconstruction-loss gradient: 8 tokens per wave, 8 lanes per token
     {
       LANE_VARS;
@@ -444,8 +449,10 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
       lds_put16(s_g2 + tok * FLD + f0, __builtin_bit_cast(u32x4, o));
       lds_put16(s_g2l + tok * FLD + f0, __builtin_bit_cast(u32x4, ol));
     }
+    TTT_STAGE(FS_LN);
     __syncthreads();
 
+    TTT_STAGE(FS_LN_BARRIER);
     // ---- G1 = (G2 W2^T) * gelu'(Z1);  state += X^T G
     {
       LANE_VARS;
@@ -493,6 +500,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
           }
         }
       }
+      TTT_STAGE(FS_F3);
       float colsum = 0.f;
 #pragma unroll
       for (int rb = 0; rb < 2; rb++)
@@ -517,6 +525,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
           }
         }
       }
+      TTT_STAGE(FS_F4);
       // W2[shard,:] += X2^T G2: X2 chained (two terms), G2 through the transposing read
       // (lane = F, contraction = tok; two terms); b2 += column sums of G2 (waves 0 and 1, rows 32v..32v+32)
       f32x16 b2acc;
@@ -557,6 +566,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
         }
       }
     }
+    TTT_STAGE(FS_F5);
     if constexpr (ROLE != 1) {
       LANE_VARS;
       if (h == 0) s_b1[hid0 + c] = b1L;      // read back below by this wave only
@@ -580,7 +590,9 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
 #pragma unroll
         for (int s = 0; s < 2; s++) g_st_stream<bf16x8>(gImg, 16 * tid, (4 + 2 * fb + s) * 8192, w2A.v[fb][s]);
       if (h == 0) gB[hid0 + c] = b1L;
+      TTT_STAGE(FS_HANDOVER);
       if (at == ring - 1 || mb == p.NC - 1) publish(w_given, grp + 1);
+      TTT_STAGE(FS_PUBLISH);
       continue;
     }
 
@@ -618,6 +630,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
       pair_sum_halves(s_Pp, [&]() { return z2_block(W2s.b[0][0]); }, [&]() { return z2_block(W2s.b[0][1]); }, pr, c, h);
     }
 
+    TTT_STAGE(FS_OUT_FORWARD);
     // ---- output LayerNorm + residual, 8 tokens per wave.  XK / XV / eta were last read before the pair sum
     //      above: the next mini-batch's leave HBM for LDS now.
     {
@@ -631,7 +644,9 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the next mini-batch's inputs have arrived in LDS
     __syncthreads();
+    TTT_STAGE(FS_OUT_LN);
   }
+  TTT_STAGES_END(p.stage_clocks == nullptr ? nullptr : p.stage_clocks + ((size_t)bh * 2 + 0) * (FW_NWAVE * STAGE_SLOTS));
 }
 
 // The output branch of the forward on its own workgroup: Out[mb] = XQ + LN(gelu(XQ W1' + b1') W2' + b2')
@@ -663,6 +678,7 @@ TTT_DEV void fwd_output_branch(const FwdParams& p, unsigned char* smem, const in
   int* const w_status = p.status;
   int* const s_flag = reinterpret_cast<int*>(smem + SM_FLAG);
 
+  TTT_STAGES_BEGIN();
   for (int mb = 0; mb < p.NC; mb++) {
     LANE_VARS;
     constexpr int ring = RING; const int grp = mb / ring, at = mb % ring, slot = (grp & 1) * ring + at;
@@ -684,6 +700,7 @@ TTT_DEV void fwd_output_branch(const FwdParams& p, unsigned char* smem, const in
       else if (tid < FWD_BIAS_FLOATS) s_b2[(mb & 1) * FD + tid - HID] = bv;
     }
     __syncthreads();   // XQ and the biases are visible; the previous mini-batch's readers of s_P are done
+    TTT_STAGE(FS_TOP);
     {
       LANE_VARS;
       OpdT<1, 4> w1A;
@@ -715,12 +732,16 @@ TTT_DEV void fwd_output_branch(const FwdParams& p, unsigned char* smem, const in
       mma(z2, w2A, x2bB);                          // rows F, lane = tok
       pair_sum_to_lds(s_Pp, z2, pr, c, h);
     }
+    TTT_STAGE(FS_OUT_FORWARD);
     {
       LANE_VARS;
       output_layernorm(s_P, s_b2 + (mb & 1) * FD, s_gam, s_bet, s_xq, gOut, mb, tok, f0);
     }
+    TTT_STAGE(FS_OUT_LN);
     if (at == ring - 1 || mb == p.NC - 1) publish(w_taken, grp + 1);
+    TTT_STAGE(FS_PUBLISH);
   }
+  TTT_STAGES_END(p.stage_clocks == nullptr ? nullptr : p.stage_clocks + ((size_t)bh * 2 + 1) * (FW_NWAVE * STAGE_SLOTS));
 #undef LANE_VARS
 }
 

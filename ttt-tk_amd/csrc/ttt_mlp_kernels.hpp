@@ -25,6 +25,9 @@ struct FwdParams {
   int* status;    // the status word behind the synchronisation words
   unsigned long long wait_limit;   // ticks of the 100 MHz clock a workgroup waits for another before it gives up
   int bh0, nbh;   // this launch covers (batch, head) pairs bh0 .. bh0 + nbh - 1
+#ifdef TTT_STAGE_CLOCKS
+  unsigned* stage_clocks;   // [B*NH][2 roles][8 waves][STAGE_SLOTS] or nullptr (see below)
+#endif
 };
 constexpr int FWD_RING_MAX = 32;               // most mini-batches per hand-over (8 or 32 are compiled)
 constexpr int FWD_IMG_BYTES = 64 * 256 * 2 * 2;  // W1 and W2 as bf16 operands
@@ -72,6 +75,9 @@ struct BwdParams {
   unsigned long long wait_limit;   // ticks of the 100 MHz clock a workgroup waits for another before it gives up
   int overwrite;  // non-zero: grad_L_XQ / XK / XV / last_eta are stored, not added to (every element is written exactly once)
   int bh0, nbh;   // this launch covers (batch, head) pairs bh0 .. bh0 + nbh - 1 (workspace pointers moved back by bh0 entries)
+#ifdef TTT_STAGE_CLOCKS
+  unsigned* stage_clocks;   // [B*NH][4 roles][8 waves][STAGE_SLOTS] or nullptr (see below)
+#endif
 };
 
 // Layout of `sync` (ints): 32 per (batch, head) - words 0 and 8 count the groups replayed by the first /
@@ -81,7 +87,63 @@ struct BwdParams {
 constexpr int BWD_SYNC_STRIDE = 32;
 inline size_t bwd_sync_ints(long long BH) { return (size_t)BH * BWD_SYNC_STRIDE + 32; }
 
+// ---- optional stage clocks.  A library built with -DTTT_STAGE_CLOCKS (stage_clocks.py builds one beside the product
+// library) reads the shader clock at the boundaries of the stages named here and adds up, per wave, the clocks
+// spent in each; every wave stores its sums when the kernel ends.  The product library
+// is built without the macro and contains none of this.  Reading the clock is a scalar-memory operation: every
+// boundary also waits for the wave's outstanding LDS reads, which makes an instrumented kernel some 10 % slower.
+// Slot of a workgroup in the buffer: forward 0 = the recurrence (or the one workgroup), 1 = the output branch;
+// backward 0 / 1 = the replaying workgroups, 2 = the reverse walk (or the one workgroup), 3 = unused.
+constexpr int STAGE_SLOTS = 24;
+enum FwdStage {
+  FS_TOP,            // barrier that opens the mini-batch, checkpoint store, wait for the other workgroup
+  FS_F1_GELU,        // Z1 = XK W1 + b1, GELU and its derivative
+  FS_X2_SPLIT,       // X2 in two terms, high-order term to LDS
+  FS_F2_PAIRSUM,     // Z2 = X2 W2 and its sum over the wave pairs (two barriers)
+  FS_LN,             // LayerNorm + loss gradient of 8 tokens per wave, G2 to LDS
+  FS_LN_BARRIER,     // barrier after it
+  FS_F3,             // G1 = (G2 W2^T) * GELU'(Z1), including the transposition of W2's terms through LDS
+  FS_F4,             // W1 step
+  FS_F5,             // W2 step and b2
+  FS_HANDOVER,       // recurrence workgroup: state images for the output branch
+  FS_PUBLISH,        // recurrence workgroup: counter for the output branch
+  FS_OUT_FORWARD,    // output branch: Z1_bar, GELU, Z2_bar and its pair sum
+  FS_OUT_LN,         // output branch: LayerNorm, residual, store; next inputs
+  FS_COUNT
+};
+enum BwdStage {
+  BS_GROUP,          // per checkpoint group: waits for the other workgroups, parking / loading of state and gradients
+  BS_R_TOP,          // replay: barrier that opens the mini-batch
+  BS_R_F1_GELU,      // replay: Z1, GELU family, images of Z1
+  BS_R_F2_PAIRSUM,   // replay: Z2 and its pair sum
+  BS_R_LN,           // replay: fused LayerNorm + loss gradient, saved tiles, barrier
+  BS_R_F3,           // replay: G1
+  BS_R_WSTEP,        // replay: W1 and W2 steps
+  BS_R_IMAGES,       // replay: operand images of the state after the step
+  BS_R_OUT_FORWARD,  // replay: output branch forward with its pair sum
+  BS_R_OUT_LN,       // replay: output LayerNorm forward and backward, next inputs, barrier
+  BS_R_OUT_BACKWARD, // replay: gZ1_bar, grad_L_XQ with its pair sum, images for the walk
+  BS_W_TOP,          // walk: tiles of the mini-batch into LDS (two barriers)
+  BS_W_BAR_TERMS,    // walk: what the output branch adds to the running gradients
+  BS_W_STEP_BACK,    // walk: the weight step backwards up to its pair sum
+  BS_W_PAIRSUM,      // walk: pair sum of it
+  BS_W_LN,           // walk: second-order pass through the fused LayerNorm loss
+  BS_W_LN_BARRIER,   // walk: barrier after it
+  BS_W_MLP_BACK,     // walk: inner MLP backwards (to the second wave-level fence)
+  BS_W_UPDATES,      // walk: updates of the running gradients
+  BS_W_DXK,          // walk: grad_L_XK with its pair sum (not with a grad_L_XK workgroup)
+  BS_PUBLISH,        // counters for the other workgroups
+  BS_COUNT
+};
+static_assert(FS_COUNT <= STAGE_SLOTS && BS_COUNT <= STAGE_SLOTS, "stage slots");
+
 }  // namespace ttt
+
+#ifdef TTT_STAGE_CLOCKS
+// Device buffers the next launches write their stage clocks to (nullptr: none): forward [B*NH][2][8][STAGE_SLOTS],
+// backward [B*NH][4][8][STAGE_SLOTS] unsigned ints, zero-filled by the caller.
+extern "C" void ttt_mlp_set_stage_clocks(unsigned* forward, unsigned* backward);
+#endif
 
 // p.sync == nullptr: one workgroup per (batch, head); otherwise two (state recurrence / output branch).
 hipError_t ttt_mlp_fwd_enqueue(const ttt::FwdParams& p, hipStream_t stream);
