@@ -853,6 +853,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         TTT_STAGE(BS_R_IMAGES);
         // post-update forward on XQ; X2_bar rows [tok][hid] -> T0, gelu'(Z1_bar) packed
         bf16x8 d1b[2][2];
+        bf16x8 gO_n;   // LayerNorm lanes: the upstream gradient of their 8 features, asked for a stage ahead
         {
           LANE_VARS;
           AccT<1, 2> z1b;
@@ -880,6 +881,10 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           mma_jit<2>(z2, [&](int rb, int s) { return piece_state(W2s, rb, s); },
                      [&](int i, int s) { return x2bQ[i][s]; });
           WAVE_SYNC();   // this wave's readers of T1 / T2 are done
+          {
+            LANE_VARS;
+            gO_n = g_ld_stream<bf16x8>(bGO, vln, mb * TILE_BYTES);   // under way during the pair sum
+          }
           pair_sum(s_own, s_partner, z2, c, h);
         }
         TTT_STAGE(BS_R_OUT_FORWARD);
@@ -906,7 +911,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
 #pragma unroll
             for (int e = 0; e < 8; e++) z[e] += b2v[e];
           }
-          ln_cvt8(gO, g_ld_stream<bf16x8>(bGO, vln, mb * TILE_BYTES));
+          ln_cvt8(gO, gO_n);
           float sd;
           ln_normalize(z, &sd);   // z = x_hat
           ln_load_f32(gam, s_gam + f0);
@@ -1068,6 +1073,11 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
               aq[i][t] = chunk_load(bDD, j * (2 * IMG_BYTES), 2 * tb[i] + t, t16);   // read again two stages on
               bq[i][t] = image_load<true>(bDD, j * (2 * IMG_BYTES) + IMG_BYTES, 2 * tb[i] + t, t16);
             }
+        } else {               // the image of Z1 (gq takes it), from which the next stage evaluates the three
+#pragma unroll
+          for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int t = 0; t < 2; t++) gq[i][t] = image_load<ROLE != 0>(bZ1, ho, 2 * tb[i] + t, t16);
         }
         mma_jit<4>(gW2s, [&](int, int s) { return x2b[s]; },                                   // X2_bar^T: lane = hid
                    [&](int fb, int s) { return piece_tr<LDX>(s_a, fb, s, lane); });            // gZ2_bar: lane = F
@@ -1111,7 +1121,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           // fetched as three images that a replaying workgroup computed the same way
           bf16x8 ac[2], bc[2];
           if constexpr (!IMG) {
-            const bf16x8 zc[2] = {image_load<ROLE != 0>(bZ1, ho, 2 * tb[i], t16), image_load<ROLE != 0>(bZ1, ho, 2 * tb[i] + 1, t16)};
+            const bf16x8 zc[2] = {gq[i][0], gq[i][1]};
 #pragma unroll
             for (int t = 0; t < 2; t++)
 #pragma unroll
