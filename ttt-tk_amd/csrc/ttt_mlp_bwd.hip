@@ -221,21 +221,21 @@ TTT_DEV float ln_normalize(float (&z)[8], float* std_out) {
   *std_out = v * rstd;  // sqrt(v)
   return rstd;
 }
-// Sum over the 8 lanes of a wave that share lane % 8 (the 8 tokens of a LayerNorm stage), result in
-// all of them: a rotation by 8 inside each row of 16 lanes, then across the four rows.
-TTT_DEV float token_sum8(float x) {
-  x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x128, 0xF, 0xF, false));  // row_ror:8
-  return half_sum_valu(row_pair_sum(x));
-}
-// acc[f0 + e] += sum over this wave's tokens of x[e]   (wave-private LDS vector)
-TTT_DEV void ln_token_sum_add(float* s_acc, const float (&x)[8], int q8, int f0) {
-  f32x4 a, b;
+// acc[f0 + e] += sum over this wave's tokens of x[e]   (wave-private LDS vector).  The 8 tokens sit in the lanes
+// that share lane % 8: lanes 8 apart inside a row of 16 (one rotation), then the four rows, two values per swap
+// (row_pair_sum2, half_sum2): in the end row r of one register holds the total of x[r], of the other that of
+// x[4 + r], and lanes 0..7 of every row add their two totals to the vector.
+TTT_DEV void ln_token_sum_add(float* s_acc, const float (&x)[8], int lane, int f0) {
+  float y[8];
 #pragma unroll
-  for (int e = 0; e < 4; e++) { a[e] = token_sum8(x[e]); b[e] = token_sum8(x[4 + e]); }
-  if (q8 == 0) {
-    f32x4* d = reinterpret_cast<f32x4*>(s_acc + f0);
-    d[0] = d[0] + a;
-    d[1] = d[1] + b;
+  for (int e = 0; e < 8; e++)
+    y[e] = x[e] + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x[e]), 0x128, 0xF, 0xF, false));  // row_ror:8
+  const float lo = half_sum2(row_pair_sum2(y[0], y[1]), row_pair_sum2(y[2], y[3]));
+  const float hi = half_sum2(row_pair_sum2(y[4], y[5]), row_pair_sum2(y[6], y[7]));
+  if ((lane & 8) == 0) {
+    float* d = s_acc + f0 + (lane >> 4);
+    d[0] += lo;
+    d[4] += hi;
   }
 }
 
@@ -917,8 +917,8 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           ln_load_f32(gam, s_gam + f0);
 #pragma unroll
           for (int e = 0; e < 8; e++) gx[e] = gO[e] * z[e];
-          ln_token_sum_add(s_dbw, gO, q8, f0);
-          ln_token_sum_add(s_dgw, gx, q8, f0);
+          ln_token_sum_add(s_dbw, gO, lane, f0);
+          ln_token_sum_add(s_dgw, gx, lane, f0);
 #pragma unroll
           for (int e = 0; e < 8; e++) gx[e] = gO[e] * gam[e];
           const float s1 = oct_sum(sum8(gx)), s2 = oct_sum(dot8(gx, z));
@@ -1244,8 +1244,8 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         sg = oct_sum(sg);
         sx = oct_sum(sx);
         if constexpr (!FIN) {   // with a grad_L_XK workgroup these token sums and grad_L_XV are formed there, from g_y and dg
-          ln_token_sum_add(s_dgw, dg, q8, f0);
-          ln_token_sum_add(s_dbw, gy, q8, f0);
+          ln_token_sum_add(s_dgw, dg, lane, f0);
+          ln_token_sum_add(s_dbw, gy, lane, f0);
         }
 #pragma unroll
         for (int e = 0; e < 8; e++) {
@@ -1588,8 +1588,8 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
       }
       g_st_stream<bf16x8>(gDXK, vln, xo, dxk_new);
       g_st_stream<bf16x8>(gDXV, vln, xo, dxv_new);
-      ln_token_sum_add(s_dgw, dgv, q8, f0);
-      ln_token_sum_add(s_dbw, gyv, q8, f0);
+      ln_token_sum_add(s_dgw, dgv, lane, f0);
+      ln_token_sum_add(s_dbw, gyv, lane, f0);
       __syncthreads();   // the readers of the pair sums are done before the next mini-batch's take their place
     }
     publish(w_finished, done + 1);

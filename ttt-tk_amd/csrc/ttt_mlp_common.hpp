@@ -118,6 +118,21 @@ TTT_DEV float row_pair_sum(float x) {
   return a + b;
 }
 
+// The same two sums for two values at once.  After v_permlane16_swap of (x0, x1) one register holds rows
+// (x0.r0, x1.r0, x0.r2, x1.r2) and the other (x0.r1, x1.r1, x0.r3, x1.r3), so their sum carries x0's row-pair sums in
+// the even rows and x1's in the odd rows; v_permlane32_swap of two such sums leaves, after the add, the totals over
+// the four rows: of the first sum's two values in rows 0 and 1, of the second's in rows 2 and 3.
+TTT_DEV float row_pair_sum2(float x0, float x1) {
+  float a = x0, b = x1;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return a + b;
+}
+TTT_DEV float half_sum2(float s01, float s23) {
+  float a = s01, b = s23;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return a + b;
+}
+
 // ---------------------------------------------------------------------------- shape-generic tiles
 // Tiles whose extent along the hidden dimension is one 32-wide block (a wave that owns 32 hidden
 // columns) mix with 64-wide token / feature extents, so blocks and k-steps are template parameters.
