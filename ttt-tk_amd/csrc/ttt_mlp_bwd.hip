@@ -894,6 +894,11 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         bf16x8 dxq_old;
         {
           LANE_VARS;
+          // The upstream gradient is taken out of its load registers before the loads below are issued: they are
+          // issued under a condition, so a wait for an older load placed after them has to be a wait for all of them.
+          ln_cvt8(gO, gO_n);
+#pragma unroll
+          for (int e = 0; e < 8; e++) asm volatile("" : "+v"(gO[e]));
           // Every reader of this mini-batch's XQ / XK / XV / eta is past the barriers of the pair sum: the next
           // mini-batch's leave HBM now - straight to LDS, no registers involved - and have the rest of this
           // mini-batch to arrive.
@@ -911,7 +916,6 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
 #pragma unroll
             for (int e = 0; e < 8; e++) z[e] += b2v[e];
           }
-          ln_cvt8(gO, gO_n);
           float sd;
           ln_normalize(z, &sd);   // z = x_hat
           ln_load_f32(gam, s_gam + f0);
