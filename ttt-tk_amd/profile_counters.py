@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """rocprofv3 counter harness for the TTT-MLP kernels: one JSON per workload under profiles/.
 
-    python ttt-tk_amd/profile_counters.py --workload c4 [--workload c5 ...] [--raw gpurun_out/counters]
+    python ttt-tk_amd/profile_counters.py --workload c4 [--workload c5 ...] [--raw DIR] [--out DIR]
 
 For each workload it runs `python3 bench.py --workload W ...` under rocprofv3 five times, each pass a run of its own
 (counters are never combined with tracing options other than the kernel trace):
@@ -37,6 +37,7 @@ import os
 import signal
 import subprocess
 import sys
+import tempfile
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
@@ -174,7 +175,7 @@ def profile(workload: str, raw_dir: str, limit_s: int):
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--workload", action="append", choices=["c2", "c3", "c4", "c5"])
-    ap.add_argument("--raw", default=os.path.join(ROOT, "gpurun_out", "counters"), help="where rocprofv3 writes its CSVs")
+    ap.add_argument("--raw", default=os.path.join(tempfile.gettempdir(), "ttt_mlp_counters"), help="where rocprofv3 writes its CSVs")
     ap.add_argument("--out", default=os.path.join(ROOT, "profiles"))
     ap.add_argument("--limit", type=int, default=170, help="seconds allowed per rocprofv3 pass")
     a = ap.parse_args()
