@@ -184,7 +184,7 @@ def main():
         one, rest, per = ctypes.c_longlong(), ctypes.c_longlong(), ctypes.c_int()
         cus = torch.cuda.get_device_properties(dev).multi_processor_count
         lib.ttt_mlp_launch_plan(1, ctypes.c_longlong(B * NH), cus, ctypes.byref(one), ctypes.byref(rest), ctypes.byref(per))
-        bwd_kernel = f"ttt_mlp_bwd_split_kernel<{2 if per.value >= 3 else 1}, {'true' if per.value == 4 else 'false'}>"
+        bwd_kernel = f"ttt_mlp_bwd_split_kernel<{2 if per.value >= 3 else 1}, {'true' if per.value >= 4 else 'false'}>"
         if one.value:
             bwd_kernel = "ttt_mlp_bwd_kernel + " + bwd_kernel
     out = {

@@ -218,7 +218,8 @@ const char* ttt_mlp_error_string(int code);
 /* How an overlapped launch of `pairs` = B*NH (batch, head) pairs is laid out on a device with
  * `compute_units` CUs (no device needed): the first *one_workgroup_pairs pairs run with one workgroup each,
  * the remaining *other_pairs with *workgroups_per_other_pair each (0 if there are none).  which = 0
- * forward, 1 backward. */
+ * forward (1 or 2 per pair), 1 backward (1 to 5: one or two that replay the checkpoint groups, one that walks
+ * them backwards, one for grad_L_XK / grad_L_XV, one that fetches the walk's operands into the L2 ahead of it). */
 int ttt_mlp_launch_plan(int which, long long pairs, int compute_units, long long* one_workgroup_pairs,
                         long long* other_pairs, int* workgroups_per_other_pair);
 

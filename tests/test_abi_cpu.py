@@ -186,12 +186,15 @@ def test_launch_plan_keeps_waiting_workgroups_within_the_device(lib):
         a, b, c = ctypes.c_longlong(), ctypes.c_longlong(), ctypes.c_int()
         assert lib.ttt_mlp_launch_plan(which, ctypes.c_longlong(pairs), cus, ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)) == 0
         return a.value, b.value, c.value
-    assert plan(1, 48, 256) == (0, 48, 4)          # the metric's configuration: four workgroups per pair
+    assert plan(1, 48, 256) == (0, 48, 5)          # the metric's configuration: four workgroups per pair + one that fetches ahead
+    assert plan(1, 56, 256) == (0, 56, 4)          # a fifth would not fit
+    assert plan(1, 44, 256) == (0, 44, 4)          # not a multiple of 8 pairs: the fifth would not share the walk's XCD
     assert plan(1, 72, 256) == (0, 72, 3)
     assert plan(1, 96, 256) == (0, 96, 2)
     assert plan(1, 200, 256) == (200, 0, 0)        # two per pair would not fit: one each
     assert plan(1, 384, 256) == (256, 128, 2)      # one full round, the rest with two each
     assert plan(1, 260, 256) == (256, 4, 4)
+    assert plan(1, 264, 256) == (256, 8, 5)
     assert plan(1, 512, 256) == (512, 0, 0)
     assert plan(0, 48, 256) == (0, 48, 2)          # forward: two per pair at most
     assert plan(0, 384, 256) == (256, 128, 2)
@@ -205,7 +208,7 @@ def test_launch_plan_keeps_waiting_workgroups_within_the_device(lib):
                 one, rest, per = plan(which, pairs, cus)
                 assert one + rest == pairs and one % cus == 0 or rest == 0
                 assert rest * per <= cus
-                assert per in ((0, 2) if which == 0 else (0, 2, 3, 4))
+                assert per in ((0, 2) if which == 0 else (0, 2, 3, 4, 5))
     assert lib.ttt_mlp_launch_plan(2, ctypes.c_longlong(1), 1, None, None, None) == 1001
 
 

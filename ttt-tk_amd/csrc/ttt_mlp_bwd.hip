@@ -1027,6 +1027,9 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
     if constexpr (ROLE != 1)
     for (int j = n_mb - 1; j >= 0; j--) {
       const int mb = k * cgs + j;
+      if constexpr (ROLE == 2 && FIN) {   // how far the walk is, for the workgroup that fetches ahead of it
+        if (threadIdx.x == 0) __hip_atomic_store(w_sync + 20, p.NC - mb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
       REFRESH_OFFSETS();
       LANE_VARS;
       const unsigned xo = mb * TILE_BYTES;       // this mini-batch in the input / output tensors
@@ -1616,13 +1619,71 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
   }
 }
 
+// ------------------------------------------------------------------ the workgroup that fetches ahead of the walk
+// The walk asks per mini-batch for 240 KiB that a replaying workgroup wrote a checkpoint group earlier (six register
+// images, four tiles) or that the caller passed in (two tiles): none of it is in the L2 by then, and one CU cannot
+// keep enough requests in flight to hide the way to HBM.  This workgroup computes nothing: it goes through the walk's
+// mini-batches in the walk's order, PREFETCH_AHEAD of them ahead of it, and reads one dword of every 128-byte line
+// the walk will ask for.  Placed on the walk's XCD, it leaves the lines in the L2 that the walk's requests go to.
+// Purely a hint: the values are dropped, nothing is written except the status word of a wait that gives up, and
+// the walk's results do not depend on whether, when or where this workgroup runs.
+constexpr int PREFETCH_AHEAD = 1;
+TTT_DEV void bwd_prefetch(const BwdParams& p, unsigned char* smem, const int bh) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int v = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int cgs = p.cgs, n_replay = p.n_replay, n_sets = 2 * n_replay;
+  int* const w_sync = p.sync + (size_t)bh * BWD_SYNC_STRIDE;
+  int* const w_step = w_sync + 20;
+  int* const s_flag = reinterpret_cast<int*>(smem + SB_FLAG);
+  const size_t ox = uni64((size_t)bh * p.NC * (CS * FD)), of = uni64((size_t)bh * cgs * (CS * FD));
+  const size_t oh = uni64((size_t)bh * cgs * (CS * HID)), opk = uni64((size_t)bh * cgs * (FD * HID));
+  const unsigned line_t = 128u * lane, line_i = 128u * (tid & 255);   // this thread's line of a tile / of an image
+  int n = 0;   // mini-batches the walk has before the one at hand
+  for (int k = p.K - 1; k >= 0; k--) {
+    const int n_mb = min(cgs, p.NC - k * cgs);
+    const int done = p.K - 1 - k, set = done % n_sets;
+    // the group has been replayed: what is fetched is what the walk will read
+    if (!wait_at_least(w_sync + 8 * (done % n_replay), done / n_replay + 1, p.status, s_flag, p.wait_limit)) return;
+#define PGRP(name) (set ? p.alt_##name[set - 1] : p.name)
+    // wave v fetches tile v (v < 6): the two inputs (indexed by the mini-batch's place in the sequence), then four of the set
+    gptr_t tile = gbuf(p.XQ + ox);
+    unsigned tile0 = k * cgs * TILE_BYTES;
+    if (v == 1) tile = gbuf(p.XK + ox);
+    if (v >= 2) tile0 = 0;
+    if (v == 2) tile = gbuf(PGRP(grad_l_wrt_Z2_group) + of);
+    if (v == 3) tile = gbuf(PGRP(grad_x_hat_fused_group) + of);
+    if (v == 4) tile = gbuf(PGRP(x_hat_fused_group) + of);
+    if (v >= 5) tile = gbuf(PGRP(grad_output_fused_group) + of);
+    // and half of three of the six images: waves 0-3 X2_bar, GELU, GELU''; waves 4-7 gZ1_bar, GELU', W2 before the step
+    const bool up = v >= 4;
+    const gptr_t img0 = up ? gbuf(PGRP(Z1_bar_group) + oh) : gbuf(PGRP(X2_bar_group) + oh);
+    const gptr_t img1 = up ? gbuf(PGRP(W1_init_group) + opk) : gbuf(PGRP(Z1_group) + oh);
+    const gptr_t img2 = up ? gbuf(PGRP(grad_l_wrt_Z1_group) + oh) : gbuf(PGRP(W1_init_group) + opk);
+#undef PGRP
+    for (int j = n_mb - 1; j >= 0; j--, n++) {
+      const int seen = wait_for_pace(w_step, n + 1 - PREFETCH_AHEAD, p.status, s_flag, p.wait_limit);
+      if (seen == 0) return;
+      if (seen - 1 > n + 1) continue;   // the walk is past this mini-batch already
+      const unsigned ho = j * IMG_BYTES;
+      unsigned got[4] = {0, 0, 0, 0};
+      if (v < 6) got[0] = g_ld<unsigned>(tile, line_t, tile0 + j * TILE_BYTES);
+      got[1] = g_ld<unsigned>(img0, line_i, ho);
+      got[2] = g_ld<unsigned>(img1, line_i, up ? 2 * ho : ho);
+      if (!up) got[3] = g_ld<unsigned>(img2, line_i, 2 * ho + IMG_BYTES);
+      else if (j > 0) got[3] = g_ld<unsigned>(img2, line_i, ho - IMG_BYTES);
+#pragma unroll
+      for (int i = 0; i < 4; i++) asm volatile("" ::"v"(got[i]));   // landed; nothing is done with them
+    }
+  }
+}
+
 // n_replay + 1 (+ 1) workgroups per (batch, head).  Workgroups are dealt to the 8 XCDs in turn, so with a
 // multiple of 8 (batch, head) pairs the workgroups of a pair are placed 8 apart: same XCD, same L2.
 // One kernel per combination, so that each holds only the code (and the register allocation) of its own roles.
 template <int NREPLAY, bool FINISH>
 __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_split_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int b = blockIdx.x, per = NREPLAY + 1 + (FINISH ? 1 : 0);
+  const int b = blockIdx.x, per = NREPLAY + 1 + (FINISH ? 1 + p.n_prefetch : 0);
   int bh, role;
   if (p.nbh % 8 == 0) {
     bh = (b / (8 * per)) * 8 + (b & 7);
@@ -1635,7 +1696,10 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_split_kernel(const Bwd
   constexpr bool IMG = NREPLAY == 2;   // two replaying workgroups also evaluate the GELU family for the walk
   if (role < NREPLAY) bwd_body<1, IMG, FINISH>(p, smem, bh, role);
   else if (role == NREPLAY) bwd_body<2, IMG, FINISH>(p, smem, bh, 0);
-  else if constexpr (FINISH) bwd_finish_dxk(p, smem, bh);
+  else if constexpr (FINISH) {
+    if (role == NREPLAY + 1) bwd_finish_dxk(p, smem, bh);
+    else bwd_prefetch(p, smem, bh);
+  }
 }
 
 __global__ void ttt_mlp_zero_words(int* w, int n) {
@@ -1659,7 +1723,7 @@ hipError_t ttt_mlp_bwd_enqueue(const ttt::BwdParams& p, hipStream_t stream) {
   const int n = static_cast<int>(ttt::bwd_sync_ints(p.nbh));
   int* const words = p.status - (size_t)p.nbh * ttt::BWD_SYNC_STRIDE;   // p.sync itself is moved back by bh0 entries
   hipLaunchKernelGGL(ttt::ttt_mlp_zero_words, dim3((n + 255) / 256), dim3(256), 0, stream, words, n);
-  const dim3 grid((p.n_replay + 1 + p.n_finish) * p.nbh), block(ttt::BW_THREADS);
+  const dim3 grid((p.n_replay + 1 + p.n_finish + p.n_prefetch) * p.nbh), block(ttt::BW_THREADS);
   auto launch = [&](auto kernel) -> hipError_t {
     hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, ttt::SM_BWD_BYTES);
     if (err != hipSuccess) return err;

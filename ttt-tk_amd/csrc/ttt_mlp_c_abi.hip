@@ -146,6 +146,7 @@ struct LaunchPlan {
   long long n_rest = 0;     // pairs n_single .. n_single+n_rest-1
   bool rest_split = false;
   int per_pair = 1;         // workgroups per pair of the rest: 2, or 3 / 4 where the kernel can use them and they fit
+  bool prefetch = false;    // backward with 4 per pair: a fifth that fetches ahead of the walk
 };
 // `three_way`: the backward can use three or four workgroups per pair, the forward two.
 LaunchPlan plan_for(long long BH, int cus, bool three_way) {
@@ -159,6 +160,8 @@ LaunchPlan plan_for(long long BH, int cus, bool three_way) {
   pl.rest_split = pl.n_rest > 0 && 2 * pl.n_rest <= cus;
   if (!pl.rest_split) { pl.n_single = BH; pl.n_rest = 0; }
   else pl.per_pair = !three_way ? 2 : 4 * pl.n_rest <= cus ? 4 : 3 * pl.n_rest <= cus ? 3 : 2;
+  // the fifth workgroup helps only from the walk's own XCD, which the kernel arranges for a multiple of 8 pairs
+  pl.prefetch = pl.per_pair == 4 && 5 * pl.n_rest <= cus && pl.n_rest % 8 == 0;
   return pl;
 }
 LaunchPlan plan_launches(long long BH, bool three_way) {
@@ -279,6 +282,7 @@ extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* wo
   p.nbh = static_cast<int>(pl.n_rest);
   p.n_replay = n_replay;
   p.n_finish = finish ? 1 : 0;
+  p.n_prefetch = pl.prefetch ? 1 : 0;
   p.wait_limit = g_wait_limit;
   if (finish) {
     p.fin_dz = reinterpret_cast<__bf16*>(base + w.off[6]) - b0 * 2 * img;
@@ -431,7 +435,7 @@ extern "C" int ttt_mlp_launch_plan(int which, long long pairs, int compute_units
   const LaunchPlan pl = plan_for(pairs, compute_units, which == 1);
   *one_workgroup_pairs = pl.n_single;
   *other_pairs = pl.n_rest;
-  *workgroups_per_other_pair = pl.n_rest > 0 ? pl.per_pair : 0;
+  *workgroups_per_other_pair = pl.n_rest > 0 ? pl.per_pair + (pl.prefetch ? 1 : 0) : 0;
   return TTT_MLP_OK;
 }
 

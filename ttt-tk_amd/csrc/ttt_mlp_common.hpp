@@ -448,6 +448,26 @@ TTT_DEV bool wait_at_least(int* word, int target, int* status, int* s_flag, uint
   __syncthreads();
   return *s_flag != 0;
 }
+// Pacing only: waits until `word` has reached `target` without ordering any data after it (no fence, so nothing in
+// the caches is invalidated).  Returns 0 if the wait gave up (as above), otherwise the value seen + 1.
+TTT_DEV int wait_for_pace(int* word, int target, int* status, int* s_flag, uint64_t limit) {
+  __syncthreads();   // the last value of the flag has been read by every wave
+  if (threadIdx.x == 0) {
+    int seen;
+    const uint64_t t0 = wall_clock64();
+    while ((seen = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) < target) {
+      if (__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 || wall_clock64() - t0 > limit) {
+        __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        seen = -1;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(8);
+    }
+    *s_flag = seen + 1;
+  }
+  __syncthreads();
+  return *s_flag;
+}
 // Everything this workgroup has written (or read) so far is ordered before the new value of `word`: every
 // wave drains its own outstanding memory operations (a workgroup-scope release alone does not wait for
 // stores that are still in flight), the barrier collects the waves, then one thread writes the L2 back at

@@ -70,6 +70,10 @@ struct BwdParams {
   __bf16* fin_dz;
   float* fin_gy;
   int n_finish;
+  // n_prefetch = 1 (with n_finish = 1 only): one more workgroup reads nothing for itself; it touches every cache
+  // line that the walk is about to ask for, one mini-batch ahead of it, so that the walk's own requests are
+  // answered by the L2 the two share instead of by HBM.
+  int n_prefetch;
   int* sync;
   int* status;    // the status word behind the synchronisation words
   unsigned long long wait_limit;   // ticks of the 100 MHz clock a workgroup waits for another before it gives up
@@ -82,7 +86,8 @@ struct BwdParams {
 
 // Layout of `sync` (ints): 32 per (batch, head) - words 0 and 8 count the groups replayed by the first /
 // second replaying workgroup (norm_partial is written before the last count), word 16 the groups the
-// reverse walk has finished, word 24 the groups the grad_L_XK workgroup has finished - then one status
+// reverse walk has finished, word 20 the mini-batches it has started (a pacing hint for the prefetching workgroup,
+// no data is ordered by it), word 24 the groups the grad_L_XK workgroup has finished - then one status
 // word (non-zero: a wait gave up).
 constexpr int BWD_SYNC_STRIDE = 32;
 inline size_t bwd_sync_ints(long long BH) { return (size_t)BH * BWD_SYNC_STRIDE + 32; }
