@@ -31,7 +31,8 @@ def _args(order, t, cgs, B, NH, NC, K):
     return Args(*[t[k].data_ptr() for k in order], cgs, B, NH, NC, K)
 
 
-@pytest.mark.parametrize("B,NH,NC,cgs", [(1, 2, 1, 1), (1, 3, 5, 8), (2, 2, 17, 4)])
+# 8 pairs: the backward runs with a fifth workgroup per pair that fetches ahead of the walk (a multiple of 8 pairs)
+@pytest.mark.parametrize("B,NH,NC,cgs", [(1, 2, 1, 1), (1, 3, 5, 8), (2, 2, 17, 4), (1, 8, 13, 4), (2, 4, 3, 8)])
 def test_overlapped_launchers_through_ctypes(B, NH, NC, cgs):
     print(f"case B={B} NH={NH} NC={NC} cgs={cgs}", flush=True)
     import ttt_mlp_host as host
@@ -76,14 +77,16 @@ def test_overlapped_launchers_through_ctypes(B, NH, NC, cgs):
         assert torch.equal(results[0][k], results[1][k]), k
 
 
-def test_a_wait_that_gives_up_is_reported_and_every_wave_exits():
+@pytest.mark.parametrize("NH", [2, 8])   # 8 pairs: with the workgroup that fetches ahead of the walk
+def test_a_wait_that_gives_up_is_reported_and_every_wave_exits(NH):
     """Forced from the host: with a wait limit of one clock tick the first workgroup that has to wait for its
     partner gives up at once, raises the status word, and all workgroups of the launch leave.  The operator
     (which synchronises by default) reports it; with the default limit the same call then succeeds."""
     import ttt_mlp_host as host
     import test_time_training as ext
     dev = torch.device("cuda:0")
-    B, NH, NC, cgs = 1, 2, 24, 4
+    B, NC, cgs = 1, 24, 4
+    print(f"case B={B} NH={NH} NC={NC} cgs={cgs}", flush=True)
     d = orc.make_inputs(B, NH, NC, seed=41)
     t = {k: d[k].to(dev).contiguous() for k in FWD_KEYS + UP_KEYS}
     t.update(host.alloc_forward_buffers(B, NH, NC, cgs, dev))

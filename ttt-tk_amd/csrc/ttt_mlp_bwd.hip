@@ -1037,6 +1037,9 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
       const unsigned ho = j * IMG_BYTES;         // its slot in the [cgs][64][256] scratch tensors
       // eta of the token this lane holds in column block i of a Q-orientation tile
       const float eta_i[2] = {bf2f(g_ldh(bETA, 2 * c, mb * (CS * 2) + 64 * tb[0])), bf2f(g_ldh(bETA, 2 * c, mb * (CS * 2) + 64 * tb[1]))};
+      // What the output branch adds to the running gradients: the replay has taken that branch backwards already
+      // and left gZ2_bar (a tile, to LDS here) and X2_bar^T, gZ1_bar^T as operand images.
+      bf16x8 x2b[4], g1b[4];   // lane = hid, contraction = tok
       {
         LANE_VARS;
         constexpr bool ST = ROLE != 0;   // tiles another workgroup left here are read once
@@ -1044,23 +1047,18 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         const u32x4 gz = ST ? g_ld_stream<u32x4>(bGZ2, t16, so) : g_ld16(bGZ2, t16, so);
         const u32x4 gzb = ST ? g_ld_stream<u32x4>(bGZB, t16, so) : g_ld16(bGZB, t16, so);
         const float eta = bf2f(g_ldh(bETA, 2 * (tid & (CS - 1)), mb * (CS * 2)));
+        // the two operand images of the next stage are asked for behind the tiles: on their way across both barriers
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+          x2b[s] = image_load<ROLE != 0>(bX2B, ho, s, t16);
+          g1b[s] = image_load<ROLE != 0>(bGZ1B, ho, s, t16);
+        }
         __syncthreads();   // the previous mini-batch's readers of these tiles are done (the loads are under way)
         lds_put16x(s_xq, tid, xq);
         lds_put16x(s_xk, tid, xk);
         lds_put16(s_gz2, tid, gz);
         lds_put16(s_a, tid, gzb);
         if (tid < CS) s_eta[tid] = eta;
-      }
-      // ---- what the output branch adds to the running gradients.  The replay has taken that branch
-      //      backwards already and left gZ2_bar (now in LDS) and X2_bar^T, gZ1_bar^T as operand images.
-      bf16x8 x2b[4], g1b[4];   // lane = hid, contraction = tok; under way across the barrier
-      {
-        LANE_VARS;
-#pragma unroll
-        for (int s = 0; s < 4; s++) {
-          x2b[s] = image_load<ROLE != 0>(bX2B, ho, s, t16);
-          g1b[s] = image_load<ROLE != 0>(bGZ1B, ho, s, t16);
-        }
       }
       __syncthreads();
 
@@ -1501,10 +1499,12 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
   float* s_dgw = s_red + (v * 2 + 0) * FD;
   float* s_dbw = s_red + (v * 2 + 1) * FD;
   if (lane < FD) { s_dgw[lane] = 0.f; s_dbw[lane] = 0.f; }
+  TTT_STAGES_BEGIN();
   for (int k = p.K - 1; k >= 0; k--) {
     const int n_mb = min(cgs, p.NC - k * cgs);
     const int done = p.K - 1 - k, set = done % n_sets;
     if (!wait_at_least(w_walked, done + 1, p.status, s_flag, p.wait_limit)) return;
+    TTT_STAGE(BS_X_GROUP);
     const size_t ofin = uni64(((size_t)bh * 2 + (done & 1)) * cgs);
     const size_t o_img = uni64((size_t)bh * cgs * (CS * HID)), o_tile = uni64((size_t)bh * cgs * (CS * FD));
     const gptr_t gIMG2 = gbuf((set ? p.alt_grad_l_wrt_Z1_group[set - 1] : p.grad_l_wrt_Z1_group) + o_img);   // W2 after each step
@@ -1582,6 +1582,7 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
       mma_jit<4>(gW1s, [&](int fb, int s) { return xpiece_tr(s_xk, fb, s, lane); },         // + XK^T dZ1
                  [&](int, int s) { return piece_tr<LDH>(T1, 0, s, lane); });
       WAVE_SYNC();   // this wave's readers of T1 / T2 are done
+      TTT_STAGE(BS_X_PRODUCTS);
       pair_sum(s_own, s_partner, dk, c, h);
       float z[8];
       ln_gather(z, s_lnrow);
@@ -1598,9 +1599,12 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
       ln_token_sum_add(s_dgw, dgv, lane, f0);
       ln_token_sum_add(s_dbw, gyv, lane, f0);
       __syncthreads();   // the readers of the pair sums are done before the next mini-batch's take their place
+      TTT_STAGE(BS_X_SUMS);
     }
     publish(w_finished, done + 1);
+    TTT_STAGE(BS_PUBLISH);
   }
+  TTT_STAGES_END(p.stage_clocks == nullptr ? nullptr : p.stage_clocks + ((size_t)bh * 4 + 3) * (BW_NWAVE * STAGE_SLOTS));
   // norm-weight / norm-bias gradients: the replaying workgroups' two sums (handed over before their last counts,
   // which the walk had acquired before its own last count) + the walk's, in the order of the other launch shapes
   __syncthreads();

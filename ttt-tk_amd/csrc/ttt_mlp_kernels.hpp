@@ -138,6 +138,9 @@ enum BwdStage {
   BS_W_UPDATES,      // walk: updates of the running gradients
   BS_W_DXK,          // walk: grad_L_XK with its pair sum (not with a grad_L_XK workgroup)
   BS_PUBLISH,        // counters for the other workgroups
+  BS_X_GROUP,        // grad_L_XK workgroup, per checkpoint group: waits for the walk to have finished the group
+  BS_X_PRODUCTS,     // grad_L_XK workgroup: operands of the mini-batch from HBM, G1 and the products, to the pair sum
+  BS_X_SUMS,         // grad_L_XK workgroup: pair sum, grad_L_XK / grad_L_XV, token sums of the norm gradients, barrier
   BS_COUNT
 };
 static_assert(FS_COUNT <= STAGE_SLOTS && BS_COUNT <= STAGE_SLOTS, "stage slots");

@@ -172,6 +172,9 @@ def main() -> int:
         mb0 = NC - (K - groups0) * cgs if n_rep == 1 else sum(min(cgs, NC - (K - 1 - g) * cgs) for g in range(0, K, 2))
         out += table(f"backward, replaying workgroup 0 of {n_rep} ({int(has_r0.sum())} pairs, {mb0} of the {NC} mini-batches)", r0[has_r0], bwd_names, mb0) + [""]
         out += table(f"backward, reverse-walk workgroup ({int(has_r0.sum())} pairs)", walk[has_r0], bwd_names, NC) + [""]
+        fin = cb[:, 3]
+        if (fin.sum(dim=(1, 2)) > 0).any():
+            out += table(f"backward, grad_L_XK workgroup ({int((fin.sum(dim=(1, 2)) > 0).sum())} pairs)", present(fin), bwd_names, NC) + [""]
     text = "\n".join(out)
     print(text)
     if a.out:
