@@ -136,12 +136,13 @@ int ttt_mlp_fwd_launch(const ttt_mlp_fwd_args* args, void* stream);
 /* Same for the remat backward. */
 int ttt_mlp_bwd_launch(const ttt_mlp_bwd_args* args, void* stream);
 
-/* The same backward (bit-identical results) with two to four workgroups per
+/* The same backward (bit-identical results) with two to five workgroups per
  * (batch, head) where the device has CUs to spare: one or two recompute checkpoint
- * group after checkpoint group, one walks each recomputed group backwards, and a
+ * group after checkpoint group, one walks each recomputed group backwards, a
  * fourth forms grad_L_XK, grad_L_XV and part of the norm gradients from what the
  * walk hands it, so that only the chain through the running gradients stays on
- * the critical path.  The reference launcher
+ * the critical path, and a fifth (with a multiple of 8 pairs, if 5*n fits) only
+ * reads ahead of the walk so that the walk's requests hit the L2.  The reference launcher
  * (kernels/ttt_backward/ttt.cu:1451-1917) has no counterpart: it spreads one
  * (batch, head) over a cluster of four thread blocks instead.
  * Workgroups that wait for each other must be resident together (one per CU),

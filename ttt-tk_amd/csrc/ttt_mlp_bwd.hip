@@ -6,9 +6,9 @@
 // activations are saved, then the group is walked backwards producing the ten output gradients.
 //
 // Mapping: workgroups of 8 wavefronts (two per SIMD, at most 256 registers each); one per (batch,
-// head), or two to four where the device has CUs to spare - then one or two replay the checkpoint
-// groups (taking turns), one walks them backwards, a group or more behind, and a fourth forms
-// grad_L_XK from what the walk hands it.  Wave v owns hidden columns [32v, 32v+32).  All [tokens x hidden] activations live in
+// head), or two to five where the device has CUs to spare - then one or two replay the checkpoint
+// groups (taking turns), one walks them backwards, a group or more behind, a fourth forms
+// grad_L_XK from what the walk hands it, and a fifth reads ahead of the walk into the L2.  Wave v owns hidden columns [32v, 32v+32).  All [tokens x hidden] activations live in
 // registers in the "Q" orientation (accumulator rows = hidden, lane = token), so per-token scalars
 // (eta, dEta partial sums) are per-lane values.  An activation that is also needed with tokens as the
 // contraction index is bounced once through a wave-private LDS tile (row store + transposing read).

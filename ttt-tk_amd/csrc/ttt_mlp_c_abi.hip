@@ -148,7 +148,7 @@ struct LaunchPlan {
   int per_pair = 1;         // workgroups per pair of the rest: 2, or 3 / 4 where the kernel can use them and they fit
   bool prefetch = false;    // backward with 4 per pair: a fifth that fetches ahead of the walk
 };
-// `three_way`: the backward can use three or four workgroups per pair, the forward two.
+// `three_way`: the backward can use three to five workgroups per pair, the forward two.
 LaunchPlan plan_for(long long BH, int cus, bool three_way) {
   LaunchPlan pl;
   if (BH <= 0 || cus <= 0) {
