@@ -375,6 +375,8 @@ TTT_DEV bf16x8 w1_before(gptr_t img, gptr_t ck, unsigned ck_off, int j, int rb, 
   return r;
 }
 
+constexpr int FIN_CHUNK = 8;   // mini-batches per hand-over to the grad_L_XK workgroup within the last group walked (a power of two)
+
 // ------------------------------------------------------------------ two workgroups per (batch, head)
 // The replay of a checkpoint group needs only the checkpoint, so it can run ahead of the reverse walk
 // on another CU: one workgroup replays group after group into two alternating sets of the per-group
@@ -1389,6 +1391,14 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
         g_st_stream<bf16x8>(bDXK, vln, xo, dxk_old);
       }
       TTT_STAGE(BS_W_DXK);
+      if constexpr (ROLE == 2 && FIN) {
+        // The last group to be walked is handed to the grad_L_XK workgroup in chunks, so that that workgroup follows
+        // FIN_CHUNK mini-batches behind instead of ending a whole group after the walk.
+        if (k == 0 && (j & (FIN_CHUNK - 1)) == 0) {
+          publish(w_sync + 12, n_mb - j);
+          TTT_STAGE(BS_PUBLISH);
+        }
+      }
     }
     if constexpr (ROLE == 2) publish(w_walked, done + 1);
     TTT_STAGE(BS_PUBLISH);
@@ -1503,7 +1513,8 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
   for (int k = p.K - 1; k >= 0; k--) {
     const int n_mb = min(cgs, p.NC - k * cgs);
     const int done = p.K - 1 - k, set = done % n_sets;
-    if (!wait_at_least(w_walked, done + 1, p.status, s_flag, p.wait_limit)) return;
+    // the walk hands over whole groups, except the last one it walks (k = 0): that one in chunks of FIN_CHUNK mini-batches
+    if (k > 0 && !wait_at_least(w_walked, done + 1, p.status, s_flag, p.wait_limit)) return;
     TTT_STAGE(BS_X_GROUP);
     const size_t ofin = uni64(((size_t)bh * 2 + (done & 1)) * cgs);
     const size_t o_img = uni64((size_t)bh * cgs * (CS * HID)), o_tile = uni64((size_t)bh * cgs * (CS * FD));
@@ -1515,6 +1526,10 @@ TTT_DEV void bwd_finish_dxk(const BwdParams& p, unsigned char* smem, const int b
     const gptr_t gIMG1 = gbuf((set ? p.alt_X2_group[set - 1] : p.X2_group) + uni64((size_t)bh * cgs * (CS * HID)));
     const unsigned ckW = static_cast<unsigned>(k) * (FD * HID * 4u);
     for (int j = n_mb - 1; j >= 0; j--) {
+      if (k == 0 && (j == n_mb - 1 || (j & (FIN_CHUNK - 1)) == FIN_CHUNK - 1)) {
+        if (!wait_at_least(w_sync + 12, n_mb - (j & ~(FIN_CHUNK - 1)), p.status, s_flag, p.wait_limit)) return;
+        TTT_STAGE(BS_X_GROUP);
+      }
       const unsigned xo = (k * cgs + j) * TILE_BYTES, so = j * TILE_BYTES, ho = j * IMG_BYTES;
       const bf16x8 dxk_ld = g_ld_stream<bf16x8>(p.overwrite ? gbuf(zero_tile) : gDXK, vln, p.overwrite ? 0u : xo);
       const bf16x8 dxv_ld = g_ld_stream<bf16x8>(p.overwrite ? gbuf(zero_tile) : gDXV, vln, p.overwrite ? 0u : xo);

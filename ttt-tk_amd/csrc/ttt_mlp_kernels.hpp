@@ -86,7 +86,8 @@ struct BwdParams {
 
 // Layout of `sync` (ints): 32 per (batch, head) - words 0 and 8 count the groups replayed by the first /
 // second replaying workgroup (norm_partial is written before the last count), word 16 the groups the
-// reverse walk has finished, word 20 the mini-batches it has started (a pacing hint for the prefetching workgroup,
+// reverse walk has finished, word 12 the mini-batches of the last group it walks that it has handed to the grad_L_XK
+// workgroup (that group is handed over in chunks), word 20 the mini-batches it has started (a pacing hint for the prefetching workgroup,
 // no data is ordered by it), word 24 the groups the grad_L_XK workgroup has finished - then one status
 // word (non-zero: a wait gave up).
 constexpr int BWD_SYNC_STRIDE = 32;
