@@ -43,6 +43,9 @@ def stage_names(header_text: str, enum: str):
     return out
 
 
+PER_WAVE = False
+
+
 def table(title, clocks, names, per_mb):
     """clocks: tensor [pairs][8 waves][SLOTS] of summed clocks; per_mb: mini-batches each wave went through."""
     mean_w = clocks.double().mean(dim=0) / per_mb          # [8][SLOTS]
@@ -52,7 +55,10 @@ def table(title, clocks, names, per_mb):
         m, mx = mean_w[:, i].mean().item(), mean_w[:, i].max().item()
         if mx <= 0:
             continue
-        lines.append(f"  {name:18s} {m:8.0f} {100 * m / tot.mean().item():5.1f} %   slowest wave {mx:8.0f}   {desc}")
+        if PER_WAVE:
+            lines.append(f"  {name:18s} {m:8.0f}   waves 0-7: " + " ".join(f"{x:6.0f}" for x in mean_w[:, i].tolist()))
+        else:
+            lines.append(f"  {name:18s} {m:8.0f} {100 * m / tot.mean().item():5.1f} %   slowest wave {mx:8.0f}   {desc}")
     return lines
 
 
@@ -60,7 +66,10 @@ def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c4")
     ap.add_argument("--out", default=None, help="also write the tables to this file")
+    ap.add_argument("--per-wave", action="store_true", help="every stage's clocks wave by wave instead of share and description")
     a = ap.parse_args()
+    global PER_WAVE
+    PER_WAVE = a.per_wave
     import torch
     sys.path.insert(0, ROOT)
     sys.path.insert(0, HERE)
