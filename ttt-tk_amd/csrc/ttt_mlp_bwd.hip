@@ -1026,6 +1026,30 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
 #define bFDZ gbuf(ka->fin_dz + ofin * (CS * HID))
 #define bFGY gbuf(ka->fin_gy + ofin * (2 * CS * FD))
     TTT_STAGE(BS_GROUP);
+    // What a mini-batch of the walk needs first - its two input tiles, the two tiles the replay left for it (gZ2 and
+    // gZ2_bar) and eta - is requested during the updates of the mini-batch walked before it and held in registers
+    // until the barrier that opens the mini-batch (the very first one of a group is requested here).  The walk is the
+    // longest chain of the backward pass; with the lines in the L2 already, a request a stage earlier hides the rest.
+    u32x4 n_xq, n_xk, n_gz, n_gzb;
+    bf16 n_eta, n_etai[2];
+    // What the output branch adds to the running gradients: the replay has taken that branch backwards already
+    // and left gZ2_bar (a tile) and X2_bar^T, gZ1_bar^T as operand images.
+    bf16x8 x2b[4], g1b[4];   // lane = hid, contraction = tok
+#define WALK_FETCH(jn)                                                                                   \
+    {                                                                                                    \
+      LANE_VARS;                                                                                         \
+      constexpr bool ST = ROLE != 0;   /* tiles another workgroup left here are read once */             \
+      const int jf = __builtin_amdgcn_readfirstlane(jn), mbf = k * cgs + jf;                             \
+      const unsigned xo = mbf * TILE_BYTES, so = jf * TILE_BYTES;                                        \
+      n_etai[0] = g_ldh(bETA, 2 * c, mbf * (CS * 2) + 64 * tb[0]);                                       \
+      n_etai[1] = g_ldh(bETA, 2 * c, mbf * (CS * 2) + 64 * tb[1]);                                       \
+      n_xq = g_ld16(bXQ, t16, xo);                                                                       \
+      n_xk = g_ld16(bXK, t16, xo);                                                                       \
+      n_gz = ST ? g_ld_stream<u32x4>(bGZ2, t16, so) : g_ld16(bGZ2, t16, so);                             \
+      n_gzb = ST ? g_ld_stream<u32x4>(bGZB, t16, so) : g_ld16(bGZB, t16, so);                            \
+      n_eta = g_ldh(bETA, 2 * (tid & (CS - 1)), mbf * (CS * 2));                                         \
+    }
+    if constexpr (ROLE != 1) WALK_FETCH(n_mb - 1);
     if constexpr (ROLE != 1)
     for (int j = n_mb - 1; j >= 0; j--) {
       const int mb = k * cgs + j;
@@ -1038,29 +1062,21 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
       const unsigned so = j * TILE_BYTES;        // its slot in the [cgs][64][64] scratch tensors
       const unsigned ho = j * IMG_BYTES;         // its slot in the [cgs][64][256] scratch tensors
       // eta of the token this lane holds in column block i of a Q-orientation tile
-      const float eta_i[2] = {bf2f(g_ldh(bETA, 2 * c, mb * (CS * 2) + 64 * tb[0])), bf2f(g_ldh(bETA, 2 * c, mb * (CS * 2) + 64 * tb[1]))};
-      // What the output branch adds to the running gradients: the replay has taken that branch backwards already
-      // and left gZ2_bar (a tile, to LDS here) and X2_bar^T, gZ1_bar^T as operand images.
-      bf16x8 x2b[4], g1b[4];   // lane = hid, contraction = tok
+      const float eta_i[2] = {bf2f(n_etai[0]), bf2f(n_etai[1])};
       {
         LANE_VARS;
-        constexpr bool ST = ROLE != 0;   // tiles another workgroup left here are read once
-        const u32x4 xq = g_ld16(bXQ, t16, xo), xk = g_ld16(bXK, t16, xo);
-        const u32x4 gz = ST ? g_ld_stream<u32x4>(bGZ2, t16, so) : g_ld16(bGZ2, t16, so);
-        const u32x4 gzb = ST ? g_ld_stream<u32x4>(bGZB, t16, so) : g_ld16(bGZB, t16, so);
-        const float eta = bf2f(g_ldh(bETA, 2 * (tid & (CS - 1)), mb * (CS * 2)));
-        // the two operand images of the next stage are asked for behind the tiles: on their way across both barriers
+        // the two operand images of the next stage are asked for here: on their way across both barriers
 #pragma unroll
         for (int s = 0; s < 4; s++) {
           x2b[s] = image_load<ROLE != 0>(bX2B, ho, s, t16);
           g1b[s] = image_load<ROLE != 0>(bGZ1B, ho, s, t16);
         }
-        __syncthreads();   // the previous mini-batch's readers of these tiles are done (the loads are under way)
-        lds_put16x(s_xq, tid, xq);
-        lds_put16x(s_xk, tid, xk);
-        lds_put16(s_gz2, tid, gz);
-        lds_put16(s_a, tid, gzb);
-        if (tid < CS) s_eta[tid] = eta;
+        __syncthreads();   // the previous mini-batch's readers of these tiles are done
+        lds_put16x(s_xq, tid, n_xq);
+        lds_put16x(s_xk, tid, n_xk);
+        lds_put16(s_gz2, tid, n_gz);
+        lds_put16(s_a, tid, n_gzb);
+        if (tid < CS) s_eta[tid] = bf2f(n_eta);
       }
       __syncthreads();
 
@@ -1359,6 +1375,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
             store_piece_rows<LDH>(T2, tb[i], t, c, h, uhp[i][t]);   // -eta u rows [tok][hid]
           }
         WAVE_SYNC();
+        WALK_FETCH(j > 0 ? j - 1 : 0);   // the next mini-batch's tiles (the last step of a group asks for its own again)
         if constexpr (!FIN)
           mma_jit<2>(dk, [&](int rb, int s) { return w1bf[rb][s]; },                           // + W1 dZ1^T, W1 before the step
                      [&](int i, int s) { return dzp[i][s]; });
@@ -1404,6 +1421,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
     TTT_STAGE(BS_PUBLISH);
 #undef bFDZ
 #undef bFGY
+#undef WALK_FETCH
   }
   TTT_STAGES_END(p.stage_clocks == nullptr ? nullptr : p.stage_clocks + ((size_t)bh * 4 + (ROLE == 1 ? turn : 2)) * (BW_NWAVE * STAGE_SLOTS));
   if constexpr (ROLE == 1) return;
