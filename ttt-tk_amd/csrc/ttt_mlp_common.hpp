@@ -410,11 +410,15 @@ TTT_DEV bf16x8 xpiece_tr(const bf16* tile, int blk, int s, int lane) {
 // Asynchronous: the data is in LDS once the wave's vmcnt has drained (and visible to other waves after a barrier).
 typedef const __attribute__((address_space(1))) unsigned* gword_t;
 typedef __attribute__((address_space(3))) unsigned* lword_t;
+// AUX = cache policy bits of the load; CPOL_NT marks a tile that is read once (streaming), so that it does not push
+// re-used lines out of the L2.
+constexpr int CPOL_NT = 2;
+template <int AUX = 0>
 TTT_DEV void tile_to_lds(gptr_t g, unsigned off, unsigned char* tile, int v, int lane) {
   const gptr_t src = g + static_cast<uint64_t>(uni(off + v * 1024)) + static_cast<uint64_t>(4u * lane);
 #pragma unroll
   for (int j = 0; j < 4; j++)
-    __builtin_amdgcn_global_load_lds((gword_t)(src + 256 * j), (lword_t)(tile + (4 * v + j) * (XPAIR * 2)), 4, 0, 0);
+    __builtin_amdgcn_global_load_lds((gword_t)(src + 256 * j), (lword_t)(tile + (4 * v + j) * (XPAIR * 2)), 4, 0, AUX);
 }
 // The 64 bf16 step sizes of a mini-batch (128 bytes), by wave 0.
 TTT_DEV void eta_to_lds(gptr_t g, unsigned off, unsigned char* dst, int v, int lane) {
