@@ -32,7 +32,8 @@ def _args(order, t, cgs, B, NH, NC, K):
 
 
 # 8 pairs: the backward runs with a fifth workgroup per pair that fetches ahead of the walk (a multiple of 8 pairs)
-@pytest.mark.parametrize("B,NH,NC,cgs", [(1, 2, 1, 1), (1, 3, 5, 8), (2, 2, 17, 4), (1, 8, 13, 4), (2, 4, 3, 8)])
+@pytest.mark.parametrize("B,NH,NC,cgs", [(1, 2, 1, 1), (1, 3, 5, 8), (2, 2, 17, 4), (1, 8, 13, 4), (2, 4, 3, 8),
+                                          (1, 16, 9, 4), (3, 8, 5, 2), (1, 48, 19, 8)])
 def test_overlapped_launchers_through_ctypes(B, NH, NC, cgs):
     print(f"case B={B} NH={NH} NC={NC} cgs={cgs}", flush=True)
     import ttt_mlp_host as host
