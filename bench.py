@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the TTT-MLP forward + remat-backward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c5|c3|c2] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c5|c3|c2] [--only] [--no-cpu-baseline]
 
 A "step" is one forward + one remat backward over one batch of synthetic input that is already
 resident in HBM (zero-filling the four accumulating gradient outputs is part of the step, as the
@@ -10,6 +10,7 @@ operator's contract makes the caller do it).  Prints ONE JSON line:
   roofline   the dominant kernel (the backward) against the dense bf16 MFMA peak, its duration
              measured with events on the launch stream inside the timed region
   cpu_baseline  the fp32 PyTorch oracle of the same math on the host cores, on a bounded sample
+  c5         (default run only) the same figures for the fill-the-chip workload, the one the 35 % target is set on
 """
 from __future__ import annotations
 
@@ -96,45 +97,60 @@ def cpu_baseline(NH, cgs, nc_sample, backward=True):
                       f"({nc_sample * 64} tokens) cgs={cgs}, {dt:.1f} s"}
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=3)
-    ap.add_argument("--warmup", type=int, default=1)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c4")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--overwrite", action="store_true",
-                    help="let ttt_backward overwrite grad_L_XQ / XK / XV / last_eta instead of adding to them "
-                         "(no zero-fill in the step; not the upstream calling convention, so not the default)")
-    ap.add_argument("--no-overlap", action="store_true",
-                    help="backward with one workgroup per (batch, head) even where two fit the device")
-    ap.add_argument("--cpu-sample-mb", type=int, default=1536, help="mini-batches in the CPU baseline sample")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run one plain 1 GiB device copy, so that a counter run has a kernel of known traffic")
-    a = ap.parse_args()
-    if a.gpus != 1:
-        sys.exit("bench.py: this build runs on ONE GPU (every (batch, head) recurrence is independent and no "
-                 "collective is involved); --gpus must be 1")
+METRICS = {
+    # the metric string follows the workload; c4's is BASELINE.json's
+    "c2": "TTT-MLP forward tokens/sec on 1 MI355X (B=1,NH=48,16K tok); % bf16 MFMA peak",
+    "c3": "TTT-MLP fwd+bwd tokens/sec on 1 MI355X (B=1,NH=48,16K tok); % bf16 MFMA peak",
+    "c4": "TTT-MLP fwd+bwd tokens/sec on 1 MI355X (B=1,NH=48,256K tok); % bf16 MFMA peak",
+    "c5": "TTT-MLP fwd+bwd tokens/sec on 1 MI355X (B=8,NH=48,32K tok/seq); % bf16 MFMA peak",
+}
 
+
+def kernel_sources_digest():
+    """sha256 over the kernel sources the library is built from: the counter summaries under profiles/ carry the digest
+    of the sources they were measured on, and a summary of other sources is not quoted."""
+    import hashlib
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "ttt-tk_amd", "csrc")
+    for name in sorted(os.listdir(csrc)):
+        if name.endswith((".hip", ".hpp")):
+            h.update(name.encode())
+            with open(os.path.join(csrc, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()
+
+
+def measured_traffic_checked(workload, which):
+    """(bytes or None, note or None): the measured HBM bytes of profiles/ if they were taken on these kernel sources."""
+    path = os.path.join(ROOT, "profiles", f"ttt_mlp_{workload}_counters.json")
+    if not os.path.exists(path):
+        return None, "no counter summary for this workload under profiles/"
+    with open(path) as f:
+        stamp = json.load(f).get("kernel_sources_sha256")
+    if stamp != kernel_sources_digest():
+        return None, "the counter summary under profiles/ was measured on other kernel sources (its kernel_sources_sha256 differs)"
+    return measured_traffic(workload, which), None
+
+
+def run_workload(name, steps, warmup, overwrite=False, no_overlap=False, calibrate_copy=False):
+    """Times `steps` forward (+ backward) steps of one workload and returns the figures of its JSON block."""
     import torch
     import ttt_mlp_host as host          # fails loudly if the HIP extension is not built
+    import test_time_training as ext
 
-    if not torch.cuda.is_available():
-        sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
-    B, NH, NC, cgs, eta_std, desc = WORKLOADS[a.workload]
+    B, NH, NC, cgs, eta_std, desc = WORKLOADS[name]
     t = make_device_inputs(B, NH, NC, eta_std, dev)
     t.update(host.alloc_forward_buffers(B, NH, NC, cgs, dev))
-    backward = a.workload != "c2"
+    backward = name != "c2"
     if backward:
         t.update(host.alloc_backward_buffers(B, NH, NC, cgs, dev))
     host.set_synchronize(False)           # time with events; the operator's default host sync is not part of the kernel
-    import test_time_training as ext
-    ext.set_overlap(not a.no_overlap)
-    ext.set_accumulate(not a.overwrite)
+    ext.set_overlap(not no_overlap)
+    ext.set_accumulate(not overwrite)
 
     def step(ev=None):
-        if backward and not a.overwrite:
+        if backward and not overwrite:
             host.zero_accumulating_grads(t)    # the operator adds to four of its outputs, as upstream does
         if ev:
             ev[0].record()
@@ -146,18 +162,18 @@ def main():
         if ev:
             ev[2].record()
 
-    for _ in range(a.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(a.steps)]
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
     t0 = time.perf_counter()
-    for i in range(a.steps):
+    for i in range(steps):
         step(events[i])
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ext.check_last_status()               # raises if workgroups of an unsynchronised launch gave up waiting for each other
     host.set_synchronize(True)
-    if a.calibrate_copy:
+    if calibrate_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)     # 1 GiB read + 1 GiB written
         dst = torch.empty_like(src)
         dst.copy_(src)
@@ -166,11 +182,10 @@ def main():
     assert bool(torch.isfinite(t["Out"].float()).all())
     assert not backward or bool(torch.isfinite(t["grad_L_W1_init"]).all())
 
-    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in events) / a.steps
-    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in events) / a.steps
-    ms_per_step = wall * 1e3 / a.steps
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in events) / steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in events) / steps
+    ms_per_step = wall * 1e3 / steps
     tokens = B * NC * 64
-    value = tokens / (ms_per_step * 1e-3)
     mb_steps = B * NH * NC
     bwd_tflops = BWD_G * G_FLOP * mb_steps / (bwd_ms * 1e-3) / 1e12 if backward else 0.0
     fwd_tflops = FWD_G * G_FLOP * mb_steps / (fwd_ms * 1e-3) / 1e12
@@ -187,26 +202,72 @@ def main():
         bwd_kernel = f"ttt_mlp_bwd_split_kernel<{2 if per.value >= 3 else 1}, {'true' if per.value >= 4 else 'false'}>"
         if one.value:
             bwd_kernel = "ttt_mlp_bwd_kernel + " + bwd_kernel
-    out = {
-        "metric": "TTT-MLP fwd+bwd tokens/sec on 1 MI355X (B=1,NH=48,256K tok); % bf16 MFMA peak" if backward
-                  else "TTT-MLP forward tokens/sec on 1 MI355X; % bf16 MFMA peak",
-        "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"{a.workload}: {desc}", "B": B, "NH": NH, "NC": NC, "tokens": tokens,
+    traffic, note = measured_traffic_checked(name, "bwd" if backward else "fwd")
+    # the dominant kernel: the backward (the forward where there is no backward)
+    roofline = {"bound": "mfma", "kernel": bwd_kernel if backward else fwd_kernel,
+                "achieved": bwd_tflops if backward else fwd_tflops, "peak": PEAK_BF16_TFLOPS,
+                "unit": "TFLOP/s", "frac": (bwd_tflops if backward else fwd_tflops) / PEAK_BF16_TFLOPS,
+                "traffic": traffic,
+                "flop_per_launch": (BWD_G if backward else FWD_G) * G_FLOP * mb_steps,
+                "avg_launch_ms": bwd_ms if backward else fwd_ms}
+    if note:
+        roofline["traffic_note"] = note
+    del t
+    torch.cuda.empty_cache()
+    return {
+        "metric": METRICS[name],
+        "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s", "ms_per_step": ms_per_step,
+        "config": {"workload": f"{name}: {desc}", "B": B, "NH": NH, "NC": NC, "tokens": tokens,
                    "checkpoint_group_size": cgs},
         "fwd_ms": fwd_ms, "bwd_ms": bwd_ms, "fwd_tflops": fwd_tflops, "fwd_bwd_tflops": all_tflops,
         "pct_of_bf16_mfma_peak": 100.0 * all_tflops / PEAK_BF16_TFLOPS,
-        # the dominant kernel: the backward (the forward where there is no backward)
-        "roofline": {"bound": "mfma", "kernel": bwd_kernel if backward else fwd_kernel,
-                     "achieved": bwd_tflops if backward else fwd_tflops, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": (bwd_tflops if backward else fwd_tflops) / PEAK_BF16_TFLOPS,
-                     "traffic": measured_traffic(a.workload, "bwd" if backward else "fwd"),
-                     "flop_per_launch": (BWD_G if backward else FWD_G) * G_FLOP * mb_steps,
-                     "avg_launch_ms": bwd_ms if backward else fwd_ms},
+        "roofline": roofline,
     }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c4")
+    ap.add_argument("--only", action="store_true",
+                    help="time the named workload alone (without this, a c4 run also times the fill-the-chip workload c5 "
+                         "and reports it in a \"c5\" block of the same JSON line)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--overwrite", action="store_true",
+                    help="let ttt_backward overwrite grad_L_XQ / XK / XV / last_eta instead of adding to them "
+                         "(no zero-fill in the step; not the upstream calling convention, so not the default)")
+    ap.add_argument("--no-overlap", action="store_true",
+                    help="backward with one workgroup per (batch, head) even where two fit the device")
+    ap.add_argument("--cpu-sample-mb", type=int, default=1536, help="mini-batches in the CPU baseline sample")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 1 GiB device copy, so that a counter run has a kernel of known traffic")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (every (batch, head) recurrence is independent and no "
+                 "collective is involved); --gpus must be 1")
+
+    import torch
+    import ttt_mlp_host  # noqa: F401    fails loudly if the HIP extension is not built
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    res = run_workload(a.workload, a.steps, a.warmup, a.overwrite, a.no_overlap, a.calibrate_copy)
+    out = {
+        "metric": res["metric"], "value": res["value"], "unit": res["unit"], "n_gpus": 1, "steps": a.steps,
+        "warmup": a.warmup, "ms_per_step": res["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic", "config": res["config"],
+        "fwd_ms": res["fwd_ms"], "bwd_ms": res["bwd_ms"], "fwd_tflops": res["fwd_tflops"],
+        "fwd_bwd_tflops": res["fwd_bwd_tflops"], "pct_of_bf16_mfma_peak": res["pct_of_bf16_mfma_peak"],
+        "roofline": res["roofline"],
+    }
+    if a.workload == "c4" and not a.only:
+        # the configuration the target (35 % of the MFMA peak) is set on, timed the same way in the same run
+        out["c5"] = run_workload("c5", a.steps, a.warmup, a.overwrite, a.no_overlap)
     if not a.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(NH, cgs, min(a.cpu_sample_mb, NC), backward)
+        B, NH, NC, cgs, _, _ = WORKLOADS[a.workload]
+        out["cpu_baseline"] = cpu_baseline(NH, cgs, min(a.cpu_sample_mb, NC), a.workload != "c2")
     print(json.dumps(out), flush=True)
 
 

@@ -68,3 +68,25 @@ def test_the_product_library_contains_no_stage_clocks():
     stages = os.path.join(PKG, "libttt_mlp_stages.so")
     if os.path.exists(stages):
         assert hasattr(ctypes.CDLL(stages), "ttt_mlp_set_stage_clocks")
+
+
+def test_algorithmic_work_per_launch_follows_the_shapes():
+    """7 / 21 contractions of 2*64*64*256 FLOP per (batch, head, mini-batch); bytes = the operator's inputs and outputs of a
+    mini-batch plus the checkpoint bytes once per group."""
+    f, b = pc.algorithmic("c4", "fwd"), pc.algorithmic("c4", "bwd")
+    assert f["units"] == b["units"] == 48 * 4096
+    assert f["flop"] == 7 * 2097152 * 48 * 4096 and b["flop"] == 21 * 2097152 * 48 * 4096
+    assert abs(f["bytes"] - 48 * 4096 * (3 * 8192 + 128 + 8192 + 132352 / 64)) < 1
+    assert abs(b["bytes"] - 48 * 4096 * (4 * 8192 + 128 + 3 * 8192 + 128 + 3 * 8192 + 132352 / 64)) < 1
+    assert pc.algorithmic("c5", "bwd")["units"] == 8 * 48 * 512
+
+
+def test_bench_and_harness_stamp_the_same_kernel_sources():
+    """bench.py quotes the measured traffic of a summary only when the digest of the kernel sources matches."""
+    sys.path.insert(0, ROOT)
+    import bench
+    assert bench.kernel_sources_digest() == pc.sources_digest()
+    assert len(pc.sources_digest()) == 64
+    for w in ("c2", "c3", "c4", "c5"):
+        assert w in bench.METRICS and w in pc.SHAPES
+        assert bench.WORKLOADS[w][:4] == pc.SHAPES[w]

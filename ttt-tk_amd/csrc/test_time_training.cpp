@@ -20,6 +20,7 @@ bool g_overlap = true;      // two workgroups per (batch, head) whenever they fi
 unsigned long long g_wait_ticks = 2000000000ull;   // mirrors the library's limit, for the error text
 torch::Tensor* g_sticky = nullptr;   // a device int, non-zero once a launch that nobody waited for gave up a wait (never freed:
                                      // a static tensor would be destroyed after the runtime at process exit)
+torch::Tensor* g_workspace = nullptr;   // caller-owned workspace of the multi-workgroup launches (set_workspace); never freed here
 int g_last_forward_mode = -1;    // 0 = one workgroup per (batch, head), 1 = two
 int g_last_backward_mode = -1;
 
@@ -88,6 +89,27 @@ bool workspace_is_affordable(size_t bytes) {
   return bytes <= free_b / 2;
 }
 
+// Where the workspace of a multi-workgroup launch comes from.  With a caller-owned workspace (set_workspace) the
+// operators allocate nothing and ask the device nothing: the launch uses it if it is large enough and on the right
+// device, and falls back to one workgroup per (batch, head) otherwise.  Without one the workspace comes from torch's
+// caching allocator (which orders its reuse after the launch on the same stream) if the device has room to spare.
+struct Workspace {
+  void* ptr = nullptr;
+  torch::Tensor held;   // keeps an allocated workspace alive until the launch has been enqueued
+};
+Workspace take_workspace(size_t bytes, const torch::Device& dev) {
+  Workspace w;
+  if (bytes == 0) return w;
+  if (g_workspace != nullptr) {
+    if (g_workspace->device() == dev && (size_t)g_workspace->numel() >= bytes) w.ptr = g_workspace->data_ptr();
+    return w;
+  }
+  if (!workspace_is_affordable(bytes)) return w;
+  w.held = torch::empty({(int64_t)bytes}, torch::TensorOptions().dtype(torch::kUInt8).device(dev));
+  w.ptr = w.held.data_ptr();
+  return w;
+}
+
 }  // namespace
 
 torch::Tensor ttt_forward(const torch::Tensor XQ, const torch::Tensor XK, const torch::Tensor XV,
@@ -131,14 +153,13 @@ torch::Tensor ttt_forward(const torch::Tensor XQ, const torch::Tensor XK, const 
   const c10::DeviceGuard guard(XQ.device());
   hipStream_t stream = c10::hip::getCurrentHIPStream(XQ.device().index()).stream();
   // With few (batch, head) pairs most CUs would idle: then a second workgroup per pair computes Out behind
-  // the state recurrence.  Its workspace comes from torch's caching allocator, which orders its reuse
-  // after this launch on the same stream.
+  // the state recurrence.  Its workspace: the caller's (set_workspace) or torch's caching allocator's.
   const size_t ws_bytes = (g_overlap && NC >= 2) ? ttt_mlp_fwd_workspace_bytes((int32_t)B, (int32_t)NH) : 0;
-  if (workspace_is_affordable(ws_bytes)) {
-    torch::Tensor ws = torch::empty({(int64_t)ws_bytes}, torch::TensorOptions().dtype(torch::kUInt8).device(XQ.device()));
+  const Workspace ws = take_workspace(ws_bytes, XQ.device());
+  if (ws.ptr != nullptr) {
     g_last_forward_mode = 1;
-    const char* status = static_cast<const char*>(ws.data_ptr()) + ttt_mlp_fwd_status_offset((int32_t)B, (int32_t)NH);
-    finish(ttt_mlp_fwd_launch_overlapped(&a, ws.data_ptr(), ws_bytes, stream), stream, "ttt_forward", XQ.device(), status);
+    const char* status = static_cast<const char*>(ws.ptr) + ttt_mlp_fwd_status_offset((int32_t)B, (int32_t)NH);
+    finish(ttt_mlp_fwd_launch_overlapped(&a, ws.ptr, ws_bytes, stream), stream, "ttt_forward", XQ.device(), status);
   } else {
     g_last_forward_mode = 0;
     finish(ttt_mlp_fwd_launch(&a, stream), stream, "ttt_forward", XQ.device());
@@ -244,14 +265,14 @@ torch::Tensor ttt_backward(
   const c10::DeviceGuard guard(XQ.device());
   hipStream_t stream = c10::hip::getCurrentHIPStream(XQ.device().index()).stream();
   // With few (batch, head) pairs most CUs would idle: then a second workgroup per pair recomputes the
-  // checkpoint groups ahead of the reverse walk.  Its workspace (a second set of the per-group tensors)
-  // comes from torch's caching allocator, which orders its reuse after this launch on the same stream.
+  // checkpoint groups ahead of the reverse walk.  Its workspace (further sets of the per-group tensors): the
+  // caller's (set_workspace) or torch's caching allocator's.
   const size_t ws_bytes = (g_overlap && K >= 2) ? ttt_mlp_bwd_workspace_bytes((int32_t)B, (int32_t)NH, checkpoint_group_size) : 0;
-  if (workspace_is_affordable(ws_bytes)) {
-    torch::Tensor ws = torch::empty({(int64_t)ws_bytes}, torch::TensorOptions().dtype(torch::kUInt8).device(XQ.device()));
+  const Workspace ws = take_workspace(ws_bytes, XQ.device());
+  if (ws.ptr != nullptr) {
     g_last_backward_mode = 1;
-    const char* status = static_cast<const char*>(ws.data_ptr()) + ttt_mlp_bwd_status_offset((int32_t)B, (int32_t)NH);
-    int rc = ttt_mlp_bwd_launch_overlapped(&a, ws.data_ptr(), ws_bytes, stream);
+    const char* status = static_cast<const char*>(ws.ptr) + ttt_mlp_bwd_status_offset((int32_t)B, (int32_t)NH);
+    int rc = ttt_mlp_bwd_launch_overlapped(&a, ws.ptr, ws_bytes, stream);
     if (rc == 0 && g_fill_group_tensors) rc = ttt_mlp_bwd_export_group0(&a, stream);
     finish(rc, stream, "ttt_backward", XQ.device(), status);
   } else {
@@ -304,6 +325,29 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "any launch since the last call gave up (the outputs of that launch are invalid).");
   m.def("set_wait_limit", [](unsigned long long ticks) { g_wait_ticks = ticks; ttt_mlp_set_wait_limit(ticks); },
         "Ticks of the GPU's 100 MHz clock a workgroup waits for its partner before giving up (default 2e9 = 20 s).");
+  // The upstream operator allocates nothing: every tensor, scratch included, is the caller's
+  // (kernels/ttt_backward/ttt.cu:1451-1917).  The launches with several workgroups per (batch, head) need a workspace
+  // beyond the upstream argument list; a caller that wants the same guarantee hands it over once.
+  m.def("workspace_bytes", [](int B, int NH, int checkpoint_group_size) {
+          const size_t f = ttt_mlp_fwd_workspace_bytes(B, NH), b = ttt_mlp_bwd_workspace_bytes(B, NH, checkpoint_group_size);
+          return (unsigned long long)(f > b ? f : b);
+        },
+        "Bytes of workspace that let ttt_forward and ttt_backward of this shape use several workgroups per (batch, head) "
+        "(0: the shape runs with one workgroup per pair and needs none).");
+  m.def("set_workspace", [](c10::optional<torch::Tensor> ws) {
+          if (!ws.has_value()) { delete g_workspace; g_workspace = nullptr; return; }
+          TORCH_CHECK(ws->device().is_cuda() && ws->is_contiguous() && ws->scalar_type() == torch::kUInt8 && ws->dim() == 1,
+                      "set_workspace: a contiguous 1-D uint8 GPU tensor is expected");
+          TORCH_CHECK(reinterpret_cast<uintptr_t>(ws->data_ptr()) % 256 == 0, "set_workspace: the tensor must be 256-byte aligned");
+          (void)sticky_word(ws->device());   // the one device word check_last_status reads exists before the first launch
+          delete g_workspace;
+          g_workspace = new torch::Tensor(*ws);
+        },
+        "Hand the operators a workspace (1-D uint8 GPU tensor of at least workspace_bytes(...) bytes) that they use for "
+        "every later call instead of allocating one: with it ttt_forward / ttt_backward allocate nothing and do not query "
+        "the device's free memory; a call whose shape needs more than the tensor holds, or that runs on another device, "
+        "uses one workgroup per (batch, head).  The contents are scratch; calls that overlap in time must not share it.  "
+        "None returns to the default (workspace from torch's caching allocator per call).");
   m.def("last_forward_mode", []() { return g_last_forward_mode; },
         "0: the last ttt_forward used one workgroup per (batch, head); 1: two; -1: none yet.");
   m.def("last_backward_mode", []() { return g_last_backward_mode; },

@@ -42,8 +42,8 @@ extern "C" const char* ttt_mlp_error_string(int code) {
     case TTT_MLP_ERR_BAD_CKPT: return "ttt_mlp: number of checkpoints K must equal ceil(NC / checkpoint_group_size)";
     case TTT_MLP_ERR_ALIGN: return "ttt_mlp: every tensor pointer must be 16-byte aligned";
     case TTT_MLP_ERR_TOO_LARGE: return "ttt_mlp: B*NH exceeds the launch grid limit, or NC > 262144, or checkpoint_group_size > 65536, or more than 32768 checkpoints";
-    case TTT_MLP_ERR_NO_ROOM: return "ttt_mlp: two workgroups per (batch, head) do not fit the compute units of this device; use ttt_mlp_bwd_launch";
-    case TTT_MLP_ERR_WORKSPACE: return "ttt_mlp: workspace smaller than ttt_mlp_bwd_workspace_bytes()";
+    case TTT_MLP_ERR_NO_ROOM: return "ttt_mlp: two workgroups per (batch, head) do not fit the compute units of this device; use ttt_mlp_fwd_launch / ttt_mlp_bwd_launch";
+    case TTT_MLP_ERR_WORKSPACE: return "ttt_mlp: workspace smaller than ttt_mlp_fwd_workspace_bytes() / ttt_mlp_bwd_workspace_bytes()";
     case TTT_MLP_ERR_SCRATCH: return "ttt_mlp: ttt_mlp_fwd_launch_static serves at most 8 (batch, head) pairs (B*NH <= 8): its workspace is a fixed array in device memory";
     default: return hipGetErrorString(static_cast<hipError_t>(code));
   }

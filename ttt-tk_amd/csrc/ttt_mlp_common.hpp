@@ -432,6 +432,7 @@ TTT_DEV void eta_to_lds(gptr_t g, unsigned off, unsigned char* dst, int v, int l
 // A wait that sees no progress for `limit` ticks of the 100 MHz clock (20 s unless the host says otherwise)
 // raises the status word and makes all workgroups of the launch leave, so every wave always exits.
 TTT_DEV bool wait_at_least(int* word, int target, int* status, int* s_flag, uint64_t limit) {
+  __syncthreads();   // every wave has read the flag's last value (waits follow one another, here and in wait_for_pace)
   if (threadIdx.x == 0) {
     int ok = 1;
     const uint64_t t0 = wall_clock64();

@@ -15,7 +15,11 @@ For each workload it runs `python3 bench.py --workload W ...` under rocprofv3 fi
 and writes profiles/ttt_mlp_<W>_counters.json with, per TTT-MLP kernel: average duration, HBM bytes read / written
 per launch and the GB/s they amount to, MFMA-pipe busy %, vector-ALU busy %, the share of LDS-pipeline cycles lost
 to bank conflicts, the share of wave cycles spent waiting, instruction counts, waves per SIMD and LDS bytes per
-workgroup.  `bench.py` takes `roofline.traffic` from that file.
+workgroup; and per launch (`launches`: forward / backward, summed over the kernels it is made of) the algorithmic
+FLOPs and bytes, the fraction of the bf16 MFMA peak, measured HBM bytes per (batch, head, mini-batch) unit and their
+ratio to the algorithmic bytes, and vector-ALU / MFMA / LDS instructions per unit.  The file carries the sha256 of the
+kernel sources it was measured on (`kernel_sources_sha256`) and the git head; `bench.py` takes `roofline.traffic`
+from it only if that digest matches the sources it runs.
 
 Derived figures (SQ_* cycle counters tick once per 4 clocks; a 32x32x16 MFMA occupies the matrix pipe of its SIMD
 for 32 clocks; every workgroup has 8 waves on the 4 SIMDs of one CU, which its LDS use fills):
@@ -58,7 +62,7 @@ def run_pass(workload: str, tag: str, prof_args, bench_args, raw_dir: str, limit
     out_dir = os.path.join(raw_dir, f"{workload}_{tag}")
     os.makedirs(out_dir, exist_ok=True)
     cmd = ["rocprofv3", *prof_args, "--output-format", "csv", "-d", out_dir, "-o", workload, "--",
-           "python3", os.path.join(ROOT, "bench.py"), "--workload", workload, "--no-cpu-baseline", *bench_args]
+           "python3", os.path.join(ROOT, "bench.py"), "--workload", workload, "--only", "--no-cpu-baseline", *bench_args]
     env = dict(os.environ, TMPDIR="/tmp")
     print("+", " ".join(cmd), flush=True)
     with open(os.path.join(out_dir, "run.log"), "w") as log:
@@ -125,6 +129,36 @@ def kernel_geometry():
     return geo
 
 
+# Algorithmic work of one launch: only the 64x64x256 contractions count as FLOPs (7 per mini-batch and (batch, head)
+# in the forward, 21 in the backward: 7 replayed + 14 new); the bytes are the operator's inputs and outputs of a
+# mini-batch (the backward's four accumulating outputs are read and written) plus the checkpoints, once per group.
+G_FLOP = 2 * 64 * 64 * 256
+PEAK_BF16_TFLOPS = 2516.6
+PEAK_HBM_GBS = 8000.0
+SHAPES = {"c2": (1, 48, 256, 16), "c3": (1, 48, 256, 16), "c4": (1, 48, 4096, 64), "c5": (8, 48, 512, 32)}   # B, NH, NC, cgs
+
+
+def algorithmic(workload: str, which: str):
+    B, NH, NC, cgs = SHAPES[workload]
+    units = B * NH * NC
+    if which == "fwd":
+        return dict(units=units, flop=7 * G_FLOP * units, bytes=units * (32896 + 132352 / cgs))
+    return dict(units=units, flop=21 * G_FLOP * units, bytes=units * (57600 + 24576 + 132352 / cgs))
+
+
+def sources_digest() -> str:
+    """sha256 over the kernel sources (the same digest bench.py checks before it quotes the traffic of a summary)."""
+    import hashlib
+    h = hashlib.sha256()
+    csrc = os.path.join(HERE, "csrc")
+    for name in sorted(os.listdir(csrc)):
+        if name.endswith((".hip", ".hpp")):
+            h.update(name.encode())
+            with open(os.path.join(csrc, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()
+
+
 def profile(workload: str, raw_dir: str, limit_s: int):
     dirs = {tag: run_pass(workload, tag, pa, ba, raw_dir, limit_s) for tag, pa, ba in PASSES}
     stats = kernel_stats(dirs["trace"])
@@ -154,6 +188,7 @@ def profile(workload: str, raw_dir: str, limit_s: int):
             e["hbm_write_bytes"] = sum(wr[0]) / len(wr[0]) * 1024 * cal["write"]["factor"]
             e["hbm_bytes"] = e["hbm_read_bytes"] + e["hbm_write_bytes"]
             e["hbm_gbs"] = e["hbm_bytes"] / e["avg_ns"]
+            e["hbm_frac_of_peak"] = e["hbm_gbs"] / PEAK_HBM_GBS
         c = {}
         for k, v in sq.items():
             if short_name(k) == key:
@@ -166,9 +201,37 @@ def profile(workload: str, raw_dir: str, limit_s: int):
             e["lds_conflict_share"] = c["SQ_LDS_BANK_CONFLICT"] / max(c["SQ_ACTIVE_INST_LDS"] * 4, 1)
             e["wait_share"] = c["SQ_WAIT_ANY"] / c["SQ_WAVE_CYCLES"]
         kernels[key] = e
-    return dict(workload=workload, device="MI355X (gfx950), one GPU", calibration=cal, kernels=kernels,
+    # Roofline per launch (forward / backward): a launch may be made of two kernels (pairs beyond a multiple of the
+    # CU count run with more workgroups each), so time, bytes and instruction counts are summed over its kernels.
+    launches = {}
+    for which in ("fwd", "bwd"):
+        ks = [e for k, e in kernels.items() if f"ttt_mlp_{which}" in k]
+        if not ks:
+            continue
+        alg = algorithmic(workload, which)
+        ms = sum(e["avg_ns"] for e in ks) / 1e6
+        L = dict(kernels=[k for k in kernels if f"ttt_mlp_{which}" in k], launch_ms=ms, units=alg["units"],
+                 algorithmic_flop=alg["flop"], algorithmic_bytes=alg["bytes"],
+                 achieved_tflops=alg["flop"] / (ms * 1e-3) / 1e12)
+        L["frac_of_bf16_mfma_peak"] = L["achieved_tflops"] / PEAK_BF16_TFLOPS
+        if all("hbm_bytes" in e for e in ks):
+            L["hbm_bytes"] = sum(e["hbm_bytes"] for e in ks)
+            L["hbm_bytes_per_unit"] = L["hbm_bytes"] / alg["units"]
+            L["traffic_over_algorithmic"] = L["hbm_bytes"] / alg["bytes"]
+            L["hbm_gbs"] = L["hbm_bytes"] / (ms * 1e6)
+        if all("counters" in e for e in ks):
+            for cn, label in (("SQ_INSTS_VALU", "valu_insts_per_unit"), ("SQ_INSTS_MFMA", "mfma_insts_per_unit"),
+                              ("SQ_INSTS_LDS", "lds_insts_per_unit")):
+                if all(cn in e["counters"] for e in ks):
+                    L[label] = sum(e["counters"][cn] for e in ks) / alg["units"]
+        launches[which] = L
+    try:
+        head = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True, text=True).stdout.strip()
+    except OSError:
+        head = ""
+    return dict(workload=workload, launches=launches, kernel_sources_sha256=sources_digest(), git_head=head, device="MI355X (gfx950), one GPU", calibration=cal, kernels=kernels,
                 commands=[" ".join(["rocprofv3", *pa, "--output-format csv -d <raw>/" + f"{workload}_{tag}", "-o", workload, "--",
-                                    "python3 bench.py --workload", workload, "--no-cpu-baseline", *ba]) for tag, pa, ba in PASSES],
+                                    "python3 bench.py --workload", workload, "--only --no-cpu-baseline", *ba]) for tag, pa, ba in PASSES],
                 note="each pass is its own run from /tmp with TMPDIR=/tmp; HBM bytes = counter KiB x 1024 x calibration factor")
 
 

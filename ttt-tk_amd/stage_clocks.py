@@ -77,8 +77,8 @@ def main() -> int:
     from bench import make_device_inputs
     from build import STAGES_LIB, LIB
 
-    if not os.path.exists(STAGES_LIB):
-        raise SystemExit(f"{STAGES_LIB} is missing: run  python ttt-tk_amd/build.py --stages  first")
+    if not os.path.exists(STAGES_LIB) or os.path.getmtime(STAGES_LIB) < os.path.getmtime(LIB):
+        raise SystemExit(f"{STAGES_LIB} is missing or older than the product library: run  python ttt-tk_amd/build.py --stages  first")
     header = open(os.path.join(HERE, "csrc", "ttt_mlp_kernels.hpp")).read()
     fwd_names, bwd_names = stage_names(header, "FwdStage"), stage_names(header, "BwdStage")
     B, NH, NC, cgs, eta_std = WORKLOADS[a.workload]

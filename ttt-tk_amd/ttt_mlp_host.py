@@ -175,3 +175,16 @@ def ttt_mlp_backward(XQ, XK, XV, last_eta, ttt_norm_weight, ttt_norm_bias, check
 def ttt_mlp(XQ, XK, XV, last_eta, ttt_norm_weight, ttt_norm_bias, W1, b1, W2, b2, checkpoint_group_size):
     """Differentiable call: see TTTMLPFunction."""
     return TTTMLPFunction.apply(XQ, XK, XV, last_eta, ttt_norm_weight, ttt_norm_bias, W1, b1, W2, b2, checkpoint_group_size)
+
+
+def workspace_bytes(B: int, NH: int, cgs: int) -> int:
+    """Bytes of workspace with which `ttt_forward` / `ttt_backward` of this shape can use several workgroups per
+    (batch, head); 0 if the shape runs with one workgroup per pair."""
+    return int(_ext.workspace_bytes(int(B), int(NH), int(cgs)))
+
+
+def set_workspace(ws) -> None:
+    """Hand the operators a caller-owned workspace (1-D uint8 GPU tensor, `workspace_bytes(...)` bytes or more): they
+    then allocate nothing per call, like the upstream operator, whose every tensor is the caller's
+    (upstream kernels/ttt_backward/ttt.cu:1451-1917).  ``None`` returns to a workspace from torch's allocator per call."""
+    _ext.set_workspace(ws)
