@@ -1,13 +1,15 @@
 """The benchmark configurations (C2 - C5) at their full sizes on the GPU.
 
-C2/C3 (16,384 tokens, 48 heads) are checked against the CPU oracle for every head.  C4 (262,144 tokens)
-and C5 (8 x 48 recurrences) run in full on the GPU; the oracle, which needs minutes for them, checks a
-subset of the independent (batch, head) recurrences (4 heads of C4, 6 pairs of C5), and size-independent
-properties cover the rest: exact linearity in the upstream gradients, zero gradients for zero upstream
-gradients, independence of heads, and agreement between two checkpoint group sizes.
+C2/C3 (16,384 tokens, 48 heads) and C4 (262,144 tokens, 48 heads) are checked against the CPU oracle for every
+head, as the upstream harness compares every head (kernels/ttt_backward/matching.py:667-705); C5 (8 x 48
+recurrences) on 48 of its (batch, head) pairs, every head once and every batch element six times.  C4 and C5 are
+also drawn with a second seed (8 heads / 16 pairs against the oracle).  Size-independent properties cover the rest:
+exact linearity in the upstream gradients, zero gradients for zero upstream gradients, independence of heads, and
+agreement between two checkpoint group sizes.
 
 Bar, on every configuration: max|hw - ref| / max|ref| <= 2e-2 and cosine >= 0.9999 per tensor (Out,
-checkpoints, ten gradients), reference = fp32 oracle on the same bf16-rounded inputs.
+checkpoints, ten gradients), reference = fp32 oracle on the same bf16-rounded inputs.  On C4 and C5 the tensor is
+all compared (batch, head) pairs together; each pair by itself is reported too and held to 3e-2 / 0.9998.
 
 Inputs: the benchmark's distributions, except that b1, b2 and the norm weight / bias are not the trivial
 zeros / ones / zeros here (b ~ N(0, 0.02), weight ~ 1 + N(0, 0.1), bias ~ N(0, 0.1)), so that the bias and
@@ -23,7 +25,8 @@ from oracle import ttt_mlp_oracle as orc
 
 pytestmark = pytest.mark.gpu
 
-MAX_REL, MIN_COS = 2e-2, 0.9999
+MAX_REL, MIN_COS = 2e-2, 0.9999              # the bar, per tensor
+PAIR_MAX_REL, PAIR_MIN_COS = 3e-2, 0.9998    # any single (batch, head) pair of C4 / C5 taken by itself
 FWD_KEYS = ("XQ", "XK", "XV", "last_eta", "ttt_norm_weight", "ttt_norm_bias", "W1", "b1", "W2", "b2")
 UP_KEYS = ("grad_L_W1_last", "grad_L_b1_last", "grad_L_W2_last", "grad_L_b2_last", "grad_L_XQW_mini_batch")
 GRADS = ("grad_L_ttt_norm_weight", "grad_L_ttt_norm_bias", "grad_L_W1_init", "grad_L_b1_init", "grad_L_W2_init",
@@ -105,12 +108,31 @@ def compare(tag, hw, ref, failures, bar=True):
 
 
 def check_subset(case, t, r, cgs, pairs, backward=True):
+    """The (batch, head) recurrences of `pairs` against the oracle.  The bar applies to each tensor as a whole (all
+    compared pairs together: the statistic the parity bar is stated for, and what the upstream harness prints,
+    kernels/ttt_backward/matching.py:9-40); every pair is also reported by itself, with the worst of them per tensor,
+    and held to PAIR_MAX_REL / PAIR_MIN_COS: the per-head tensors of the bias and norm gradients have 64 - 256
+    elements, whose cosine scatters from head to head around the whole tensor's."""
     torch.set_num_threads(min(16, os.cpu_count() or 1))
     failures = []
     ref = oracle(cpu_pairs(t, pairs), cgs, backward)
+    hw_all = {k: torch.cat([r[k][b:b + 1, h:h + 1] for b, h in pairs], dim=1).float().cpu() for k in ref}
+    worst = {}
     for i, (b, h) in enumerate(pairs):
-        hw = {k: r[k][b:b + 1, h:h + 1].float().cpu() for k in ref}
-        compare(f"{case} (b={b},h={h})", hw, {k: v[:, i:i + 1] for k, v in ref.items()}, failures)
+        hw = {k: v[:, i:i + 1] for k, v in hw_all.items()}
+        ri = {k: v[:, i:i + 1] for k, v in ref.items()}
+        compare(f"{case} (b={b},h={h})", hw, ri, [], bar=False)
+        for k, v in ri.items():
+            if v.abs().max() > 0:
+                st = orc.parity_stats(hw[k], v)
+                w = worst.setdefault(k, [0.0, 1.0])
+                w[0], w[1] = max(w[0], st["max_rel"]), min(w[1], st["cosine"])
+    for k, (mr, cs) in worst.items():
+        ok = mr <= PAIR_MAX_REL and cs >= PAIR_MIN_COS
+        report(f"{case} worst single pair of {len(pairs)} {k:24s} max_rel={mr:.3e} cos={cs:.6f}{'' if ok else '  <-- FAIL'}")
+        if not ok:
+            failures.append((case, "worst pair", k, mr, cs))
+    compare(f"{case} all {len(pairs)} pairs", hw_all, ref, failures)
     assert not failures, failures
 
 
@@ -143,7 +165,7 @@ def test_c4_long_sequence_262k_tokens():
     r = run(t, 64)
     for k in GRADS + ("Out",):
         assert bool(torch.isfinite(r[k].float()).all()), k
-    check_subset("C4", t, r, 64, [(0, 0), (0, 13), (0, 30), (0, 47)])
+    check_subset("C4", t, r, 64, [(0, h) for h in range(48)])
     # exact linearity: doubling every upstream gradient doubles every output gradient bit for bit
     t2 = dict(t)
     for k in UP_KEYS:
@@ -165,7 +187,7 @@ def test_c5_fill_the_chip_384_recurrences():
     r = run(t, 32)
     for k in GRADS + ("Out",):
         assert bool(torch.isfinite(r[k].float()).all()), k
-    check_subset("C5", t, r, 32, [(0, 0), (1, 40), (3, 17), (4, 5), (6, 29), (7, 47)])
+    check_subset("C5", t, r, 32, [((5 * h + h // 8) % 8, h) for h in range(48)])
     # zero upstream gradients give zero gradients everywhere
     tz = dict(t)
     for k in UP_KEYS:
@@ -179,3 +201,16 @@ def test_c5_fill_the_chip_384_recurrences():
     rf = run(tf, 32)
     for k in GRADS + ("Out",):
         assert torch.equal(rf[k].flip(1), r[k]), k
+
+
+def test_c4_and_c5_second_seed():
+    """The same two configurations drawn with another seed: the margin to the bar must not hang on one draw."""
+    report("case C4 seed 1: forward+backward B=1 NH=48 NC=4096 cgs=64")
+    t = device_inputs(1, 48, 4096, 1.0, seed=1)
+    r = run(t, 64)
+    check_subset("C4 seed 1", t, r, 64, [(0, h) for h in (1, 7, 12, 22, 28, 35, 41, 46)])
+    del t, r
+    report("case C5 seed 1: forward+backward B=8 NH=48 NC=512 cgs=32, wide eta")
+    t = device_inputs(8, 48, 512, 2.0, seed=1)
+    r = run(t, 32)
+    check_subset("C5 seed 1", t, r, 32, [(i % 8, 3 * i) for i in range(16)])

@@ -863,8 +863,20 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           LANE_VARS;
           AccT<1, 2> z1b;
           acc_init_rows_lds(z1b, s_b1w, h);
-          mma_jit<4>(z1b, [&](int, int s) { return piece_state(W1s, 0, s); },
-                     [&](int i, int s) { return xpiece_rows(s_xq, tb[i], s, c, h); });
+          // W1 after the step in two terms: its rounding pattern persists over many mini-batches, so the error it
+          // leaves in Z1_bar - and through it in every gradient the output branch feeds - does not average out
+#pragma unroll
+          for (int s = 0; s < 4; s++) {
+            bf16x8 wh, wl, xq[2];
+            split8(W1s.b[s >> 1][0], s & 1, wh, wl);
+#pragma unroll
+            for (int i = 0; i < 2; i++) xq[i] = xpiece_rows(s_xq, tb[i], s, c, h);
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+              z1b.b[0][i] = MFMA(wl, xq[i], z1b.b[0][i]);
+              z1b.b[0][i] = MFMA(wh, xq[i], z1b.b[0][i]);
+            }
+          }
           bf16x8 x2bQ[2][2];
           WAVE_SYNC();   // the weight step's readers of T0 are done
 #pragma unroll
@@ -950,8 +962,29 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
             LANE_VARS;
             AccT<1, 2> gz1b;   // (gZ2_bar W2^T) * gelu'(Z1_bar): rows hid, lane = tok
             acc_zero(gz1b);
-            mma_jit<4>(gz1b, [&](int, int s) { return w2a[s]; },
-                       [&](int i, int s) { return piece_rows<LDX>(s_a, tb[i], s, c, h); });
+            // W2 after the step in two terms here as well (see W1 above): the low-order term goes through T2 like the
+            // high-order one went through T1 for the image
+#pragma unroll
+            for (int fb = 0; fb < 2; fb++)
+#pragma unroll
+              for (int s = 0; s < 2; s++) {
+                bf16x8 ph, pl;
+                split8(W2s.b[0][fb], s, ph, pl);
+                store_piece_rows<LDH>(T2, fb, s, c, h, pl);
+              }
+            WAVE_SYNC();
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+              const bf16x8 wl = piece_tr<LDH>(T2, 0, s, lane);
+              bf16x8 gb[2];
+#pragma unroll
+              for (int i = 0; i < 2; i++) gb[i] = piece_rows<LDX>(s_a, tb[i], s, c, h);
+#pragma unroll
+              for (int i = 0; i < 2; i++) {
+                gz1b.b[0][i] = MFMA(wl, gb[i], gz1b.b[0][i]);
+                gz1b.b[0][i] = MFMA(w2a[s], gb[i], gz1b.b[0][i]);
+              }
+            }
 #pragma unroll
             for (int i = 0; i < 2; i++)
 #pragma unroll
