@@ -230,10 +230,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=3)
     ap.add_argument("--warmup", type=int, default=1)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c4")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c4")   # ("custom" is what --shape registers)
     ap.add_argument("--only", action="store_true",
                     help="time the named workload alone (without this, a c4 run also times the fill-the-chip workload c5 "
                          "and reports it in a \"c5\" block of the same JSON line)")
+    ap.add_argument("--shape", default=None, metavar="B,NH,NC,CGS",
+                    help="time this shape instead of a named workload (implies --only; the line's metric names the shape); "
+                         "for launch-plan measurements at head counts other than the benchmark's")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--overwrite", action="store_true",
                     help="let ttt_backward overwrite grad_L_XQ / XK / XV / last_eta instead of adding to them "
@@ -253,6 +256,11 @@ def main():
 
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
+    if a.shape:
+        B, NH, NC, cgs = (int(x) for x in a.shape.split(","))
+        a.workload, a.only, a.no_cpu_baseline = "custom", True, True
+        WORKLOADS["custom"] = (B, NH, NC, cgs, 1.0, f"fwd+bwd B={B} NH={NH} {NC * 64} tokens/sequence cgs={cgs}")
+        METRICS["custom"] = f"TTT-MLP fwd+bwd tokens/sec on 1 MI355X (B={B},NH={NH},{NC * 64} tok/seq); % bf16 MFMA peak"
     res = run_workload(a.workload, a.steps, a.warmup, a.overwrite, a.no_overlap, a.calibrate_copy)
     out = {
         "metric": res["metric"], "value": res["value"], "unit": res["unit"], "n_gpus": 1, "steps": a.steps,

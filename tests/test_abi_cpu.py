@@ -187,7 +187,10 @@ def test_launch_plan_keeps_waiting_workgroups_within_the_device(lib):
         assert lib.ttt_mlp_launch_plan(which, ctypes.c_longlong(pairs), cus, ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)) == 0
         return a.value, b.value, c.value
     assert plan(1, 48, 256) == (0, 48, 5)          # the metric's configuration: four workgroups per pair + one that fetches ahead
+    assert plan(1, 32, 256) == (0, 32, 5)
     assert plan(1, 56, 256) == (0, 56, 4)          # a fifth would not fit
+    assert plan(1, 64, 256) == (0, 64, 4)          # four per pair fill the device exactly
+    assert plan(1, 128, 256) == (0, 128, 2)
     assert plan(1, 44, 256) == (0, 44, 4)          # not a multiple of 8 pairs: the fifth would not share the walk's XCD
     assert plan(1, 72, 256) == (0, 72, 3)
     assert plan(1, 96, 256) == (0, 96, 2)
