@@ -181,7 +181,9 @@ int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* args, void* workspace,
  * and serves at most 8 (batch, head) pairs: B*NH > 8 returns TTT_MLP_ERR_SCRATCH, a device without room
  * for two workgroups per pair TTT_MLP_ERR_NO_ROOM, before anything is enqueued.  Every call on a GPU uses
  * that GPU's one array: calls that overlap in time on one GPU (two streams, two threads) race - serialise
- * them.  `sticky_word` (may be NULL): a device int owned by the caller; as ttt_mlp_status_accumulate, the
+ * them.  The launch goes to the current device (make it the stream's); the first call on a device looks the
+ * array's address up, which is not a stream operation: a caller that captures the call into a HIP graph makes
+ * one ordinary call on that device first.  `sticky_word` (may be NULL): a device int owned by the caller; as ttt_mlp_status_accumulate, the
  * call enqueues `if (status != 0) *sticky_word = 1` behind the kernels. */
 int ttt_mlp_fwd_launch_static(const ttt_mlp_fwd_args* args, int* sticky_word, void* stream);
 

@@ -1,5 +1,7 @@
 // extern "C" entry points declared in include/ttt_mlp.h: argument validation on the host, then
 // one asynchronous kernel launch.  Nothing here allocates or synchronises.
+#include <atomic>
+
 #include "../../include/ttt_mlp.h"
 #include "ttt_mlp_kernels.hpp"
 
@@ -376,20 +378,22 @@ constexpr size_t static_scratch_bytes() {
 static __device__ __align__(256) unsigned char scratch[static_scratch_bytes()];   // 32.6 MiB
 
 constexpr int MAX_DEVICES = 64;
-void* g_scratch_ptr[MAX_DEVICES] = {};   // address of `scratch` on each device, looked up at the first call there
+// address of `scratch` on each device, looked up at the first call there; host threads may race to the first
+// call - every one of them finds the same address, so an atomic slot per device is all the guard it needs
+std::atomic<void*> g_scratch_ptr[MAX_DEVICES] = {};
 
 // The current device's copy of the array (the device that the launch goes to).  Looked up once per device.
 int static_scratch(void** ptr) {
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev)) return static_cast<int>(e);
   if (dev < 0 || dev >= MAX_DEVICES) return TTT_MLP_ERR_BAD_ARG;
-  if (g_scratch_ptr[dev] == nullptr) {
-    void* p = nullptr;
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
     if (hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch))) return static_cast<int>(e);
     if (p == nullptr) return TTT_MLP_ERR_BAD_ARG;
-    g_scratch_ptr[dev] = p;
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
   }
-  *ptr = g_scratch_ptr[dev];
+  *ptr = p;
   return TTT_MLP_OK;
 }
 
