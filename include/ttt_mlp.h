@@ -215,6 +215,13 @@ int ttt_mlp_bwd_export_group0(const ttt_mlp_bwd_args* args, void* stream);
  * for tests of that path (a limit of 1 makes the first wait give up) and for hosts that want a shorter one. */
 void ttt_mlp_set_wait_limit(unsigned long long ticks_100mhz);
 
+/* Workgroups of an overlapped launch wait for each other, so all of them must be resident at once; the launch
+ * plans count on every compute unit the device reports.  A host that runs these launches under a CU mask, or
+ * beside another kernel that holds CUs for their whole duration, says here how many CUs they can count on
+ * (process-wide; 0 = all the device reports, the default): shapes that no longer fit run with one workgroup per
+ * (batch, head), and ttt_mlp_*_workspace_bytes() follow.  No counterpart in the reference. */
+void ttt_mlp_set_compute_units(int compute_units);
+
 /* Human-readable text for a return code of the two launchers. */
 const char* ttt_mlp_error_string(int code);
 

@@ -35,7 +35,7 @@ def test_header_declares_the_expected_entry_points():
     assert declared_functions() == ["ttt_mlp_abi_version", "ttt_mlp_bwd_export_group0", "ttt_mlp_bwd_launch", "ttt_mlp_bwd_launch_overlapped",
                                     "ttt_mlp_bwd_status_offset", "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_error_string",
                                     "ttt_mlp_fwd_launch", "ttt_mlp_fwd_launch_overlapped", "ttt_mlp_fwd_launch_static", "ttt_mlp_fwd_status_offset",
-                                    "ttt_mlp_fwd_workspace_bytes", "ttt_mlp_kernel_info", "ttt_mlp_launch_plan", "ttt_mlp_set_wait_limit",
+                                    "ttt_mlp_fwd_workspace_bytes", "ttt_mlp_kernel_info", "ttt_mlp_launch_plan", "ttt_mlp_set_compute_units", "ttt_mlp_set_wait_limit",
                                     "ttt_mlp_status_accumulate"]
 
 

@@ -70,3 +70,34 @@ def test_operators_allocate_nothing_with_a_caller_workspace():
             ext.set_workspace(torch.zeros(16, dtype=torch.float32, device=dev))
     finally:
         host.set_workspace(None)
+
+
+def test_compute_unit_budget_turns_the_waiting_launches_off():
+    """Workgroups that wait for each other must all be resident; a host that cannot promise the whole device says how
+    many CUs there are, and shapes that no longer fit run with one workgroup per (batch, head) - same results."""
+    import test_time_training as ext
+    import ttt_mlp_host as host
+    dev = torch.device("cuda:0")
+    B, NH, NC, cgs = 1, 8, 12, 4
+    print(f"case B={B} NH={NH} NC={NC} cgs={cgs}", flush=True)
+    d = orc.make_inputs(B, NH, NC, seed=6)
+    t = {k: d[k].to(dev).contiguous() for k in FWD_KEYS + UP_KEYS}
+    t.update(host.alloc_forward_buffers(B, NH, NC, cgs, dev))
+    t.update(host.alloc_backward_buffers(B, NH, NC, cgs, dev))
+    ref = _run(host, t, cgs)
+    assert ext.last_forward_mode() == 1 and ext.last_backward_mode() == 1
+    try:
+        ext.set_compute_units(15)             # 2 x 8 workgroups do not fit 15 CUs
+        assert host.workspace_bytes(B, NH, cgs) == 0
+        got = _run(host, t, cgs)
+        assert ext.last_forward_mode() == 0 and ext.last_backward_mode() == 0
+        for k, r in ref.items():
+            assert torch.equal(got[k], r), k
+        ext.set_compute_units(16)             # two per pair fit, more do not
+        assert host.workspace_bytes(B, NH, cgs) > 0
+        got = _run(host, t, cgs)
+        assert ext.last_forward_mode() == 1 and ext.last_backward_mode() == 1
+        for k, r in ref.items():
+            assert torch.equal(got[k], r), k
+    finally:
+        ext.set_compute_units(0)

@@ -348,6 +348,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "the device's free memory; a call whose shape needs more than the tensor holds, or that runs on another device, "
         "uses one workgroup per (batch, head).  The contents are scratch; calls that overlap in time must not share it.  "
         "None returns to the default (workspace from torch's caching allocator per call).");
+  m.def("set_compute_units", [](int n) { ttt_mlp_set_compute_units(n); },
+        "CUs the multi-workgroup launches may count on (their workgroups wait for each other and must all be resident): "
+        "say so when the process runs under a CU mask or beside a kernel that holds CUs; 0 (default) = all of the device.");
   m.def("last_forward_mode", []() { return g_last_forward_mode; },
         "0: the last ttt_forward used one workgroup per (batch, head); 1: two; -1: none yet.");
   m.def("last_backward_mode", []() { return g_last_backward_mode; },

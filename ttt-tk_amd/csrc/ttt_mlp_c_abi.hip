@@ -27,6 +27,7 @@ int check_sizes(int B, int NH, int NC, int K, int cgs) {
 }
 
 unsigned long long g_wait_limit = 2000000000ull;   // 20 s of the 100 MHz clock
+int g_cu_budget = 0;   // CUs the caller says these launches can count on (0: all the device reports)
 
 inline const __bf16* bf(const uint16_t* p) { return reinterpret_cast<const __bf16*>(p); }
 inline __bf16* bf(uint16_t* p) { return reinterpret_cast<__bf16*>(p); }
@@ -36,6 +37,8 @@ inline __bf16* bf(uint16_t* p) { return reinterpret_cast<__bf16*>(p); }
 extern "C" int ttt_mlp_abi_version(void) { return TTT_MLP_ABI_VERSION; }
 
 extern "C" void ttt_mlp_set_wait_limit(unsigned long long ticks_100mhz) { g_wait_limit = ticks_100mhz; }
+
+extern "C" void ttt_mlp_set_compute_units(int compute_units) { g_cu_budget = compute_units > 0 ? compute_units : 0; }
 
 extern "C" const char* ttt_mlp_error_string(int code) {
   switch (code) {
@@ -170,6 +173,7 @@ LaunchPlan plan_launches(long long BH, bool three_way) {
   int dev = 0, cus = 0;
   if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
     cus = 0;
+  if (g_cu_budget > 0 && g_cu_budget < cus) cus = g_cu_budget;
   return plan_for(BH, cus, three_way);
 }
 
