@@ -729,6 +729,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           ln_store_g<ROLE != 0>(bGZ2, vln, j * TILE_BYTES, gx);
 #pragma unroll
           for (int e = 0; e < 8; e++) gx[e] *= neg_eta;                             // G2, in two terms (the second in
+          ln_token_sum_store(s_deta + v * CS, gx, lane, f0);   // b2's step: this wave's share (s_deta is the walk's otherwise)
           {                                                                          // the tile gZ2_bar takes later)
             bf16x8 gh, gl;
             split8(gx, gh, gl);
@@ -738,6 +739,13 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
           if ((lane & 7) == 0) g_stf(bSDF, vtok, j * (CS * 4), sd);
         }
         __syncthreads();
+        if (v == 0) {   // b2 += sum over the tokens of G2: the eight waves' fp32 shares in a fixed order (next read: the output LayerNorm)
+          LANE_VARS;
+          float b = s_b2[lane];
+#pragma unroll
+          for (int u = 0; u < BW_NWAVE; u++) b += s_deta[u * CS + lane];
+          s_b2[lane] = b;
+        }
         TTT_STAGE(BS_R_LN);
         // G1 = (W2 G2^T) * gelu'(Z1)  (rows hid, lane = tok) -> T1 rows [tok][hid]; weight step
         {
@@ -828,10 +836,6 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
               W2s.b[0][fb] = MFMA(xh, gl[fb], W2s.b[0][fb]);
               W2s.b[0][fb] = MFMA(xh, gh[fb], W2s.b[0][fb]);
             }
-          }
-          if (v < 2) {
-            lds_rowsum_add_jit(s_b2 + 32 * v, [&](int s) { return piece_tr<LDX>(s_a, v, s, lane); }, ones, c, h);
-            lds_rowsum_add_jit(s_b2 + 32 * v, [&](int s) { return piece_tr<LDX>(s_gz2, v, s, lane); }, ones, c, h);
           }
           WAVE_SYNC();   // this wave's readers of T1 / T2 are done
         }

@@ -133,6 +133,24 @@ TTT_DEV float half_sum2(float s01, float s23) {
   return a + b;
 }
 
+// vec[f0 + e] = sum over this wave's 8 LayerNorm tokens of x[e], for a wave whose lane l holds token l / 8 and the 8
+// features f0 = 8 (l % 8) ... of it.  The tokens sit in the lanes that share lane % 8: lanes 8 apart inside a row of
+// 16 (one rotation), then the four rows, two values per swap: in the end row r of one register holds the total of
+// x[r], of the other that of x[4 + r], and lanes 0..7 of every row store their two totals.  Fixed order, fp32.
+TTT_DEV void ln_token_sum_store(float* vec, const float (&x)[8], int lane, int f0) {
+  float y[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++)
+    y[e] = x[e] + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x[e]), 0x128, 0xF, 0xF, false));  // row_ror:8
+  const float lo = half_sum2(row_pair_sum2(y[0], y[1]), row_pair_sum2(y[2], y[3]));
+  const float hi = half_sum2(row_pair_sum2(y[4], y[5]), row_pair_sum2(y[6], y[7]));
+  if ((lane & 8) == 0) {
+    float* d = vec + f0 + (lane >> 4);
+    d[0] = lo;
+    d[4] = hi;
+  }
+}
+
 // ---------------------------------------------------------------------------- shape-generic tiles
 // Tiles whose extent along the hidden dimension is one 32-wide block (a wave that owns 32 hidden
 // columns) mix with 64-wide token / feature extents, so blocks and k-steps are template parameters.

@@ -62,7 +62,8 @@ constexpr int SM_B2 = SM_B1 + HID * 4;
 constexpr int SM_ETA = SM_B2 + FD * 4;
 constexpr int SM_GAM = SM_ETA + CS * 4;
 constexpr int SM_BET = SM_GAM + FD * 4;
-constexpr int SM_FLAG = SM_BET + FD * 4;                 // outcome of a wait on the other workgroup
+constexpr int SM_B2P = SM_BET + FD * 4;                  // per wave: the sum of G2 over its 8 LayerNorm tokens (the step of b2)
+constexpr int SM_FLAG = SM_B2P + FW_NWAVE * FD * 4;      // outcome of a wait on the other workgroup
 constexpr int SM_FWD_BYTES = SM_FLAG + 16;
 static_assert(SM_FWD_BYTES <= 160 * 1024, "forward LDS budget");
 
@@ -241,7 +242,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
   // ---- state -> registers
   AccT<2, 1> W1s;
   AccT<1, 2> W2s;
-  float b1L;      // b1 of hidden column hid0 + c; b2 lives in LDS (fp32) and is updated there by waves 0 and 1
+  float b1L;      // b1 of hidden column hid0 + c; b2 lives in LDS (fp32) and is updated there by wave 0
   {
     const gptr_t W1 = gbuf(p.W1 + (size_t)bh * FD * HID), W2 = gbuf(p.W2 + (size_t)bh * HID * FD);
 #pragma unroll
@@ -260,9 +261,6 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
       s_bet[tid] = p.ttt_norm_bias[head * FD + tid];
     }
   }
-  bf16x8 ones;
-#pragma unroll
-  for (int j = 0; j < 8; j++) ones[j] = (bf16)1.0f;
 
   // HBM addressing: scalar base of this (batch, head) + scalar offset of the mini-batch + lane offset
   const size_t x_base = uni64((size_t)bh * p.NC * (CS * FD));
@@ -301,7 +299,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
     }
 
     // ROLE 1 ends a mini-batch without a barrier: this one makes the inputs staged at the end of the last mini-batch
-    // visible, and b2 as waves 0 and 1 left it
+    // visible
     if constexpr (ROLE == 1) {
       if (mb > 0) __syncthreads();
     }
@@ -445,6 +443,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
       bf16x8 o, ol;
 #pragma unroll
       for (int e = 0; e < 8; e++) gx[e] = (FD * gx[e] - s1 - z[e] * s2) * scale;
+      ln_token_sum_store(reinterpret_cast<float*>(smem + SM_B2P) + v * FD, gx, lane, f0);   // b2's step, this wave's share
       split8(gx, o, ol);
       lds_put16(s_g2 + tok * FLD + f0, __builtin_bit_cast(u32x4, o));
       lds_put16(s_g2l + tok * FLD + f0, __builtin_bit_cast(u32x4, ol));
@@ -453,6 +452,17 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
     __syncthreads();
 
     TTT_STAGE(FS_LN_BARRIER);
+    // b2 += sum over the tokens of G2: the eight waves' fp32 shares, added in a fixed order by wave 0 (read again
+    // after the next workgroup barrier at the earliest)
+    if (v == 0) {
+      LANE_VARS;
+      const float* part = reinterpret_cast<const float*>(smem + SM_B2P);
+      float b = s_b2[lane];
+#pragma unroll
+      for (int u = 0; u < FW_NWAVE; u++) b += part[u * FD + lane];
+      s_b2[lane] = b;
+      if constexpr (ROLE == 1) gB[HID + lane] = b;
+    }
     // ---- G1 = (G2 W2^T) * gelu'(Z1);  state += X^T G
     {
       LANE_VARS;
@@ -527,16 +537,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
       }
       TTT_STAGE(FS_F4);
       // W2[shard,:] += X2^T G2: X2 chained (two terms), G2 through the transposing read
-      // (lane = F, contraction = tok; two terms); b2 += column sums of G2 (waves 0 and 1, rows 32v..32v+32)
-      f32x16 b2acc;
-      if (v < 2) {
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-          const f32x4 x = *reinterpret_cast<const f32x4*>(s_b2 + 32 * v + 8 * g + 4 * h);
-#pragma unroll
-          for (int e = 0; e < 4; e++) b2acc[4 * g + e] = x[e];
-        }
-      }
+      // (lane = F, contraction = tok; two terms)
 #pragma unroll
       for (int s = 0; s < 4; s++) {
         bf16x8 gh[2], gl[2];
@@ -551,18 +552,6 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
           W2s.b[0][fb] = MFMA(xl, gh[fb], W2s.b[0][fb]);
           W2s.b[0][fb] = MFMA(xh, gl[fb], W2s.b[0][fb]);
           W2s.b[0][fb] = MFMA(xh, gh[fb], W2s.b[0][fb]);
-        }
-        if (v < 2) {
-          b2acc = MFMA(v == 0 ? gl[0] : gl[1], ones, b2acc);
-          b2acc = MFMA(v == 0 ? gh[0] : gh[1], ones, b2acc);
-        }
-      }
-      if (v < 2 && c == 0) {                                           // read after the next workgroup barrier
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-          f32x4 x = {b2acc[4 * g], b2acc[4 * g + 1], b2acc[4 * g + 2], b2acc[4 * g + 3]};
-          *reinterpret_cast<f32x4*>(s_b2 + 32 * v + 8 * g + 4 * h) = x;
-          if constexpr (ROLE == 1) *reinterpret_cast<f32x4*>(gB + HID + 32 * v + 8 * g + 4 * h) = x;
         }
       }
     }
