@@ -90,3 +90,25 @@ def test_bench_and_harness_stamp_the_same_kernel_sources():
     for w in ("c2", "c3", "c4", "c5"):
         assert w in bench.METRICS and w in pc.SHAPES
         assert bench.WORKLOADS[w][:4] == pc.SHAPES[w]
+
+
+def test_launch_summary_adds_up_the_kernels_of_one_launch():
+    """c5's backward is two kernels in a row (one workgroup per pair, then the rest with two each): time, bytes and
+    instruction counts of a launch are their sums, the roofline figures follow from the algorithmic work."""
+    kernels = {
+        "ttt_mlp_bwd_kernel": dict(avg_ns=24e6, hbm_bytes=9e10, counters=dict(SQ_INSTS_VALU=5e9, SQ_INSTS_MFMA=3e8, SQ_INSTS_LDS=8e8)),
+        "ttt_mlp_bwd_split_kernel<1, false>": dict(avg_ns=12e6, hbm_bytes=4.5e10, counters=dict(SQ_INSTS_VALU=3e9, SQ_INSTS_MFMA=1e8, SQ_INSTS_LDS=4e8)),
+        "ttt_mlp_fwd_kernel": dict(avg_ns=10e6),
+    }
+    L = pc.launch_summary("c5", kernels)
+    units = 8 * 48 * 512
+    b = L["bwd"]
+    assert b["kernels"] == ["ttt_mlp_bwd_kernel", "ttt_mlp_bwd_split_kernel<1, false>"] and b["units"] == units
+    assert abs(b["launch_ms"] - 36.0) < 1e-9 and abs(b["hbm_bytes"] - 1.35e11) < 1
+    assert abs(b["achieved_tflops"] - 21 * 2097152 * units / 36e-3 / 1e12) < 1e-6
+    assert abs(b["frac_of_bf16_mfma_peak"] - b["achieved_tflops"] / 2516.6) < 1e-12
+    assert abs(b["traffic_over_algorithmic"] - 1.35e11 / (units * (57600 + 24576 + 132352 / 32))) < 1e-9
+    assert abs(b["valu_insts_per_unit"] - 8e9 / units) < 1e-6 and abs(b["mfma_insts_per_unit"] - 4e8 / units) < 1e-6
+    assert abs(b["hbm_gbs"] - 1.35e11 / 36e6) < 1e-6
+    f = L["fwd"]
+    assert "hbm_bytes" not in f and "valu_insts_per_unit" not in f and abs(f["launch_ms"] - 10.0) < 1e-9

@@ -159,6 +159,34 @@ def sources_digest() -> str:
     return h.hexdigest()
 
 
+def launch_summary(workload: str, kernels: dict) -> dict:
+    """Roofline per launch (forward / backward): a launch may be made of two kernels (pairs beyond a multiple of the CU
+    count run with more workgroups each), so time, bytes and instruction counts are summed over its kernels."""
+    launches = {}
+    for which in ("fwd", "bwd"):
+        ks = [e for k, e in kernels.items() if f"ttt_mlp_{which}" in k]
+        if not ks:
+            continue
+        alg = algorithmic(workload, which)
+        ms = sum(e["avg_ns"] for e in ks) / 1e6
+        L = dict(kernels=[k for k in kernels if f"ttt_mlp_{which}" in k], launch_ms=ms, units=alg["units"],
+                 algorithmic_flop=alg["flop"], algorithmic_bytes=alg["bytes"],
+                 achieved_tflops=alg["flop"] / (ms * 1e-3) / 1e12)
+        L["frac_of_bf16_mfma_peak"] = L["achieved_tflops"] / PEAK_BF16_TFLOPS
+        if all("hbm_bytes" in e for e in ks):
+            L["hbm_bytes"] = sum(e["hbm_bytes"] for e in ks)
+            L["hbm_bytes_per_unit"] = L["hbm_bytes"] / alg["units"]
+            L["traffic_over_algorithmic"] = L["hbm_bytes"] / alg["bytes"]
+            L["hbm_gbs"] = L["hbm_bytes"] / (ms * 1e6)
+        if all("counters" in e for e in ks):
+            for cn, label in (("SQ_INSTS_VALU", "valu_insts_per_unit"), ("SQ_INSTS_MFMA", "mfma_insts_per_unit"),
+                              ("SQ_INSTS_LDS", "lds_insts_per_unit")):
+                if all(cn in e["counters"] for e in ks):
+                    L[label] = sum(e["counters"][cn] for e in ks) / alg["units"]
+        launches[which] = L
+    return launches
+
+
 def profile(workload: str, raw_dir: str, limit_s: int):
     dirs = {tag: run_pass(workload, tag, pa, ba, raw_dir, limit_s) for tag, pa, ba in PASSES}
     stats = kernel_stats(dirs["trace"])
@@ -201,30 +229,7 @@ def profile(workload: str, raw_dir: str, limit_s: int):
             e["lds_conflict_share"] = c["SQ_LDS_BANK_CONFLICT"] / max(c["SQ_ACTIVE_INST_LDS"] * 4, 1)
             e["wait_share"] = c["SQ_WAIT_ANY"] / c["SQ_WAVE_CYCLES"]
         kernels[key] = e
-    # Roofline per launch (forward / backward): a launch may be made of two kernels (pairs beyond a multiple of the
-    # CU count run with more workgroups each), so time, bytes and instruction counts are summed over its kernels.
-    launches = {}
-    for which in ("fwd", "bwd"):
-        ks = [e for k, e in kernels.items() if f"ttt_mlp_{which}" in k]
-        if not ks:
-            continue
-        alg = algorithmic(workload, which)
-        ms = sum(e["avg_ns"] for e in ks) / 1e6
-        L = dict(kernels=[k for k in kernels if f"ttt_mlp_{which}" in k], launch_ms=ms, units=alg["units"],
-                 algorithmic_flop=alg["flop"], algorithmic_bytes=alg["bytes"],
-                 achieved_tflops=alg["flop"] / (ms * 1e-3) / 1e12)
-        L["frac_of_bf16_mfma_peak"] = L["achieved_tflops"] / PEAK_BF16_TFLOPS
-        if all("hbm_bytes" in e for e in ks):
-            L["hbm_bytes"] = sum(e["hbm_bytes"] for e in ks)
-            L["hbm_bytes_per_unit"] = L["hbm_bytes"] / alg["units"]
-            L["traffic_over_algorithmic"] = L["hbm_bytes"] / alg["bytes"]
-            L["hbm_gbs"] = L["hbm_bytes"] / (ms * 1e6)
-        if all("counters" in e for e in ks):
-            for cn, label in (("SQ_INSTS_VALU", "valu_insts_per_unit"), ("SQ_INSTS_MFMA", "mfma_insts_per_unit"),
-                              ("SQ_INSTS_LDS", "lds_insts_per_unit")):
-                if all(cn in e["counters"] for e in ks):
-                    L[label] = sum(e["counters"][cn] for e in ks) / alg["units"]
-        launches[which] = L
+    launches = launch_summary(workload, kernels)
     try:
         head = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True, text=True).stdout.strip()
     except OSError:
