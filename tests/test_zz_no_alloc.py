@@ -1,7 +1,8 @@
 """The forward entry point that allocates nothing (`ttt_mlp_fwd_launch_static`: its workspace is a fixed array in
 the library's device memory) against the entry point it is a variant of (`ttt_mlp_fwd_launch_overlapped` with a
 caller-owned workspace), through the C ABI: bit-identical Out and checkpoints on two calls in a row, the second
-with a smaller input, so that whatever the first call left in the array must not matter."""
+with a smaller input, so that whatever the first call left in the array must not matter; and the same call
+replayed from a captured graph against the eager call."""
 import ctypes
 import os
 
@@ -82,3 +83,54 @@ def test_static_scratch_forward_rejects_more_pairs_than_its_array_serves():
     torch.cuda.synchronize()
     assert t["Out"].float().abs().max() == 0          # nothing was launched
     assert lib.ttt_mlp_fwd_launch_static(None, None, None) == 1001
+
+
+def test_static_scratch_forward_replayed_from_a_captured_graph():
+    """A caller that captures: one ordinary call first (it looks the array's address up and loads the code), then
+    the same call recorded into a graph.  The launch records kernels only (its counters are cleared by a small
+    kernel, not by a memset node).  Every replay, on fresh inputs and with eager work and synchronisations in
+    between, must give what the eager call gives on the same inputs."""
+    import ttt_mlp_host as host
+    lib = ctypes.CDLL(LIB)
+    lib.ttt_mlp_error_string.restype = ctypes.c_char_p
+    dev = torch.device("cuda:0")
+    B, NH, NC, cgs = 1, 4, 24, 8
+    K = host.num_checkpoints(NC, cgs)
+    d = orc.make_inputs(B, NH, NC, seed=60, with_grads=False)
+    t = {k: d[k].to(dev).contiguous() for k in FWD_KEYS}
+    t.update(host.alloc_forward_buffers(B, NH, NC, cgs, dev))
+    a = _args(host.FWD_ORDER, t, cgs, B, NH, NC, K)
+    sticky = torch.zeros(1, dtype=torch.int32, device=dev)
+
+    def eager():
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        rc = lib.ttt_mlp_fwd_launch_static(ctypes.byref(a), ctypes.c_void_p(sticky.data_ptr()), stream)
+        assert rc == 0, lib.ttt_mlp_error_string(rc)
+        torch.cuda.synchronize()
+
+    print("ordinary call ahead of the capture", flush=True)
+    eager()
+    graph = torch.cuda.CUDAGraph()
+    print("capture", flush=True)
+    with torch.cuda.graph(graph):
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        rc = lib.ttt_mlp_fwd_launch_static(ctypes.byref(a), ctypes.c_void_p(sticky.data_ptr()), stream)
+    assert rc == 0, lib.ttt_mlp_error_string(rc)
+    for rep in range(3):
+        print(f"replay {rep}", flush=True)
+        d = orc.make_inputs(B, NH, NC, seed=61 + rep, with_grads=False)
+        for k in FWD_KEYS:
+            t[k].copy_(d[k].to(dev))
+        for k in OUT_KEYS:
+            t[k].fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = {k: t[k].float().cpu() for k in OUT_KEYS}
+        for k in OUT_KEYS:
+            t[k].fill_(float("nan"))
+        eager()
+        for k in OUT_KEYS:
+            assert torch.isfinite(got[k]).all(), (rep, k)
+            assert torch.equal(got[k], t[k].float().cpu()), (rep, k)
+    assert sticky.item() == 0, "a workgroup gave up waiting for the other"
