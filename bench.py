@@ -193,11 +193,21 @@ def run_workload(name, steps, warmup, overwrite=False, no_overlap=False, calibra
     # one kernel per combination of roles: ttt_mlp_bwd_split_kernel<replaying workgroups, grad_L_XK workgroup>
     bwd_kernel = "ttt_mlp_bwd_kernel"
     fwd_kernel = "ttt_mlp_fwd_kernel" if ext.last_forward_mode() == 0 else f"ttt_mlp_fwd_split_kernel<{32 if NC >= 512 else 8}>"
-    if backward and ext.last_backward_mode() == 1:
-        import ctypes
-        lib = ctypes.CDLL(os.path.join(os.path.dirname(os.path.abspath(host.__file__)), "libttt_mlp.so"))
+    import ctypes
+    lib = ctypes.CDLL(os.path.join(os.path.dirname(os.path.abspath(host.__file__)), "libttt_mlp.so"))
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+
+    def cut(which, overlapped):   # launches of a call whose sequences are cut at checkpoints (0: they are not)
+        seg, launches = ctypes.c_int(), ctypes.c_int()
+        lib.ttt_mlp_segment_plan(which, ctypes.c_longlong(B * NH), cus, NC, cgs, 1 if overlapped else 0, ctypes.byref(seg), ctypes.byref(launches))
+        return launches.value if seg.value > 0 else 0
+
+    if cut(0, ext.last_forward_mode() == 1):
+        fwd_kernel = f"ttt_mlp_fwd_kernel x {cut(0, ext.last_forward_mode() == 1)} (sequences cut at checkpoints)"
+    if backward and cut(1, ext.last_backward_mode() == 1):
+        bwd_kernel = f"ttt_mlp_bwd_kernel x {cut(1, ext.last_backward_mode() == 1)} (sequences cut at checkpoints)"
+    elif backward and ext.last_backward_mode() == 1:
         one, rest, per = ctypes.c_longlong(), ctypes.c_longlong(), ctypes.c_int()
-        cus = torch.cuda.get_device_properties(dev).multi_processor_count
         lib.ttt_mlp_launch_plan(1, ctypes.c_longlong(B * NH), cus, ctypes.byref(one), ctypes.byref(rest), ctypes.byref(per))
         bwd_kernel = f"ttt_mlp_bwd_split_kernel<{2 if per.value >= 3 else 1}, {'true' if per.value >= 4 else 'false'}>"
         if one.value:

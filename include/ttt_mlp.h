@@ -233,6 +233,21 @@ const char* ttt_mlp_error_string(int code);
 int ttt_mlp_launch_plan(int which, long long pairs, int compute_units, long long* one_workgroup_pairs,
                         long long* other_pairs, int* workgroups_per_other_pair);
 
+/* With more (batch, head) pairs than CUs the launchers cut every sequence into segments at checkpoint boundaries
+ * where that shortens the call: a forward segment starts from the checkpoint that the segment before it left in
+ * the caller's checkpoint tensors; a backward segment (the sequence's last groups first) takes the running
+ * gradients from grad_L_W1/b1/W2/b2_init, where the one before it left them, and the norm-gradient sums from
+ * x_hat_ln_group (needs checkpoint_group_size >= 2).  The (segment, pair) jobs are launched `compute_units` at a
+ * time, so a last round that is not full costs a fraction of a sequence instead of a whole one (384 pairs on
+ * 256 CUs: 3 launches of half a sequence).  Results do not change by a bit.  This query (no device needed) says
+ * what the launchers do for `pairs` pairs of `NC` mini-batches (which = 0 forward, 1 backward; compute_units = 0:
+ * the current device's, as the launchers count them):
+ * *segment_minibatches = mini-batches per segment (0: sequences are not cut) and *launches = kernel launches of
+ * the call; with_workspace = 0 for ttt_mlp_*_launch, 1 for ttt_mlp_*_launch_overlapped.  No counterpart in the
+ * reference (kernels/ttt/ttt.cu:699-706 launches one grid of B*NH clusters for whole sequences). */
+int ttt_mlp_segment_plan(int which, long long pairs, int compute_units, int NC, int checkpoint_group_size, int with_workspace,
+                         int* segment_minibatches, int* launches);
+
 /* Static facts about the compiled kernels, for harnesses: LDS bytes per
  * workgroup and threads per workgroup of the forward (which = 0) or backward
  * (which = 1) kernel.  Returns 0 on success. */

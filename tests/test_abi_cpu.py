@@ -35,7 +35,7 @@ def test_header_declares_the_expected_entry_points():
     assert declared_functions() == ["ttt_mlp_abi_version", "ttt_mlp_bwd_export_group0", "ttt_mlp_bwd_launch", "ttt_mlp_bwd_launch_overlapped",
                                     "ttt_mlp_bwd_status_offset", "ttt_mlp_bwd_workspace_bytes", "ttt_mlp_error_string",
                                     "ttt_mlp_fwd_launch", "ttt_mlp_fwd_launch_overlapped", "ttt_mlp_fwd_launch_static", "ttt_mlp_fwd_status_offset",
-                                    "ttt_mlp_fwd_workspace_bytes", "ttt_mlp_kernel_info", "ttt_mlp_launch_plan", "ttt_mlp_set_compute_units", "ttt_mlp_set_wait_limit",
+                                    "ttt_mlp_fwd_workspace_bytes", "ttt_mlp_kernel_info", "ttt_mlp_launch_plan", "ttt_mlp_segment_plan", "ttt_mlp_set_compute_units", "ttt_mlp_set_wait_limit",
                                     "ttt_mlp_status_accumulate"]
 
 
@@ -217,3 +217,39 @@ def test_launch_plan_keeps_waiting_workgroups_within_the_device(lib):
 
 def test_export_of_group_zero_validates_like_the_backward(lib):
     assert lib.ttt_mlp_bwd_export_group0(None, None) == 1001
+
+
+def test_segment_plan_cuts_sequences_where_a_last_round_would_idle(lib):
+    """More pairs than CUs: the sequences are cut at checkpoint boundaries and the (segment, pair) jobs launched a
+    device's worth at a time, when that is shorter than whole rounds (or than a last round with several workgroups per
+    pair).  A pair's earlier segment must sit in an earlier launch, the segments are whole checkpoint groups, and the
+    backward needs two mini-batch slots of x_hat_ln_group for its parked sums."""
+    def plan(which, pairs, cus, NC, cgs, ws):
+        a, b = ctypes.c_int(-1), ctypes.c_int(-1)
+        assert lib.ttt_mlp_segment_plan(which, ctypes.c_longlong(pairs), cus, NC, cgs, ws, ctypes.byref(a), ctypes.byref(b)) == 0
+        return a.value, b.value
+    for which in (0, 1):
+        for ws in (0, 1):
+            assert plan(which, 384, 256, 512, 32, ws) == (256, 3)      # the fill-the-chip configuration: 1.5 rounds
+            assert plan(which, 48, 256, 4096, 64, ws)[0] == 0         # fewer pairs than CUs: nothing to gain
+            assert plan(which, 256, 256, 512, 32, ws)[0] == 0
+            assert plan(which, 512, 256, 512, 32, ws)[0] == 0         # full rounds
+            assert plan(which, 384, 256, 512, 512, ws)[0] == 0        # one checkpoint group: nowhere to cut
+    assert plan(0, 257, 256, 512, 32, 1) == (64, 9)                   # 8 segments: 9 launches of an eighth
+    assert plan(1, 384, 256, 512, 1, 0)[0] == 0                       # backward, groups of one mini-batch
+    assert plan(0, 384, 256, 512, 1, 0)[0] > 0
+    assert plan(0, 384, 256, 512, 32, 1) == plan(0, 384, 256, 512, 32, 0)
+    assert lib.ttt_mlp_segment_plan(2, ctypes.c_longlong(8), 8, 8, 8, 0, ctypes.byref(ctypes.c_int()), ctypes.byref(ctypes.c_int())) == 1001
+    assert lib.ttt_mlp_segment_plan(0, ctypes.c_longlong(8), 8, 8, 8, 0, None, None) == 1001
+    for which in (0, 1):
+        for cus in (2, 8, 104, 256):
+            for pairs in (cus + 1, cus + cus // 2, 2 * cus - 1, 2 * cus + 1, 3 * cus + 5):
+                for NC, cgs in ((512, 32), (100, 8), (90, 3), (7, 2), (4096, 64)):
+                    seg, launches = plan(which, pairs, cus, NC, cgs, 1)
+                    if seg == 0:
+                        continue
+                    assert seg % cgs == 0 and seg < NC
+                    segments = -(-NC // seg)
+                    assert launches == -(-segments * pairs // cus)
+                    # job (segment s, pair p) has index s * pairs + p: the launch of (s, p) comes after that of (s - 1, p)
+                    assert all((s * pairs + p) // cus > ((s - 1) * pairs + p) // cus for s in range(1, segments) for p in (0, pairs - 1))

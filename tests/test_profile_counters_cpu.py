@@ -112,3 +112,19 @@ def test_launch_summary_adds_up_the_kernels_of_one_launch():
     assert abs(b["hbm_gbs"] - 1.35e11 / 36e6) < 1e-6
     f = L["fwd"]
     assert "hbm_bytes" not in f and "valu_insts_per_unit" not in f and abs(f["launch_ms"] - 10.0) < 1e-9
+
+
+def test_launch_summary_counts_every_dispatch_of_a_cut_launch():
+    """c5 with the sequences cut at checkpoints: a launch is three dispatches of the one-workgroup kernel, and the
+    per-dispatch averages of the profiler are multiplied out."""
+    kernels = {
+        "ttt_mlp_bwd_kernel": dict(avg_ns=12e6, dispatches_per_launch=3, hbm_bytes=4.5e10,
+                                   counters=dict(SQ_INSTS_VALU=3e9, SQ_INSTS_MFMA=1e8, SQ_INSTS_LDS=4e8)),
+        "ttt_mlp_fwd_kernel": dict(avg_ns=3e6, dispatches_per_launch=3),
+    }
+    L = pc.launch_summary("c5", kernels)
+    units = 8 * 48 * 512
+    assert abs(L["bwd"]["launch_ms"] - 36.0) < 1e-9 and abs(L["bwd"]["hbm_bytes"] - 1.35e11) < 1
+    assert abs(L["bwd"]["valu_insts_per_unit"] - 9e9 / units) < 1e-6
+    assert abs(L["fwd"]["launch_ms"] - 9.0) < 1e-9
+    assert pc.TRACE_LAUNCHES == 3

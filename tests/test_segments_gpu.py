@@ -1,0 +1,68 @@
+"""More (batch, head) pairs than CUs: the forward cuts every sequence into segments at checkpoint boundaries and
+launches the (segment, pair) jobs a device's worth at a time (a segment starts from the checkpoint the one before it
+left).  Forced here on a few pairs by a small compute-unit budget; the results must not change by a bit - Out, all
+checkpoints, and the backward that starts from those checkpoints."""
+import ctypes
+import os
+
+import pytest
+import torch
+
+from oracle import ttt_mlp_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "ttt-tk_amd", "libttt_mlp.so")
+FWD_KEYS = ("XQ", "XK", "XV", "last_eta", "ttt_norm_weight", "ttt_norm_bias", "W1", "b1", "W2", "b2")
+UP_KEYS = ("grad_L_W1_last", "grad_L_b1_last", "grad_L_W2_last", "grad_L_b2_last", "grad_L_XQW_mini_batch")
+CK_KEYS = ("W1_checkpoints", "b1_checkpoints", "W2_checkpoints", "b2_checkpoints")
+
+
+def _plan(lib, which, pairs, cus, NC, cgs, with_workspace):
+    seg, launches = ctypes.c_int(-1), ctypes.c_int(-1)
+    rc = lib.ttt_mlp_segment_plan(which, ctypes.c_longlong(pairs), cus, NC, cgs, with_workspace, ctypes.byref(seg), ctypes.byref(launches))
+    assert rc == 0
+    return seg.value, launches.value
+
+
+@pytest.mark.parametrize("NC,cgs", [(96, 8), (100, 8), (90, 3)])
+def test_cut_sequences_give_the_same_forward(NC, cgs):
+    import test_time_training as ext
+    import ttt_mlp_host as host
+    lib = ctypes.CDLL(LIB)
+    dev = torch.device("cuda:0")
+    B, NH = 1, 3
+    print(f"case B={B} NH={NH} NC={NC} cgs={cgs}", flush=True)
+    d = orc.make_inputs(B, NH, NC, seed=71)
+    t = {k: d[k].to(dev).contiguous() for k in FWD_KEYS + UP_KEYS}
+    t.update(host.alloc_forward_buffers(B, NH, NC, cgs, dev))
+    t.update(host.alloc_backward_buffers(B, NH, NC, cgs, dev))
+
+    def run():
+        for k in ("Out",) + CK_KEYS:
+            t[k].fill_(float("nan"))
+        host.zero_accumulating_grads(t)
+        host.forward(t, cgs)
+        host.backward(t, cgs)
+        torch.cuda.synchronize()
+        return {k: t[k].clone() for k in ("Out",) + CK_KEYS + host.GRAD_NAMES}
+
+    ref = run()                                   # 3 pairs on the whole device: whole sequences
+    for k, r in ref.items():
+        assert torch.isfinite(r.float()).all(), k
+    try:
+        ext.set_compute_units(2)                  # 3 pairs on 2 CUs
+        for overlap in (True, False):             # with the operator's workspace, and the plain launch
+            for which in (0, 1):
+                seg, launches = _plan(lib, which, B * NH, 2, NC, cgs, 1 if overlap else 0)
+                print(f"  overlap={overlap} {('forward', 'backward')[which]}: segments of {seg} mini-batches, {launches} launches", flush=True)
+                if not overlap:                   # against whole rounds a cut always pays here
+                    assert seg > 0 and seg % cgs == 0 and launches >= 3, "the shape was meant to be cut"
+            ext.set_overlap(overlap)
+            got = run()
+            for k, r in ref.items():
+                assert torch.equal(got[k], r), (overlap, k)
+    finally:
+        ext.set_overlap(True)
+        ext.set_compute_units(0)

@@ -93,6 +93,14 @@ bool workspace_is_affordable(size_t bytes) {
 // operators allocate nothing and ask the device nothing: the launch uses it if it is large enough and on the right
 // device, and falls back to one workgroup per (batch, head) otherwise.  Without one the workspace comes from torch's
 // caching allocator (which orders its reuse after the launch on the same stream) if the device has room to spare.
+// Whether the launcher would cut the sequences of this shape at checkpoints even with a workspace at hand (it then runs
+// one workgroup per pair and the workspace would go unused).
+bool sequences_cut(int which, int64_t pairs, int64_t NC, int64_t cgs) {
+  int seg = 0, launches = 0;
+  if (ttt_mlp_segment_plan(which, (long long)pairs, 0, (int)NC, (int)cgs, 1, &seg, &launches) != 0) return false;
+  return seg > 0;
+}
+
 struct Workspace {
   void* ptr = nullptr;
   torch::Tensor held;   // keeps an allocated workspace alive until the launch has been enqueued
@@ -154,7 +162,9 @@ torch::Tensor ttt_forward(const torch::Tensor XQ, const torch::Tensor XK, const 
   hipStream_t stream = c10::hip::getCurrentHIPStream(XQ.device().index()).stream();
   // With few (batch, head) pairs most CUs would idle: then a second workgroup per pair computes Out behind
   // the state recurrence.  Its workspace: the caller's (set_workspace) or torch's caching allocator's.
-  const size_t ws_bytes = (g_overlap && NC >= 2) ? ttt_mlp_fwd_workspace_bytes((int32_t)B, (int32_t)NH) : 0;
+  // (more pairs than CUs and sequences that the launcher cuts at checkpoints: no second workgroup, no workspace)
+  const size_t ws_bytes = (g_overlap && NC >= 2 && !sequences_cut(0, B * NH, NC, checkpoint_group_size))
+                              ? ttt_mlp_fwd_workspace_bytes((int32_t)B, (int32_t)NH) : 0;
   const Workspace ws = take_workspace(ws_bytes, XQ.device());
   if (ws.ptr != nullptr) {
     g_last_forward_mode = 1;
@@ -267,7 +277,8 @@ torch::Tensor ttt_backward(
   // With few (batch, head) pairs most CUs would idle: then a second workgroup per pair recomputes the
   // checkpoint groups ahead of the reverse walk.  Its workspace (further sets of the per-group tensors): the
   // caller's (set_workspace) or torch's caching allocator's.
-  const size_t ws_bytes = (g_overlap && K >= 2) ? ttt_mlp_bwd_workspace_bytes((int32_t)B, (int32_t)NH, checkpoint_group_size) : 0;
+  const size_t ws_bytes = (g_overlap && K >= 2 && !sequences_cut(1, B * NH, NC, checkpoint_group_size))
+                              ? ttt_mlp_bwd_workspace_bytes((int32_t)B, (int32_t)NH, checkpoint_group_size) : 0;
   const Workspace ws = take_workspace(ws_bytes, XQ.device());
   if (ws.ptr != nullptr) {
     g_last_backward_mode = 1;

@@ -395,7 +395,9 @@ constexpr int FIN_CHUNK = 8;   // mini-batches per hand-over to the grad_L_XK wo
 // fourth workgroup the walk hands over the operands of its two products (gW1, G1, dZ1 as register images)
 // and g_y, and that workgroup (bwd_finish_dxk) forms the products, their pair sum and the final sum.
 template <int ROLE, bool IMG, bool FIN>
-TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, const int turn) {
+// k_hi, k_lo: the checkpoint groups k_hi, k_hi - 1, .. k_lo of the sequence (ROLE 0: a segment; the other roles take
+// the whole sequence, K - 1 .. 0).
+TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, const int turn, const int k_hi, const int k_lo) {
   static_assert(!(ROLE == 0 && (IMG || FIN)), "one workgroup per (batch, head) does everything itself");
   bf16* s_xq = reinterpret_cast<bf16*>(smem + SB_XQ);
   bf16* s_xk = reinterpret_cast<bf16*>(smem + SB_XK);
@@ -431,13 +433,16 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
   float* s_b1w = s_b1 + hid0;
   float* s_gb1w = s_gb1 + hid0;
   const int cgs = p.cgs;
+  // a segment that is not the first to run continues where the one before it stopped; one that is not the last leaves
+  // what the next one needs instead of the norm gradients
+  const bool seg_first = k_hi == p.K - 1, seg_last = k_lo == 0;
 
   if (tid < FD) {
     s_gam[tid] = p.ttt_norm_weight[head * FD + tid];
     s_bet[tid] = p.ttt_norm_bias[head * FD + tid];
-    s_gb2[tid] = p.grad_L_b2_last[(size_t)bh * FD + tid];
+    s_gb2[tid] = (seg_first ? p.grad_L_b2_last : p.grad_L_b2_init)[(size_t)bh * FD + tid];
   }
-  if (tid < HID) s_gb1[tid] = p.grad_L_b1_last[(size_t)bh * HID + tid];
+  if (tid < HID) s_gb1[tid] = (seg_first ? p.grad_L_b1_last : p.grad_L_b1_init)[(size_t)bh * HID + tid];
   // Norm-weight / norm-bias gradients accumulate per wave in LDS (summed over the wave's 8 tokens
   // with cross-lane adds in a fixed order); summed over the waves at the end.  The replay and the
   // reverse walk each contribute, and their sums are kept apart (so that the result does not depend on
@@ -525,8 +530,8 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
   AccT<2, 1> gW1s;
   AccT<1, 2> gW2s;
   if constexpr (ROLE != 1) {
-    acc_load_rows(gW1s, gbuf(p.grad_L_W1_last + (size_t)bh * FD * HID), 0, HID, 0, hid0, c, h);
-    acc_load_rows(gW2s, gbuf(p.grad_L_W2_last + (size_t)bh * HID * FD), 0, FD, hid0, 0, c, h);
+    acc_load_rows(gW1s, gbuf((seg_first ? p.grad_L_W1_last : p.grad_L_W1_init) + (size_t)bh * FD * HID), 0, HID, 0, hid0, c, h);
+    acc_load_rows(gW2s, gbuf((seg_first ? p.grad_L_W2_last : p.grad_L_W2_init) + (size_t)bh * HID * FD), 0, FD, hid0, 0, c, h);
   }
   int* const w_sync = p.sync + (size_t)bh * BWD_SYNC_STRIDE;   // + 0, + 8: groups replayed by workgroup 0 / 1
   int* const w_walked = w_sync + 16;
@@ -542,13 +547,17 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
   const gptr_t gPark = ROLE == 0 ? gbuf(p.x_hat_ln_group + (size_t)bh * cgs * (CS * FD))
                                  : gbuf(p.norm_park + (size_t)bh * (BW_NWAVE * 2 * FD));
   constexpr unsigned PARK_BYTES = BW_NWAVE * 2 * FD * 4;
-  if (ROLE == 0 || (ROLE == 1 && n_replay == 1)) {   // parked sums start at zero
+  if (ROLE == 0 ? seg_first : (ROLE == 1 && n_replay == 1)) {   // parked sums start at zero
     g_stf(gPark, np_off, 0, 0.f);
     g_stf(gPark, np_off, FD * 4, 0.f);
     if constexpr (ROLE == 0) {
       g_stf(gPark, np_off, PARK_BYTES, 0.f);
       g_stf(gPark, np_off, PARK_BYTES + FD * 4, 0.f);
     }
+  }
+  if (ROLE == 0 && !seg_first) {   // the walk's sum as the segment before this one left it (a third slot of the park)
+    s_dgw[lane] = g_ldf(gPark, np_off, 2 * PARK_BYTES);
+    s_dbw[lane] = g_ldf(gPark, np_off, 2 * PARK_BYTES + FD * 4);
   }
   // Exchanges the wave's LDS accumulators with a parked sum (every lane owns two words of both).
   auto norm_swap = [&](unsigned slot) {
@@ -563,7 +572,7 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
   };
 
   TTT_STAGES_BEGIN();
-  for (int k = p.K - 1; k >= 0; k--) {
+  for (int k = k_hi; k >= k_lo; k--) {
     const int n_mb = min(cgs, p.NC - k * cgs);
     const int done = p.K - 1 - k;                    // number of this group, counted from the end of the sequence
     if (ROLE == 1 && done % n_replay != turn) continue;
@@ -1481,6 +1490,11 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
   // last counts this workgroup has acquired (a second replaying workgroup has nothing to hand over if there is
   // one group only).
   if constexpr (FIN) return;   // with a grad_L_XK workgroup the walk holds no share of these sums: they are written there
+  if (ROLE == 0 && !seg_last) {   // the next segment goes on with the walk's sum (the replay's two are parked already)
+    g_stf(gPark, np_off, 2 * PARK_BYTES, s_dgw[lane]);
+    g_stf(gPark, np_off, 2 * PARK_BYTES + FD * 4, s_dbw[lane]);
+    return;
+  }
   if (tid < 2 * FD) {
     const int which = tid / FD, f = tid % FD;
     const float* rp = ROLE == 0 ? reinterpret_cast<const float*>(p.x_hat_ln_group + (size_t)bh * cgs * (CS * FD))
@@ -1527,7 +1541,14 @@ TTT_DEV void bwd_body(const BwdParams& p, unsigned char* smem, const int bh, con
 
 __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  bwd_body<0, false, false>(p, smem, p.bh0 + blockIdx.x, 0);
+  int bh = p.bh0 + blockIdx.x, k_hi = p.K - 1, k_lo = 0;
+  if (p.seg_groups > 0) {
+    const int pairs = p.B * p.NH, job = p.job0 + blockIdx.x, seg = job / pairs;
+    bh = job - seg * pairs;
+    k_hi = p.K - 1 - seg * p.seg_groups;
+    k_lo = k_hi - p.seg_groups + 1 > 0 ? k_hi - p.seg_groups + 1 : 0;
+  }
+  bwd_body<0, false, false>(p, smem, bh, 0, k_hi, k_lo);
 }
 
 // grad_L_XK on a workgroup of its own: for every mini-batch of every group, as soon as the walk is done with the
@@ -1777,8 +1798,8 @@ __global__ __launch_bounds__(BW_THREADS) void ttt_mlp_bwd_split_kernel(const Bwd
   }
   bh += p.bh0;
   constexpr bool IMG = NREPLAY == 2;   // two replaying workgroups also evaluate the GELU family for the walk
-  if (role < NREPLAY) bwd_body<1, IMG, FINISH>(p, smem, bh, role);
-  else if (role == NREPLAY) bwd_body<2, IMG, FINISH>(p, smem, bh, 0);
+  if (role < NREPLAY) bwd_body<1, IMG, FINISH>(p, smem, bh, role, p.K - 1, 0);
+  else if (role == NREPLAY) bwd_body<2, IMG, FINISH>(p, smem, bh, 0, p.K - 1, 0);
   else if constexpr (FINISH) {
     if (role == NREPLAY + 1) bwd_finish_dxk(p, smem, bh);
     else bwd_prefetch(p, smem, bh);

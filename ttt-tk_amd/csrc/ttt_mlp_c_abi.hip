@@ -177,6 +177,93 @@ LaunchPlan plan_launches(long long BH, bool three_way) {
   return plan_for(BH, cus, three_way);
 }
 
+// More (batch, head) pairs than CUs, one workgroup each: the hardware runs them in rounds, and a last round that is
+// not full leaves CUs idle for a whole sequence.  The forward can cut every sequence into segments at checkpoint
+// boundaries instead - a segment starts from the checkpoint before its first mini-batch, which the segment before it
+// left in the caller's checkpoint tensors - and launch the (segment, pair) jobs segment-major, one launch per `cus`
+// jobs: a pair's earlier segment is always in an earlier launch (pairs >= cus), and the rounds are a fraction of a
+// sequence long, so 384 pairs on 256 CUs take 3 launches of half a sequence, 1.5 sequences instead of 2 (or 1.76 with
+// the last 128 pairs on two workgroups each).  Same arithmetic on the same state: results do not change.
+struct SegmentPlan {
+  int seg_len = 0;      // mini-batches per segment, a multiple of cgs; 0 = sequences are not cut
+  int groups = 0;       // checkpoint groups per segment
+  int launches = 1;
+  long long jobs = 0;
+};
+// `alt_x1000`: what the alternative costs, in thousandths of a mini-batch of one workgroup.
+SegmentPlan plan_segments(long long pairs, int cus, int NC, int cgs, long long alt_x1000) {
+  SegmentPlan best;
+#ifndef TTT_STAGE_CLOCKS   // the stage clocks are kept per pair and sequence
+  if (pairs <= cus || cus <= 0 || NC <= 0 || cgs <= 0) return best;
+  const int K = (NC + cgs - 1) / cgs;
+#ifndef TTT_CUT_PERCENT
+#define TTT_CUT_PERCENT 99   // a cut must gain 1 % by this estimate
+#endif
+  long long best_t = alt_x1000 * TTT_CUT_PERCENT / 100;
+  for (int S = 2; S <= 8 && S <= K; S++) {
+    const int groups = (K + S - 1) / S, segs = (K + groups - 1) / groups;
+    const long long len = (long long)groups * cgs, jobs = segs * pairs, launches = (jobs + cus - 1) / cus;
+    const long long t = launches * (len * 1000 + 2000);   // + 2 mini-batches' worth per launch: gaps, state in and out
+    if (t < best_t) {
+      best_t = t;
+      best.seg_len = static_cast<int>(len);
+      best.groups = groups;
+      best.launches = static_cast<int>(launches);
+      best.jobs = jobs;
+    }
+  }
+#endif
+  return best;
+}
+// Thousandths of a one-workgroup mini-batch that the pairs take uncut: full rounds, and the rest either one more
+// round or, with several workgroups per pair, a shorter one - measured with every CU busy: the forward's recurrence
+// workgroup runs at 0.755 of one workgroup's time per mini-batch; the backward's walk with one replaying workgroup
+// at 0.56, and about 0.4 / 0.3 with more workgroups per pair.
+long long uncut_x1000(const LaunchPlan& pl, long long pairs, int cus, int NC, bool with_workspace, bool backward) {
+  if (cus <= 0) return (long long)NC * 1000;
+  if (with_workspace && pl.rest_split) {
+    const int rest = !backward ? 755 : pl.per_pair == 2 ? 560 : pl.per_pair == 3 ? 400 : 300;
+    return (pl.n_single / cus * 1000 + rest) * NC;
+  }
+  return (pairs + cus - 1) / cus * 1000 * NC;
+}
+int device_cus() {
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+    return 0;
+  return g_cu_budget > 0 && g_cu_budget < cus ? g_cu_budget : cus;
+}
+// The forward's launches with the sequences cut (plan.seg_len > 0).
+int launch_fwd_segments(ttt::FwdParams p, const SegmentPlan& plan, int cus, hipStream_t stream) {
+  p.sync = nullptr;
+  p.bh0 = 0;
+  p.seg_len = plan.seg_len;
+  for (long long j0 = 0; j0 < plan.jobs; j0 += cus) {
+    p.job0 = static_cast<int>(j0);
+    p.nbh = static_cast<int>(plan.jobs - j0 < cus ? plan.jobs - j0 : cus);
+    if (hipError_t e = ttt_mlp_fwd_enqueue(p, stream)) return static_cast<int>(e);
+  }
+  return TTT_MLP_OK;
+}
+
+// The backward's launches with the sequences cut: segment 0 = the last groups of every sequence.  The third parked
+// norm-gradient sum needs a second mini-batch slot in x_hat_ln_group, hence cgs >= 2 (plan_bwd_segments).
+int launch_bwd_segments(ttt::BwdParams p, const SegmentPlan& plan, int cus, hipStream_t stream) {
+  p.sync = nullptr;
+  p.bh0 = 0;
+  p.seg_groups = plan.groups;
+  for (long long j0 = 0; j0 < plan.jobs; j0 += cus) {
+    p.job0 = static_cast<int>(j0);
+    p.nbh = static_cast<int>(plan.jobs - j0 < cus ? plan.jobs - j0 : cus);
+    if (hipError_t e = ttt_mlp_bwd_enqueue(p, stream)) return static_cast<int>(e);
+  }
+  return TTT_MLP_OK;
+}
+SegmentPlan plan_bwd_segments(const LaunchPlan& pl, long long pairs, int cus, int NC, int cgs, bool with_workspace) {
+  if (cgs < 2) return SegmentPlan{};
+  return plan_segments(pairs, cus, NC, cgs, uncut_x1000(pl, pairs, cus, NC, with_workspace, true));
+}
+
 // Workspace of the backward with 2 or 3 workgroups per pair, for n (batch, head) pairs: the synchronisation
 // words, the replay's shares of the norm gradients (two sums per pair + one parking slot), then 1 or 3
 // alternate sets of the ten per-group tensors that carry a replayed group to the reverse walk; each part
@@ -237,6 +324,12 @@ int check_workspace(const void* workspace) {
 extern "C" int ttt_mlp_bwd_launch(const ttt_mlp_bwd_args* a, void* stream) {
   ttt::BwdParams p;
   if (int rc = make_bwd_params(a, p)) return rc;
+  {
+    const long long pairs = (long long)p.B * p.NH;
+    const int cus = device_cus();
+    const SegmentPlan seg = plan_bwd_segments(LaunchPlan{}, pairs, cus, p.NC, p.cgs, false);
+    if (seg.seg_len > 0) return launch_bwd_segments(p, seg, cus, static_cast<hipStream_t>(stream));
+  }
   p.bh0 = 0;
   p.nbh = p.B * p.NH;
   return static_cast<int>(ttt_mlp_bwd_enqueue(p, static_cast<hipStream_t>(stream)));
@@ -274,13 +367,25 @@ extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* wo
   const bool finish = pl.per_pair == 4;
   const BwdWorkspace w(pl.n_rest, p.cgs, alt_sets, finish);
   if (workspace_bytes < w.total) return TTT_MLP_ERR_WORKSPACE;
+  char* base = static_cast<char*>(workspace);
+  {
+    // cut sequences where they beat a last round on several workgroups per pair (see the forward)
+    const long long pairs = (long long)p.B * p.NH;
+    const int cus = device_cus();
+    const SegmentPlan seg = plan_bwd_segments(pl, pairs, cus, p.NC, p.cgs, true);
+    if (seg.seg_len > 0) {
+      if (hipError_t e = ttt_mlp_fwd_clear_words(reinterpret_cast<int*>(base + w.off[0]), static_cast<int>(ttt::bwd_sync_ints(pl.n_rest)),
+                                                 static_cast<hipStream_t>(stream)))
+        return static_cast<int>(e);
+      return launch_bwd_segments(p, seg, cus, static_cast<hipStream_t>(stream));
+    }
+  }
   if (pl.n_single > 0) {
     p.bh0 = 0;
     p.nbh = static_cast<int>(pl.n_single);
     if (hipError_t e = ttt_mlp_bwd_enqueue(p, static_cast<hipStream_t>(stream))) return static_cast<int>(e);
   }
   // The kernels index the workspace by the global pair number: every pointer is moved back by bh0 entries.
-  char* base = static_cast<char*>(workspace);
   const size_t b0 = (size_t)pl.n_single;
   const size_t tile = (size_t)p.cgs * TTT_MLP_CS * TTT_MLP_F, img = (size_t)p.cgs * TTT_MLP_CS * TTT_MLP_HID, vec = (size_t)p.cgs * TTT_MLP_CS;
   const size_t norm = 8 * 2 * TTT_MLP_F;
@@ -320,6 +425,10 @@ extern "C" int ttt_mlp_bwd_launch_overlapped(const ttt_mlp_bwd_args* a, void* wo
 extern "C" int ttt_mlp_fwd_launch(const ttt_mlp_fwd_args* a, void* stream) {
   ttt::FwdParams p;
   if (int rc = make_fwd_params(a, p)) return rc;
+  const long long pairs = (long long)p.B * p.NH;
+  const int cus = device_cus();
+  const SegmentPlan seg = plan_segments(pairs, cus, p.NC, p.cgs, uncut_x1000(LaunchPlan{}, pairs, cus, p.NC, false, false));
+  if (seg.seg_len > 0) return launch_fwd_segments(p, seg, cus, static_cast<hipStream_t>(stream));
   p.bh0 = 0;
   p.nbh = p.B * p.NH;
   return static_cast<int>(ttt_mlp_fwd_enqueue(p, static_cast<hipStream_t>(stream)));
@@ -345,12 +454,25 @@ extern "C" int ttt_mlp_fwd_launch_overlapped(const ttt_mlp_fwd_args* a, void* wo
   if (!pl.rest_split) return TTT_MLP_ERR_NO_ROOM;
   const FwdWorkspace w(pl.n_rest);
   if (workspace_bytes < w.total) return TTT_MLP_ERR_WORKSPACE;
+  char* base = static_cast<char*>(workspace);
+  {
+    // cut sequences beat a last round on two workgroups per pair where there are full rounds before it: the
+    // workspace then only has its words cleared (callers read the status word behind them)
+    const long long pairs = (long long)p.B * p.NH;
+    const int cus = device_cus();
+    const SegmentPlan seg = plan_segments(pairs, cus, p.NC, p.cgs, uncut_x1000(pl, pairs, cus, p.NC, true, false));
+    if (seg.seg_len > 0) {
+      if (hipError_t e = ttt_mlp_fwd_clear_words(reinterpret_cast<int*>(base + w.off[0]), static_cast<int>(ttt::bwd_sync_ints(pl.n_rest)),
+                                                 static_cast<hipStream_t>(stream)))
+        return static_cast<int>(e);
+      return launch_fwd_segments(p, seg, cus, static_cast<hipStream_t>(stream));
+    }
+  }
   if (pl.n_single > 0) {
     p.bh0 = 0;
     p.nbh = static_cast<int>(pl.n_single);
     if (hipError_t e = ttt_mlp_fwd_enqueue(p, static_cast<hipStream_t>(stream))) return static_cast<int>(e);
   }
-  char* base = static_cast<char*>(workspace);
   const size_t b0 = (size_t)pl.n_single;
   p.bh0 = static_cast<int>(pl.n_single);
   p.nbh = static_cast<int>(pl.n_rest);
@@ -444,6 +566,21 @@ extern "C" int ttt_mlp_launch_plan(int which, long long pairs, int compute_units
   *one_workgroup_pairs = pl.n_single;
   *other_pairs = pl.n_rest;
   *workgroups_per_other_pair = pl.n_rest > 0 ? pl.per_pair + (pl.prefetch ? 1 : 0) : 0;
+  return TTT_MLP_OK;
+}
+
+extern "C" int ttt_mlp_segment_plan(int which, long long pairs, int compute_units, int NC, int checkpoint_group_size, int with_workspace,
+                                    int* segment_minibatches, int* launches) {
+  if (compute_units == 0) compute_units = device_cus();   // the current device's, or the budget set for it
+  if (segment_minibatches == nullptr || launches == nullptr || pairs <= 0 || compute_units <= 0 || NC <= 0 ||
+      checkpoint_group_size <= 0 || (which != 0 && which != 1))
+    return TTT_MLP_ERR_BAD_ARG;
+  const LaunchPlan pl = plan_for(pairs, compute_units, which == 1);
+  const SegmentPlan seg = which == 1 ? plan_bwd_segments(pl, pairs, compute_units, NC, checkpoint_group_size, with_workspace != 0)
+                                     : plan_segments(pairs, compute_units, NC, checkpoint_group_size,
+                                                     uncut_x1000(pl, pairs, compute_units, NC, with_workspace != 0, false));
+  *segment_minibatches = seg.seg_len;
+  *launches = seg.seg_len > 0 ? seg.launches : (with_workspace != 0 && pl.rest_split && pl.n_single > 0 ? 2 : 1);
   return TTT_MLP_OK;
 }
 

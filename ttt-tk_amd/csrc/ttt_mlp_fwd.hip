@@ -212,7 +212,9 @@ TTT_DEV void output_layernorm(const float* s_P, const float* s_b2, const float* 
 // the new state is left in HBM as ready-made bf16 operands for the workgroup that runs fwd_output_branch.
 // RING: mini-batches per hand-over (ROLE 1).
 template <int ROLE, int RING>
-TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
+// mb0, mb1: the mini-batches [mb0, mb1) of the sequence (ROLE 0: a segment; mb0 is a multiple of the checkpoint group
+// size, and so is mb1 unless it is the sequence's end).
+TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh, const int mb0, const int mb1) {
   bf16* s_g2 = reinterpret_cast<bf16*>(smem + SM_G2);
   bf16* s_g2l = reinterpret_cast<bf16*>(smem + SM_G2L);
   float* s_P = reinterpret_cast<float*>(smem + SM_P);
@@ -239,12 +241,17 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
   const int tok = 8 * v + (lane >> 3), f0 = 8 * (lane & 7);                     \
   (void)h; (void)c; (void)tid; (void)tok; (void)f0
 
-  // ---- state -> registers
+  // ---- state -> registers: the caller's initial state, or (a later segment) the checkpoint before mini-batch mb0
   AccT<2, 1> W1s;
   AccT<1, 2> W2s;
   float b1L;      // b1 of hidden column hid0 + c; b2 lives in LDS (fp32) and is updated there by wave 0
   {
-    const gptr_t W1 = gbuf(p.W1 + (size_t)bh * FD * HID), W2 = gbuf(p.W2 + (size_t)bh * HID * FD);
+    const size_t from = mb0 > 0 ? (size_t)bh * p.K + mb0 / p.cgs : (size_t)bh;
+    const float* const W1src = (mb0 > 0 ? p.W1_ck : p.W1) + from * FD * HID;
+    const float* const W2src = (mb0 > 0 ? p.W2_ck : p.W2) + from * HID * FD;
+    const float* const b1src = (mb0 > 0 ? p.b1_ck : p.b1) + from * HID;
+    const float* const b2src = (mb0 > 0 ? p.b2_ck : p.b2) + from * FD;
+    const gptr_t W1 = gbuf(W1src), W2 = gbuf(W2src);
 #pragma unroll
     for (int b = 0; b < 2; b++)
 #pragma unroll
@@ -253,10 +260,10 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
         W1s.b[b][0][i] = g_ldf(W1, (4 * h * HID + c) * 4, ((32 * b + row) * HID + hid0) * 4);
         W2s.b[0][b][i] = g_ldf(W2, (4 * h * FD + c) * 4, ((hid0 + row) * FD + 32 * b) * 4);
       }
-    b1L = p.b1[(size_t)bh * HID + hid0 + c];
-    if (tid < HID) s_b1[tid] = p.b1[(size_t)bh * HID + tid];
+    b1L = b1src[hid0 + c];
+    if (tid < HID) s_b1[tid] = b1src[tid];
     if (tid < FD) {
-      s_b2[tid] = p.b2[(size_t)bh * FD + tid];
+      s_b2[tid] = b2src[tid];
       s_gam[tid] = p.ttt_norm_weight[head * FD + tid];
       s_bet[tid] = p.ttt_norm_bias[head * FD + tid];
     }
@@ -269,8 +276,8 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
   const gptr_t gW1ck = gbuf(p.W1_ck + uni64((size_t)bh * p.K * FD * HID)), gW2ck = gbuf(p.W2_ck + uni64((size_t)bh * p.K * HID * FD));
   {
     Staged st;
-    stage_load(st, gXQ, gXK, gXV, gEta, 0, tid);
-    stage_store(st, smem, 0, tid);
+    stage_load(st, gXQ, gXK, gXV, gEta, mb0, tid);
+    stage_store(st, smem, mb0 & 1, tid);
   }
   __syncthreads();
 
@@ -279,8 +286,25 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
   int* const w_status = p.status;
   int* const s_flag = reinterpret_cast<int*>(smem + SM_FLAG);
 
+  // the state as checkpoint number `ck_slot` of this (batch, head)
+  auto store_checkpoint = [&](int ck_slot) {
+    LANE_VARS;
+    const size_t slot = (size_t)bh * p.K + ck_slot;
+    const unsigned ck = static_cast<unsigned>(ck_slot) * (FD * HID * 4u);   // byte offset of the slot in gW1ck / gW2ck
+#pragma unroll
+    for (int b = 0; b < 2; b++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        const int row = 8 * (i >> 2) + (i & 3);   // + 4h in the lane offset
+        g_stf(gW1ck, (4 * h * HID + c) * 4, ck + ((32 * b + row) * HID + hid0) * 4, W1s.b[b][0][i]);
+        g_stf(gW2ck, (4 * h * FD + c) * 4, ck + ((hid0 + row) * FD + 32 * b) * 4, W2s.b[0][b][i]);
+      }
+    if (h == 0) p.b1_ck[slot * HID + hid0 + c] = b1L;
+    if (tid < FD) p.b2_ck[slot * FD + tid] = s_b2[tid];
+  };
+
   TTT_STAGES_BEGIN();
-  for (int mb = 0; mb < p.NC; mb++) {
+  for (int mb = mb0; mb < mb1; mb++) {
     LANE_VARS;
     const bf16* s_xq = reinterpret_cast<const bf16*>(smem + SM_XQ + (mb & 1) * SM_TILE);
     // ROLE 1 has no use for XQ (nor for b1 in LDS): their space holds a second XK / XV / eta buffer, so that
@@ -304,21 +328,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
       if (mb > 0) __syncthreads();
     }
     // ---- checkpoint: the state before this mini-batch
-    if (mb % p.cgs == 0) {
-      LANE_VARS;
-      const size_t slot = (size_t)bh * p.K + mb / p.cgs;
-      const unsigned ck = static_cast<unsigned>(mb / p.cgs) * (FD * HID * 4u);   // byte offset of the slot in gW1ck / gW2ck
-#pragma unroll
-      for (int b = 0; b < 2; b++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-          const int row = 8 * (i >> 2) + (i & 3);   // + 4h in the lane offset
-          g_stf(gW1ck, (4 * h * HID + c) * 4, ck + ((32 * b + row) * HID + hid0) * 4, W1s.b[b][0][i]);
-          g_stf(gW2ck, (4 * h * FD + c) * 4, ck + ((hid0 + row) * FD + 32 * b) * 4, W2s.b[0][b][i]);
-        }
-      if (h == 0) p.b1_ck[slot * HID + hid0 + c] = b1L;
-      if (tid < FD) p.b2_ck[slot * FD + tid] = s_b2[tid];
-    }
+    if (mb % p.cgs == 0) store_checkpoint(mb / p.cgs);
 
     TTT_STAGE(FS_TOP);
     // ---- Z1 = XK W1 + b1 (rows tok, lane = hid);  X2 = gelu(Z1), D1 = gelu'(Z1)
@@ -386,7 +396,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
         // The next mini-batch's XK / XV / eta leave HBM for the other LDS buffers now (last read a mini-batch ago,
         // two barriers back) without passing through registers: wave v fetches rows 8v .. 8v+7 of both tiles,
         // one pair of rows (256 contiguous bytes) per load, wave 0 also the 128 bytes of eta.
-        if (mb + 1 < p.NC) {
+        if (mb + 1 < mb1) {
           tile_to_lds(gXK, (mb + 1) * TILE_BYTES, smem + (alt ? SM_XK : SM_XQ), v, lane);
           tile_to_lds(gXV, (mb + 1) * TILE_BYTES, smem + (alt ? SM_XV : SM_XQ + SM_TILE), v, lane);
           eta_to_lds(gEta, (mb + 1) * (CS * 2), smem + (alt ? SM_ETA : SM_B1), v, lane);
@@ -394,7 +404,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
       } else {
         // One workgroup: XQ has two buffers, so the next XQ can leave HBM now; XK / XV / eta follow once their
         // last readers are done (after the pair sum of the output branch).
-        if (mb + 1 < p.NC) tile_to_lds(gXQ, (mb + 1) * TILE_BYTES, smem + SM_XQ + ((mb + 1) & 1) * SM_TILE, v, lane);
+        if (mb + 1 < mb1) tile_to_lds(gXQ, (mb + 1) * TILE_BYTES, smem + SM_XQ + ((mb + 1) & 1) * SM_TILE, v, lane);
       }
       float z[8];
       {
@@ -624,7 +634,7 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
     //      above: the next mini-batch's leave HBM for LDS now.
     {
       LANE_VARS;
-      if (mb + 1 < p.NC) {
+      if (mb + 1 < mb1) {
         tile_to_lds(gXK, (mb + 1) * TILE_BYTES, smem + SM_XK, v, lane);
         tile_to_lds(gXV, (mb + 1) * TILE_BYTES, smem + SM_XV, v, lane);
         eta_to_lds(gEta, (mb + 1) * (CS * 2), smem + SM_ETA, v, lane);
@@ -635,6 +645,9 @@ TTT_DEV void fwd_body(const FwdParams& p, unsigned char* smem, const int bh) {
     __syncthreads();
     TTT_STAGE(FS_OUT_LN);
   }
+  // a segment that is not the sequence's last leaves the checkpoint the next one starts from (b2 in LDS: every wave is
+  // past the barrier that closes the last mini-batch)
+  if (mb1 < p.NC) store_checkpoint(mb1 / p.cgs);
   TTT_STAGES_END(p.stage_clocks == nullptr ? nullptr : p.stage_clocks + ((size_t)bh * 2 + 0) * (FW_NWAVE * STAGE_SLOTS));
 }
 
@@ -736,7 +749,14 @@ TTT_DEV void fwd_output_branch(const FwdParams& p, unsigned char* smem, const in
 
 __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_kernel(const FwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  fwd_body<0, 8>(p, smem, p.bh0 + blockIdx.x);
+  int bh = p.bh0 + blockIdx.x, mb0 = 0, mb1 = p.NC;
+  if (p.seg_len > 0) {
+    const int pairs = p.B * p.NH, job = p.job0 + blockIdx.x, seg = job / pairs;
+    bh = job - seg * pairs;
+    mb0 = seg * p.seg_len;
+    mb1 = mb0 + p.seg_len < p.NC ? mb0 + p.seg_len : p.NC;
+  }
+  fwd_body<0, 8>(p, smem, bh, mb0, mb1);
 }
 
 // Two workgroups per (batch, head), placed like those of the backward (same XCD where the count allows).
@@ -755,7 +775,7 @@ __global__ __launch_bounds__(FW_THREADS) void ttt_mlp_fwd_split_kernel(const Fwd
     role = b & 1;
   }
   bh += p.bh0;
-  if (role == 0) fwd_body<1, RING>(p, smem, bh);
+  if (role == 0) fwd_body<1, RING>(p, smem, bh, 0, p.NC);
   else fwd_output_branch<RING>(p, smem, bh);
 }
 
@@ -768,6 +788,11 @@ __global__ void ttt_mlp_fwd_zero_words(int* w, int n) {
 
 extern "C" int ttt_mlp_fwd_lds_bytes() { return ttt::SM_FWD_BYTES; }
 extern "C" int ttt_mlp_fwd_threads() { return ttt::FW_THREADS; }
+
+hipError_t ttt_mlp_fwd_clear_words(int* words, int n, hipStream_t stream) {
+  hipLaunchKernelGGL(ttt::ttt_mlp_fwd_zero_words, dim3((n + 255) / 256), dim3(256), 0, stream, words, n);
+  return hipGetLastError();
+}
 
 hipError_t ttt_mlp_fwd_enqueue(const ttt::FwdParams& p, hipStream_t stream) {
   // Per-device attribute; cheap enough to set on every launch.

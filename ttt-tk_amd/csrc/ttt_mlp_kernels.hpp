@@ -25,6 +25,10 @@ struct FwdParams {
   int* status;    // the status word behind the synchronisation words
   unsigned long long wait_limit;   // ticks of the 100 MHz clock a workgroup waits for another before it gives up
   int bh0, nbh;   // this launch covers (batch, head) pairs bh0 .. bh0 + nbh - 1
+  // One workgroup per pair, sequence cut into segments (seg_len > 0, a multiple of cgs): workgroup i of the launch
+  // runs job job0 + i, job q = segment q / (B*NH) of pair q % (B*NH); a segment starts from the checkpoint that the
+  // segment before it left (an earlier launch on the same stream) and leaves the one the next starts from.
+  int seg_len, job0;
 #ifdef TTT_STAGE_CLOCKS
   unsigned* stage_clocks;   // [B*NH][2 roles][8 waves][STAGE_SLOTS] or nullptr (see below)
 #endif
@@ -79,6 +83,11 @@ struct BwdParams {
   unsigned long long wait_limit;   // ticks of the 100 MHz clock a workgroup waits for another before it gives up
   int overwrite;  // non-zero: grad_L_XQ / XK / XV / last_eta are stored, not added to (every element is written exactly once)
   int bh0, nbh;   // this launch covers (batch, head) pairs bh0 .. bh0 + nbh - 1 (workspace pointers moved back by bh0 entries)
+  // One workgroup per pair, sequence cut into segments of seg_groups checkpoint groups (> 0): workgroup i of the launch
+  // runs job job0 + i, job q = segment q / (B*NH) of pair q % (B*NH), segment 0 being the sequence's last groups.  A
+  // segment takes the running gradients from grad_L_*_init, where the segment before it (an earlier launch on the same
+  // stream) left them, and the norm-gradient sums from the pair's slots of x_hat_ln_group.
+  int seg_groups, job0;
 #ifdef TTT_STAGE_CLOCKS
   unsigned* stage_clocks;   // [B*NH][4 roles][8 waves][STAGE_SLOTS] or nullptr (see below)
 #endif
@@ -156,6 +165,7 @@ extern "C" void ttt_mlp_set_stage_clocks(unsigned* forward, unsigned* backward);
 
 // p.sync == nullptr: one workgroup per (batch, head); otherwise two (state recurrence / output branch).
 hipError_t ttt_mlp_fwd_enqueue(const ttt::FwdParams& p, hipStream_t stream);
+hipError_t ttt_mlp_fwd_clear_words(int* words, int n, hipStream_t stream);   // zeroes n ints with a small kernel
 // p.sync == nullptr: one workgroup per (batch, head); otherwise two (replay / reverse walk).
 hipError_t ttt_mlp_bwd_enqueue(const ttt::BwdParams& p, hipStream_t stream);
 // Replays checkpoint group 0 and writes the sixteen per-group tensors row-major (side path, one workgroup per pair).

@@ -58,6 +58,9 @@ PASSES = (
 )
 
 
+TRACE_LAUNCHES = sum(int(PASSES[0][2][i + 1]) for i in (0, 2))   # --steps + --warmup of the trace pass
+
+
 def run_pass(workload: str, tag: str, prof_args, bench_args, raw_dir: str, limit_s: int) -> str:
     out_dir = os.path.join(raw_dir, f"{workload}_{tag}")
     os.makedirs(out_dir, exist_ok=True)
@@ -161,20 +164,22 @@ def sources_digest() -> str:
 
 def launch_summary(workload: str, kernels: dict) -> dict:
     """Roofline per launch (forward / backward): a launch may be made of two kernels (pairs beyond a multiple of the CU
-    count run with more workgroups each), so time, bytes and instruction counts are summed over its kernels."""
+    count run with more workgroups each) or of several dispatches of one (sequences cut at checkpoints), so time, bytes
+    and instruction counts are summed over its kernels, each times its `dispatches_per_launch`."""
     launches = {}
     for which in ("fwd", "bwd"):
         ks = [e for k, e in kernels.items() if f"ttt_mlp_{which}" in k]
         if not ks:
             continue
         alg = algorithmic(workload, which)
-        ms = sum(e["avg_ns"] for e in ks) / 1e6
+        n = [e.get("dispatches_per_launch", 1) for e in ks]
+        ms = sum(e["avg_ns"] * d for e, d in zip(ks, n)) / 1e6
         L = dict(kernels=[k for k in kernels if f"ttt_mlp_{which}" in k], launch_ms=ms, units=alg["units"],
                  algorithmic_flop=alg["flop"], algorithmic_bytes=alg["bytes"],
                  achieved_tflops=alg["flop"] / (ms * 1e-3) / 1e12)
         L["frac_of_bf16_mfma_peak"] = L["achieved_tflops"] / PEAK_BF16_TFLOPS
         if all("hbm_bytes" in e for e in ks):
-            L["hbm_bytes"] = sum(e["hbm_bytes"] for e in ks)
+            L["hbm_bytes"] = sum(e["hbm_bytes"] * d for e, d in zip(ks, n))
             L["hbm_bytes_per_unit"] = L["hbm_bytes"] / alg["units"]
             L["traffic_over_algorithmic"] = L["hbm_bytes"] / alg["bytes"]
             L["hbm_gbs"] = L["hbm_bytes"] / (ms * 1e6)
@@ -182,7 +187,7 @@ def launch_summary(workload: str, kernels: dict) -> dict:
             for cn, label in (("SQ_INSTS_VALU", "valu_insts_per_unit"), ("SQ_INSTS_MFMA", "mfma_insts_per_unit"),
                               ("SQ_INSTS_LDS", "lds_insts_per_unit")):
                 if all(cn in e["counters"] for e in ks):
-                    L[label] = sum(e["counters"][cn] for e in ks) / alg["units"]
+                    L[label] = sum(e["counters"][cn] * d for e, d in zip(ks, n)) / alg["units"]
         launches[which] = L
     return launches
 
@@ -208,7 +213,9 @@ def profile(workload: str, raw_dir: str, limit_s: int):
             continue
         key = short_name(name)
         g = geo["fwd" if "fwd" in key else "bwd"]
-        e = dict(calls=st["calls"], avg_ns=st["avg_ns"], **g)
+        # the trace pass makes TRACE_LAUNCHES forward and backward launches; a launch whose sequences are cut at
+        # checkpoints dispatches the kernel several times
+        e = dict(calls=st["calls"], dispatches_per_launch=max(1, round(st["calls"] / TRACE_LAUNCHES)), avg_ns=st["avg_ns"], **g)
         rd = [v["FETCH_SIZE"] for k, v in fetch.items() if short_name(k) == key and "FETCH_SIZE" in v]
         wr = [v["WRITE_SIZE"] for k, v in write.items() if short_name(k) == key and "WRITE_SIZE" in v]
         if rd and wr:
