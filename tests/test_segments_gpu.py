@@ -66,3 +66,45 @@ def test_cut_sequences_give_the_same_forward(NC, cgs):
     finally:
         ext.set_overlap(True)
         ext.set_compute_units(0)
+
+
+def test_cut_backward_with_the_overwrite_policy_and_the_group_tensors():
+    """The cut backward under the operator's other switches: outputs overwritten instead of added to (garbage in the
+    four accumulating outputs must not matter), and the sixteen group tensors filled behind it (x_hat_ln_group carries
+    the cut backward's parked sums before that kernel rewrites it)."""
+    import test_time_training as ext
+    import ttt_mlp_host as host
+    dev = torch.device("cuda:0")
+    B, NH, NC, cgs = 1, 3, 64, 8
+    print(f"case B={B} NH={NH} NC={NC} cgs={cgs}", flush=True)
+    d = orc.make_inputs(B, NH, NC, seed=72)
+    t = {k: d[k].to(dev).contiguous() for k in FWD_KEYS + UP_KEYS}
+    t.update(host.alloc_forward_buffers(B, NH, NC, cgs, dev))
+    t.update(host.alloc_backward_buffers(B, NH, NC, cgs, dev))
+    group_keys = [k for k in host.BWD_ORDER if k.endswith("_group")]
+    assert len(group_keys) == 16
+
+    def run(garbage):
+        host.zero_accumulating_grads(t)
+        if garbage:
+            for k in ("grad_L_XQ", "grad_L_XK", "grad_L_XV", "grad_L_last_eta"):
+                t[k].fill_(3.0)
+        host.forward(t, cgs)
+        host.backward(t, cgs)
+        torch.cuda.synchronize()
+        return {k: t[k].clone() for k in ("Out",) + host.GRAD_NAMES + tuple(group_keys)}
+
+    try:
+        host.set_fill_group_tensors(True)
+        ref = run(False)                          # whole sequences, accumulation into zeros
+        ext.set_compute_units(2)
+        ext.set_overlap(False)
+        host.set_accumulate(False)
+        got = run(True)
+        for k, r in ref.items():
+            assert torch.equal(got[k], r), k
+    finally:
+        host.set_accumulate(True)
+        host.set_fill_group_tensors(False)
+        ext.set_overlap(True)
+        ext.set_compute_units(0)
