@@ -190,15 +190,15 @@ struct SegmentPlan {
   int launches = 1;
   long long jobs = 0;
 };
+#ifndef TTT_CUT_PERCENT
+#define TTT_CUT_PERCENT 99   // a cut must gain 1 % by the estimate below
+#endif
 // `alt_x1000`: what the alternative costs, in thousandths of a mini-batch of one workgroup.
 SegmentPlan plan_segments(long long pairs, int cus, int NC, int cgs, long long alt_x1000) {
   SegmentPlan best;
 #ifndef TTT_STAGE_CLOCKS   // the stage clocks are kept per pair and sequence
-  if (pairs <= cus || cus <= 0 || NC <= 0 || cgs <= 0) return best;
+  if (pairs <= cus || pairs > (1 << 27) || cus <= 0 || NC <= 0 || cgs <= 0) return best;   // (job numbers are ints)
   const int K = (NC + cgs - 1) / cgs;
-#ifndef TTT_CUT_PERCENT
-#define TTT_CUT_PERCENT 99   // a cut must gain 1 % by this estimate
-#endif
   long long best_t = alt_x1000 * TTT_CUT_PERCENT / 100;
   for (int S = 2; S <= 8 && S <= K; S++) {
     const int groups = (K + S - 1) / S, segs = (K + groups - 1) / groups;
@@ -233,31 +233,27 @@ int device_cus() {
     return 0;
   return g_cu_budget > 0 && g_cu_budget < cus ? g_cu_budget : cus;
 }
-// The forward's launches with the sequences cut (plan.seg_len > 0).
-int launch_fwd_segments(ttt::FwdParams p, const SegmentPlan& plan, int cus, hipStream_t stream) {
+// The launches of a call with the sequences cut: `cus` jobs each, in job order, on the one stream.
+template <class Params, class Enqueue>
+int launch_segments(Params p, const SegmentPlan& plan, int cus, Enqueue enqueue) {
   p.sync = nullptr;
   p.bh0 = 0;
-  p.seg_len = plan.seg_len;
   for (long long j0 = 0; j0 < plan.jobs; j0 += cus) {
     p.job0 = static_cast<int>(j0);
     p.nbh = static_cast<int>(plan.jobs - j0 < cus ? plan.jobs - j0 : cus);
-    if (hipError_t e = ttt_mlp_fwd_enqueue(p, stream)) return static_cast<int>(e);
+    if (hipError_t e = enqueue(p)) return static_cast<int>(e);
   }
   return TTT_MLP_OK;
 }
-
-// The backward's launches with the sequences cut: segment 0 = the last groups of every sequence.  The third parked
-// norm-gradient sum needs a second mini-batch slot in x_hat_ln_group, hence cgs >= 2 (plan_bwd_segments).
+int launch_fwd_segments(ttt::FwdParams p, const SegmentPlan& plan, int cus, hipStream_t stream) {
+  p.seg_len = plan.seg_len;
+  return launch_segments(p, plan, cus, [stream](const ttt::FwdParams& q) { return ttt_mlp_fwd_enqueue(q, stream); });
+}
+// Backward: segment 0 = the last groups of every sequence.  The third parked norm-gradient sum needs a second
+// mini-batch slot in x_hat_ln_group, hence cgs >= 2 (plan_bwd_segments).
 int launch_bwd_segments(ttt::BwdParams p, const SegmentPlan& plan, int cus, hipStream_t stream) {
-  p.sync = nullptr;
-  p.bh0 = 0;
   p.seg_groups = plan.groups;
-  for (long long j0 = 0; j0 < plan.jobs; j0 += cus) {
-    p.job0 = static_cast<int>(j0);
-    p.nbh = static_cast<int>(plan.jobs - j0 < cus ? plan.jobs - j0 : cus);
-    if (hipError_t e = ttt_mlp_bwd_enqueue(p, stream)) return static_cast<int>(e);
-  }
-  return TTT_MLP_OK;
+  return launch_segments(p, plan, cus, [stream](const ttt::BwdParams& q) { return ttt_mlp_bwd_enqueue(q, stream); });
 }
 SegmentPlan plan_bwd_segments(const LaunchPlan& pl, long long pairs, int cus, int NC, int cgs, bool with_workspace) {
   if (cgs < 2) return SegmentPlan{};
