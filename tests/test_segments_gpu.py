@@ -1,7 +1,8 @@
-"""More (batch, head) pairs than CUs: the forward cuts every sequence into segments at checkpoint boundaries and
-launches the (segment, pair) jobs a device's worth at a time (a segment starts from the checkpoint the one before it
-left).  Forced here on a few pairs by a small compute-unit budget; the results must not change by a bit - Out, all
-checkpoints, and the backward that starts from those checkpoints."""
+"""More (batch, head) pairs than CUs: the launchers cut every sequence into segments at checkpoint boundaries and
+launch the (segment, pair) jobs a device's worth at a time.  A forward segment starts from the checkpoint the one
+before it left; a backward segment takes the running gradients and the norm-gradient sums from where the one before it
+left them.  Forced here on a few pairs by a small compute-unit budget; the results must not change by a bit - Out, all
+checkpoints and all ten gradients."""
 import ctypes
 import os
 
