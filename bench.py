@@ -44,8 +44,12 @@ def measured_traffic(workload, which):
     if not os.path.exists(path):
         return None
     with open(path) as f:
-        kernels = json.load(f)["kernels"]
-    vals = [k["hbm_bytes"] for name, k in kernels.items() if f"ttt_mlp_{which}" in name and "hbm_bytes" in k]
+        summary = json.load(f)
+    launch = summary.get("launches", {}).get(which)     # summed over the kernels and dispatches a launch is made of
+    if launch is not None:
+        return launch.get("hbm_bytes")
+    vals = [k["hbm_bytes"] * k.get("dispatches_per_launch", 1) for name, k in summary["kernels"].items()
+            if f"ttt_mlp_{which}" in name and "hbm_bytes" in k]
     return sum(vals) if vals else None
 
 

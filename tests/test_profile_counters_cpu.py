@@ -128,3 +128,22 @@ def test_launch_summary_counts_every_dispatch_of_a_cut_launch():
     assert abs(L["bwd"]["valu_insts_per_unit"] - 9e9 / units) < 1e-6
     assert abs(L["fwd"]["launch_ms"] - 9.0) < 1e-9
     assert pc.TRACE_LAUNCHES == 3
+
+
+def test_bench_reads_the_traffic_of_a_whole_launch(tmp_path, monkeypatch):
+    """`roofline.traffic` is per launch: where a launch is several dispatches of one kernel the per-dispatch bytes of
+    the counter summary are not the figure."""
+    import json
+    import bench
+    prof = tmp_path / "profiles"
+    prof.mkdir()
+    (prof / "ttt_mlp_c5_counters.json").write_text(json.dumps({
+        "kernels": {"ttt_mlp_bwd_kernel": {"hbm_bytes": 4.0e10, "dispatches_per_launch": 3}},
+        "launches": {"bwd": {"hbm_bytes": 1.2e11}}}))
+    (prof / "ttt_mlp_c4_counters.json").write_text(json.dumps({      # a summary without the per-launch block
+        "kernels": {"ttt_mlp_bwd_kernel": {"hbm_bytes": 4.0e10, "dispatches_per_launch": 3},
+                    "ttt_mlp_bwd_split_kernel<1, false>": {"hbm_bytes": 1.0e10}}}))
+    monkeypatch.setattr(bench, "ROOT", str(tmp_path))
+    assert bench.measured_traffic("c5", "bwd") == 1.2e11
+    assert bench.measured_traffic("c4", "bwd") == 1.3e11
+    assert bench.measured_traffic("c5", "fwd") is None and bench.measured_traffic("c3", "bwd") is None
